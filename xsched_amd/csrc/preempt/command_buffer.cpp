@@ -1,0 +1,127 @@
+// reference preempt/src/xqueue/command_buffer.cpp
+#include "xsched/utils/xassert.h"
+#include "xsched/preempt/sched/agent.h"
+#include "xsched/preempt/xqueue/async_xqueue.h"
+
+using namespace xsched::sched;
+
+namespace xsched::preempt
+{
+
+// The buffer starts with one drain marker so that "last enqueued command" is
+// always defined and an idle queue always ends in a (completed) drain marker.
+CommandBuffer::CommandBuffer(XQueueHandle xq_h): kXQueueHandle(xq_h)
+{
+    Enqueue(std::make_shared<XQueueWaitAllCommand>());
+}
+
+void CommandBuffer::WaitForNextIdle()
+{
+    std::unique_lock<std::mutex> lock(mtx_);
+    if (xq_state_ == kQueueStateIdle) return;
+    const uint64_t seen = idle_cnt_;
+    idle_cv_.wait(lock, [&]() { return idle_cnt_ != seen; });
+}
+
+XQueueState CommandBuffer::GetXQueueState()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    return xq_state_;
+}
+
+// When the FIFO is empty the launch thread does not go to sleep right away: the
+// buffer hands it, in turn, a batch-sync (retire the oldest marked batch), then
+// a full drain marker, and only after that drain has completed does the XQueue
+// become Idle (command_buffer.cpp:39-97). The Idle/Ready events are sent with
+// the buffer lock held so that a scheduler sees them in the order they happened.
+std::shared_ptr<XCommand> CommandBuffer::Dequeue()
+{
+    std::unique_lock<std::mutex> lock(mtx_);
+
+    if (cmds_.empty()) {
+        switch (last_enqueued_cmd_->GetType()) {
+        case kCommandTypeXQueueWaitAll:
+            if (xq_state_ == kQueueStateReady) {
+                xq_state_ = kQueueStateIdle;
+                idle_cnt_++;
+                idle_cv_.notify_all();
+                SchedAgent::SendEvent(std::make_shared<XQueueIdleEvent>(kXQueueHandle));
+            }
+            consumer_waiting_ = true;
+            cv_.wait(lock, [this]() { return !cmds_.empty(); });
+            consumer_waiting_ = false;
+            break;
+
+        case kCommandTypeBatchSynchronize:
+        {
+            auto drain = std::make_shared<XQueueWaitAllCommand>();
+            drain->SetState(kCommandStatePending);
+            last_enqueued_cmd_ = drain;
+            return drain;
+        }
+
+        default:
+        {
+            auto batch = std::make_shared<BatchSynchronizeCommand>();
+            batch->SetState(kCommandStatePending);
+            last_enqueued_cmd_ = batch;
+            return batch;
+        }
+        }
+    }
+
+    auto xcmd = std::move(cmds_.front());
+    cmds_.pop_front();
+    return xcmd;
+}
+
+void CommandBuffer::Enqueue(std::shared_ptr<XCommand> xcmd)
+{
+    const auto ready_time = std::chrono::system_clock::now();
+    XASSERT(xcmd != nullptr, "xcmd should not be nullptr");
+    xcmd->SetState(kCommandStatePending);
+
+    bool wake;
+    {
+        std::lock_guard<std::mutex> lock(mtx_);
+        if (xcmd->GetType() == kCommandTypeHardware && xq_state_ == kQueueStateIdle) {
+            xq_state_ = kQueueStateReady;
+            SchedAgent::SendEvent(std::make_shared<XQueueReadyEvent>(kXQueueHandle, ready_time));
+        }
+        last_enqueued_cmd_ = xcmd;
+        cmds_.emplace_back(std::move(xcmd));
+        wake = consumer_waiting_;
+    }
+    if (wake) cv_.notify_one();
+}
+
+void CommandBuffer::DropAll()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    for (auto &xcmd : cmds_) xcmd->SetState(kCommandStateCompleted);
+    cmds_.clear();
+}
+
+std::shared_ptr<XQueueWaitAllCommand> CommandBuffer::EnqueueXQueueWaitAllCommand()
+{
+    std::unique_lock<std::mutex> lock(mtx_);
+
+    // Idle: the tail is the drain marker that made the queue idle (completed).
+    // Not idle but the tail is already a drain marker: share it.
+    if (xq_state_ == kQueueStateIdle || last_enqueued_cmd_->GetType() == kCommandTypeXQueueWaitAll) {
+        auto tail = std::dynamic_pointer_cast<XQueueWaitAllCommand>(last_enqueued_cmd_);
+        XASSERT(tail != nullptr, "an idle XQueue must end in a drain marker");
+        return tail;
+    }
+
+    auto drain = std::make_shared<XQueueWaitAllCommand>();
+    drain->SetState(kCommandStatePending);
+    last_enqueued_cmd_ = drain;
+    cmds_.emplace_back(drain);
+    const bool wake = consumer_waiting_;
+    lock.unlock();
+    if (wake) cv_.notify_one();
+    return drain;
+}
+
+} // namespace xsched::preempt
