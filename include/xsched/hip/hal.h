@@ -1,0 +1,94 @@
+/* MI355X HIP hardware-queue adapter: C entry points.
+ *
+ * HipQueueCreate() is the adapter constructor XSched applications and the HIP
+ * interception shim already call (reference
+ * platforms/hip/hal/include/xsched/hip/hal/hal.h:11, implemented there in
+ * platforms/hip/hal/src/hip_queue.cpp:56-71). The queue it returns supports
+ * preemption levels 1 (block) AND 2 (deactivate / reactivate) and switches
+ * between them at run time; the reference adapter is level 1 only
+ * (hip_queue.h:25-26).
+ *
+ * The Hip*CommandCreate() functions build HwCommands for XQueueSubmit(). In
+ * XSched the same objects are C++ classes constructed by the shim (reference
+ * platforms/hip/hal/include/xsched/hip/hal/hip_command.h:22-254); here they are
+ * reachable from C so that any language can submit work without the shim.
+ *
+ * All pointers are device pointers unless said otherwise. Streams are passed as
+ * void* (a hipStream_t). Nothing here takes ownership of user buffers: they must
+ * stay valid until the command has completed.
+ */
+#ifndef XSCHED_HIP_HAL_H_
+#define XSCHED_HIP_HAL_H_
+
+#include "xsched/types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Register `stream` as a hardware queue. The handle equals the stream pointer
+ * (reference handle.h:9-12). The default (null) stream is refused with
+ * NotSupported, as in the reference (hip_queue.cpp:62-65). */
+XResult HipQueueCreate(HwQueueHandle *hwq, void *stream);
+
+/* Counters of one queue, for tests and benches. `out` receives 8 values:
+ * [0] launches, [1] replayed launches, [2] deactivations, [3] reactivations,
+ * [4] marker waits that returned while polling, [5] marker waits that had to
+ * block in the driver, [6] bitmap slots in use, [7] current preempt epoch. */
+XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
+
+/* ---- guarded victim kernels: flushable at level 2 ---------------------------
+ * `guard`: 0 = plain kernel (never flushable, property None),
+ *          1 = guarded kernel, property Deactivatable: at level 2 it carries the
+ *              work-group entry guard and a progress bitmap; at level 1 the same
+ *              command launches the plain variant.
+ *          2 = always launch the guarded variant, even at level 1 (for measuring
+ *              the cost of the guard). */
+
+/* y[i] = fma(alpha, x[i], y[i]) in place, fp32, i < n. 128-bit loads/stores when
+ * x and y are 16-byte aligned. */
+XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, void *y,
+                             size_t n, int guard);
+
+/* C[M,N] = A[M,K] * B[K,N]; A, B, C row-major bf16, fp32 accumulation in ascending
+ * k, round-to-nearest-even on store. M, N multiples of 256 and K a multiple of 64
+ * use the 256x256-tile MFMA kernel; other shapes are refused (InvalidValue). */
+XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void *B, void *C,
+                                 int M, int N, int K, int guard);
+
+/* bins[keys[i]] += 1 for i < n; keys are int32 in [0, n_bins), bins are uint32 and
+ * are NOT cleared by the command. n_bins <= 65536. */
+XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t n, void *bins,
+                                  uint32_t n_bins, int guard);
+
+/* ---- generic commands (level 1 semantics; they are drain points at level 2) -- */
+
+/* hipMemcpyAsync; `kind` is a hipMemcpyKind value. reference hip_command.h:188 */
+XResult HipMemcpyCommandCreate(HwCommandHandle *cmd, void *dst, const void *src, size_t bytes,
+                               int kind);
+
+/* hipMemsetAsync. reference hip_command.h:189 */
+XResult HipMemsetCommandCreate(HwCommandHandle *cmd, void *dst, int value, size_t bytes);
+
+/* hipEventRecord(event) in queue order; property Idempotent, always
+ * synchronizable. reference hip_command.h:197-219 */
+XResult HipEventRecordCommandCreate(HwCommandHandle *cmd, void *event);
+
+/* hipStreamWaitEvent(event, flags) in queue order. reference hip_command.h:236-254 */
+XResult HipEventWaitCommandCreate(HwCommandHandle *cmd, void *event, uint32_t flags);
+
+/* hipLaunchKernel of an arbitrary kernel. `args[i]` points to argument i of
+ * `arg_sizes[i]` bytes; the values are copied at creation (the reference gets the
+ * sizes from code-object metadata instead: hip_command.cpp:53-73,
+ * kernel_param.cpp:256-345). `host_func` is the kernel's host-side symbol. */
+XResult HipKernelCommandCreate(HwCommandHandle *cmd, const void *host_func,
+                               uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                               uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                               void **args, const size_t *arg_sizes, size_t n_args,
+                               uint32_t shared_mem_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* XSCHED_HIP_HAL_H_ */

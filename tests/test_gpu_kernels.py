@@ -1,0 +1,169 @@
+"""GPU parity: the guarded kernels, launched through the C ABI and an XQueue, against
+the CPU oracle on the same seeded inputs. Integer and fp32-AXPY results must be
+bit-exact; the bf16 GEMM is bit-exact where the arithmetic is exact (small-integer
+inputs) and within a stated tolerance otherwise."""
+import ctypes
+from ctypes import byref, c_uint64, c_void_p
+
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+class Queue:
+    """One stream + HwQueue + XQueue."""
+
+    def __init__(self, xs, torch, level=1, threshold=8, batch=4):
+        self.xs, self.torch = xs, torch
+        self.stream = torch.cuda.Stream()
+        self.hwq = xs.hip_queue_create(self.stream.cuda_stream)
+        self.xq = xs.xqueue_create(self.hwq, level)
+        xs.check(xs.preempt().XQueueSetLaunchConfig(self.xq, threshold, batch))
+
+    def submit(self, cmd):
+        self.xs.check(self.xs.preempt().XQueueSubmit(self.xq, cmd))
+
+    def wait(self):
+        self.xs.check(self.xs.preempt().XQueueWaitAll(self.xq))
+
+    def close(self):
+        p = self.xs.preempt()
+        self.xs.check(p.XQueueDestroy(self.xq))
+        self.xs.check(p.HwQueueDestroy(self.hwq))
+
+
+def axpy_cmd(xs, alpha, x, y, n, guard):
+    cmd = c_uint64()
+    xs.check(xs.halhip().HipAxpyCommandCreate(byref(cmd), alpha, x.data_ptr(), y.data_ptr(), n, guard))
+    return cmd.value
+
+
+def gemm_cmd(xs, a, b, c, M, N, K, guard):
+    cmd = c_uint64()
+    xs.check(xs.halhip().HipGemmBf16CommandCreate(byref(cmd), a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                                                  M, N, K, guard))
+    return cmd.value
+
+
+def hist_cmd(xs, keys, n, bins, n_bins, guard):
+    cmd = c_uint64()
+    xs.check(xs.halhip().HipHistogramCommandCreate(byref(cmd), keys.data_ptr(), n, bins.data_ptr(),
+                                                   n_bins, guard))
+    return cmd.value
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 5, 1023, 4096, 4097, (1 << 20) + 7, 1 << 22])
+@pytest.mark.parametrize("level,guard", [(1, 0), (1, 2), (2, 1)])
+def test_axpy_bit_exact(xs, gpu, n, level, guard):
+    torch = gpu
+    print(f"case axpy n={n} level={level} guard={guard}", flush=True)
+    x_h = oracle.fill_uniform(0, 1, 0, max(n, 1))[:n]
+    y_h = oracle.fill_uniform(0, 2, 0, max(n, 1))[:n]
+    x = torch.from_numpy(x_h.copy()).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, level)
+    times = 3
+    for _ in range(times):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, guard))
+    q.wait()
+    torch.cuda.synchronize()
+    want = oracle.axpy(0.5, x_h, y_h, times)
+    got = y.cpu().numpy()
+    q.close()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_axpy_general_alpha_and_unaligned(xs, gpu):
+    """alpha whose product is inexact (one rounding: fma) and a pointer that is only
+    4-byte aligned (scalar fallback kernel)."""
+    torch = gpu
+    n = 100003
+    x_h = oracle.fill_uniform(3, 1, 0, n + 1)
+    y_h = oracle.fill_uniform(3, 2, 0, n + 1)
+    x = torch.from_numpy(x_h.copy()).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, 2)
+    alpha = 0.3337
+    q.submit(axpy_cmd(xs, alpha, x, y, n, 1))          # aligned
+    q.wait()
+    want = oracle.axpy(np.float32(alpha), x_h[:n], y_h[:n])
+    assert np.array_equal(y.cpu().numpy()[:n].view(np.uint32), want.view(np.uint32))
+    xo, yo = x[1:], y[1:]                               # misaligned by 4 bytes
+    y_before = y.cpu().numpy().copy()
+    q.submit(axpy_cmd(xs, alpha, xo, yo, n, 1))
+    q.wait()
+    want2 = oracle.axpy(np.float32(alpha), x_h[1:n + 1], y_before[1:n + 1])
+    got = y.cpu().numpy()
+    q.close()
+    assert np.array_equal(got[1:n + 1].view(np.uint32), want2.view(np.uint32))
+    assert got[0] == y_before[0]
+
+
+@pytest.mark.parametrize("n,n_bins", [(0, 65536), (1, 65536), (1000, 65536), (65536 + 13, 65536),
+                                      (1 << 20, 65536), (300000, 1000), (5000, 7)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_histogram_bit_exact(xs, gpu, n, n_bins, level, guard):
+    torch = gpu
+    print(f"case hist n={n} bins={n_bins} level={level} guard={guard}", flush=True)
+    table = oracle.zipf_table(n_bins)
+    keys_h = oracle.fill_zipf(0, 1, 0, max(n, 1), table, n_bins)[:n]
+    keys = torch.from_numpy(np.ascontiguousarray(keys_h) if n else np.zeros(1, np.int32)).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, level)
+    q.submit(hist_cmd(xs, keys, n, bins, n_bins, guard))
+    q.submit(hist_cmd(xs, keys, n, bins, n_bins, guard))   # accumulates: bins are not cleared
+    q.wait()
+    got = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    want = oracle.histogram(keys_h, n_bins)
+    want = oracle.histogram(keys_h, n_bins, want)
+    assert int(got.sum()) == 2 * n
+    assert np.array_equal(got, want)
+
+
+def _gemm_case(xs, torch, a_bits, b_bits, M, N, K, level, guard):
+    a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
+    b = torch.from_numpy(b_bits.view(np.int16).reshape(K, N)).cuda()
+    c = torch.zeros(M, N, dtype=torch.int16, device="cuda")
+    q = Queue(xs, torch, level)
+    q.submit(gemm_cmd(xs, a, b, c, M, N, K, guard))
+    q.wait()
+    got = c.cpu().numpy().view(np.uint16)
+    q.close()
+    return got
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 512, 128), (512, 256, 192)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_gemm_exact_on_small_integers(xs, gpu, M, N, K, level, guard):
+    """Inputs are integers in [-4, 4]: every product and partial sum is an integer below
+    2^24, so fp32 accumulation is exact in any order and the bf16 result is determined;
+    any indexing or layout mistake changes it."""
+    print(f"case gemm-int M={M} N={N} K={K} level={level} guard={guard}", flush=True)
+    rng = np.random.default_rng(7)
+    a_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b_i = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    a_bits, b_bits = oracle.f32_to_bf16_bits(a_i), oracle.f32_to_bf16_bits(b_i)
+    got = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, level, guard)
+    want_int = a_i.astype(np.int64) @ b_i.astype(np.int64)
+    want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K)
+    assert np.array_equal(want, oracle.f32_to_bf16_bits(want_int.astype(np.float32)).reshape(M, N))
+    assert np.array_equal(got, want)
+
+
+def test_gemm_normal_inputs_within_tolerance(xs, gpu):
+    """Seeded N(0,1)-like inputs: the MFMA's internal summation order is not the
+    oracle's, so the comparison is on values. Tolerance: one bf16 unit in the last
+    place of the result (2^-8 relative) plus fp32 accumulation noise 2^-20*sqrt(K)."""
+    M, N, K = 256, 256, 512
+    a_bits = oracle.fill_normal_bf16(11, 1, 0, M * K)
+    b_bits = oracle.fill_normal_bf16(11, 2, 0, K * N)
+    got = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, 2, 1)
+    want_bits, want_f32 = oracle.gemm_bf16(a_bits, b_bits, M, N, K, want_f32=True)
+    got_f = oracle.bf16_bits_to_f32(got.ravel()).reshape(M, N)
+    tol = np.abs(want_f32) * 2.0 ** -8 + 2.0 ** -20 * np.sqrt(K) * 16
+    assert np.all(np.abs(got_f - want_f32) <= tol)
+    assert np.mean(got == want_bits) > 0.95

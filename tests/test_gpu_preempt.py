@@ -1,0 +1,183 @@
+"""GPU: Level-2 deactivate / reactivate. Results of runs that are suspended and
+resumed many times must be bit-identical to uninterrupted runs (and, for the integer
+and fp32 kernels, to the CPU oracle)."""
+import random
+import threading
+import time
+from ctypes import byref, c_int, c_uint64
+
+import numpy as np
+import pytest
+
+import oracle
+from test_gpu_kernels import Queue, axpy_cmd, gemm_cmd, hist_cmd
+
+pytestmark = pytest.mark.gpu
+
+
+def hip_stats(xs, hwq):
+    out = (c_uint64 * 8)()
+    xs.check(xs.halhip().HipQueueGetStats(hwq, out))
+    return list(out)
+
+
+def churn(xs, q, stop, seed, flags=0):
+    """Suspend / resume the queue at random moments until told to stop."""
+    rnd = random.Random(seed)
+    p = xs.preempt()
+    cycles = 0
+    while not stop.is_set():
+        time.sleep(rnd.uniform(0.0002, 0.002))
+        xs.check(p.XQueueSuspend(q.xq, flags))
+        time.sleep(rnd.uniform(0.0001, 0.001))
+        xs.check(p.XQueueResume(q.xq, 0))
+        cycles += 1
+    return cycles
+
+
+@pytest.mark.parametrize("suspend_flags", [0, 1])  # 1 = kQueueSuspendFlagSyncHwQueue
+def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags):
+    torch = gpu
+    n, times = 1 << 24, 60
+    print(f"case axpy-preempt n={n} times={times} flags={suspend_flags}", flush=True)
+    x_h = oracle.fill_uniform(5, 1, 0, n)
+    y_h = oracle.fill_uniform(5, 2, 0, n)
+    x = torch.from_numpy(x_h).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, level=2, threshold=4, batch=2)
+    stop = threading.Event()
+    result = {}
+    t = threading.Thread(target=lambda: result.setdefault("cycles", churn(xs, q, stop, 1, suspend_flags)))
+    t.start()
+    for _ in range(times):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    # Keep churning while the queue drains, then stop and let it finish.
+    time.sleep(0.05)
+    stop.set()
+    t.join()
+    q.wait()
+    st = hip_stats(xs, q.hwq)
+    got = y.cpu().numpy()
+    q.close()
+    want = oracle.axpy(0.5, x_h, y_h, times)
+    print("stats", st, "cycles", result.get("cycles"), flush=True)
+    assert st[2] > 0 and st[3] > 0, "no deactivation happened: the test did not exercise level 2"
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_histogram_preempt_resume_bit_exact(xs, gpu):
+    torch = gpu
+    n, n_bins, times = 1 << 24, 65536, 40
+    print(f"case hist-preempt n={n} times={times}", flush=True)
+    table = oracle.zipf_table(n_bins)
+    keys_h = oracle.fill_zipf(9, 1, 0, n, table, n_bins)
+    keys = torch.from_numpy(keys_h).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, level=2, threshold=4, batch=2)
+    stop = threading.Event()
+    t = threading.Thread(target=churn, args=(xs, q, stop, 2))
+    t.start()
+    for _ in range(times):
+        q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+    time.sleep(0.05)
+    stop.set()
+    t.join()
+    q.wait()
+    st = hip_stats(xs, q.hwq)
+    got = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    one = oracle.histogram(keys_h, n_bins).astype(np.uint64)
+    print("stats", st, flush=True)
+    assert st[2] > 0
+    assert int(got.sum()) == times * n
+    assert np.array_equal(got.astype(np.uint64), one * times)
+
+
+def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu):
+    torch = gpu
+    M = N = K = 2048
+    times = 12
+    print(f"case gemm-preempt {M}^3 times={times}", flush=True)
+    a_bits = oracle.fill_normal_bf16(13, 1, 0, M * K)
+    b_bits = oracle.fill_normal_bf16(13, 2, 0, K * N)
+    a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
+    b = torch.from_numpy(b_bits.view(np.int16).reshape(K, N)).cuda()
+    c_ref = torch.zeros(M, N, dtype=torch.int16, device="cuda")
+    q1 = Queue(xs, torch, level=1)
+    q1.submit(gemm_cmd(xs, a, b, c_ref, M, N, K, 0))
+    q1.wait()
+    q1.close()
+
+    outs = [torch.zeros(M, N, dtype=torch.int16, device="cuda") for _ in range(times)]
+    q = Queue(xs, torch, level=2, threshold=4, batch=2)
+    stop = threading.Event()
+    t = threading.Thread(target=churn, args=(xs, q, stop, 3))
+    t.start()
+    for c in outs:
+        q.submit(gemm_cmd(xs, a, b, c, M, N, K, 1))
+    time.sleep(0.02)
+    stop.set()
+    t.join()
+    q.wait()
+    st = hip_stats(xs, q.hwq)
+    print("stats", st, flush=True)
+    q.close()
+    assert st[2] > 0
+    for c in outs:
+        assert torch.equal(c, c_ref)
+
+
+def test_resume_with_drop_commands(xs, gpu):
+    """After a suspend, resuming with DropCommands completes everything submitted so
+    far without executing what had not started (reference async_xqueue.cpp:137-149)."""
+    torch = gpu
+    n = 1 << 22
+    x = torch.ones(n, device="cuda")
+    y = torch.zeros(n, device="cuda")
+    q = Queue(xs, torch, level=2, threshold=2, batch=1)
+    p = xs.preempt()
+    xs.check(p.XQueueSuspend(q.xq, 0))
+    for _ in range(20):
+        q.submit(axpy_cmd(xs, 1.0, x, y, n, 1))
+    xs.check(p.XQueueResume(q.xq, 1))  # kQueueResumeFlagDropCommands
+    q.wait()
+    state = c_int()
+    xs.check(p.XQueueQuery(q.xq, byref(state)))
+    assert state.value == xs.kQueueStateIdle
+    got = y.cpu().numpy()
+    assert np.all(got == 0.0)
+    # The queue is usable afterwards.
+    q.submit(axpy_cmd(xs, 1.0, x, y, n, 1))
+    q.wait()
+    assert np.all(y.cpu().numpy() == 1.0)
+    q.close()
+
+
+def test_dynamic_level_switch(xs, gpu):
+    """The reference HIP adapter refuses level changes (hip_queue.h:25); this one
+    moves between 1 and 2 and refuses 3."""
+    torch = gpu
+    q = Queue(xs, torch, level=1)
+    p = xs.preempt()
+    assert p.XQueueSetPreemptLevel(q.xq, xs.kPreemptLevelDeactivate) == xs.kXSchedSuccess
+    assert p.XQueueSetPreemptLevel(q.xq, xs.kPreemptLevelBlock) == xs.kXSchedSuccess
+    assert p.XQueueSetPreemptLevel(q.xq, 0) == xs.kXSchedErrorInvalidValue
+    # Level 3 is above the adapter's maximum: accepted call, level unchanged (warning).
+    assert p.XQueueSetPreemptLevel(q.xq, xs.kPreemptLevelInterrupt) == xs.kXSchedSuccess
+    n = 4096
+    x = torch.ones(n, device="cuda"); y = torch.zeros(n, device="cuda")
+    q.submit(axpy_cmd(xs, 2.0, x, y, n, 1))
+    q.wait()
+    assert np.all(y.cpu().numpy() == 2.0)
+    q.close()
+
+
+def test_null_stream_and_bad_arguments(xs, gpu):
+    h = xs.halhip()
+    hwq = c_uint64()
+    assert h.HipQueueCreate(byref(hwq), None) == xs.kXSchedErrorNotSupported
+    assert h.HipQueueCreate(None, 1) == xs.kXSchedErrorInvalidValue
+    cmd = c_uint64()
+    assert h.HipGemmBf16CommandCreate(byref(cmd), 16, 16, 16, 100, 256, 64, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipHistogramCommandCreate(byref(cmd), 16, 4, 16, 70000, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipAxpyCommandCreate(byref(cmd), 1.0, None, None, 4, 0) == xs.kXSchedErrorInvalidValue

@@ -41,8 +41,7 @@ PREEMPT_SRCS = [
 HOST_SRCS = ["host/host_queue.cpp"]
 SERVER_SRCS = ["service/xserver.cpp"]
 HIP_SRCS = ["hip/hip_queue.hip", "hip/hip_command.hip", "hip/kernels_axpy.hip",
-            "hip/kernels_gemm.hip", "hip/kernels_hist.hip", "hip/hal_api.hip",
-            "bench/harness.hip"]
+            "hip/kernels_gemm.hip", "hip/kernels_hist.hip", "bench/harness.hip"]
 
 
 def _run(cmd):

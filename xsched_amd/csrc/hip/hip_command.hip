@@ -1,0 +1,146 @@
+// Generic HIP commands: copies, fills, events, arbitrary kernels. None of them can
+// be flushed; at level 2 the launch thread lets earlier flushable commands finish
+// before it launches one of these (except the event commands, which write no
+// memory and are tagged idempotent, as the reference's CUDA adapter does:
+// platforms/cuda/hal/src/common/cuda_command.cpp:160-161).
+#include <cstring>
+
+#include "hip_hal.h"
+#include "xsched/hip/hal.h"
+
+using namespace xsched::preempt;
+
+namespace xsched::hip
+{
+
+namespace
+{
+
+class HipMemcpyCommand final : public HipCommand
+{
+public:
+    HipMemcpyCommand(void *dst, const void *src, size_t bytes, hipMemcpyKind kind)
+        : dst_(dst), src_(src), bytes_(bytes), kind_(kind) {}
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    { return hipMemcpyAsync(dst_, src_, bytes_, kind_, q.Stream()); }
+private:
+    void *dst_; const void *src_; size_t bytes_; hipMemcpyKind kind_;
+};
+
+class HipMemsetCommand final : public HipCommand
+{
+public:
+    HipMemsetCommand(void *dst, int value, size_t bytes): dst_(dst), value_(value), bytes_(bytes) {}
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    { return hipMemsetAsync(dst_, value_, bytes_, q.Stream()); }
+private:
+    void *dst_; int value_; size_t bytes_;
+};
+
+// The user's event is the marker: always synchronizable (hip_command.h:197-219).
+class HipEventRecordCommand final : public HipCommand
+{
+public:
+    explicit HipEventRecordCommand(hipEvent_t event): HipCommand(kCommandPropertyIdempotent), event_(event) {}
+    virtual void Synchronize() override { HIP_ASSERT(hipEventSynchronize(event_)); }
+    virtual bool Synchronizable() override { return true; }
+    virtual bool EnableSynchronization() override { return true; }
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override { return hipEventRecord(event_, q.Stream()); }
+private:
+    hipEvent_t event_;
+};
+
+class HipEventWaitCommand final : public HipCommand
+{
+public:
+    HipEventWaitCommand(hipEvent_t event, unsigned flags)
+        : HipCommand(kCommandPropertyIdempotent), event_(event), flags_(flags) {}
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    { return hipStreamWaitEvent(q.Stream(), event_, flags_); }
+private:
+    hipEvent_t event_; unsigned flags_;
+};
+
+// Arguments are copied at creation, so the caller's storage may go away before the
+// launch thread gets to the command.
+class HipKernelCommand final : public HipCommand
+{
+public:
+    HipKernelCommand(const void *func, dim3 grid, dim3 block, void **args, const size_t *sizes,
+                     size_t n_args, uint32_t shmem)
+        : func_(func), grid_(grid), block_(block), shmem_(shmem)
+    {
+        size_t total = 0;
+        for (size_t i = 0; i < n_args; ++i) total += ROUND_UP(sizes[i], 16);
+        storage_.resize(total);
+        arg_ptrs_.resize(n_args);
+        size_t off = 0;
+        for (size_t i = 0; i < n_args; ++i) {
+            memcpy(storage_.data() + off, args[i], sizes[i]);
+            arg_ptrs_[i] = storage_.data() + off;
+            off += ROUND_UP(sizes[i], 16);
+        }
+    }
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    { return hipLaunchKernel(func_, grid_, block_, arg_ptrs_.data(), shmem_, q.Stream()); }
+private:
+    const void *func_; dim3 grid_, block_; uint32_t shmem_;
+    std::vector<char> storage_;
+    std::vector<void *> arg_ptrs_;
+};
+
+} // namespace
+
+} // namespace xsched::hip
+
+using namespace xsched::hip;
+
+EXPORT_C_FUNC XResult HipMemcpyCommandCreate(HwCommandHandle *cmd, void *dst, const void *src,
+                                             size_t bytes, int kind)
+{
+    if (cmd == nullptr || kind < 0 || kind > (int)hipMemcpyDefault) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipMemcpyCommand>(dst, src, bytes, (hipMemcpyKind)kind));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipMemsetCommandCreate(HwCommandHandle *cmd, void *dst, int value, size_t bytes)
+{
+    if (cmd == nullptr) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipMemsetCommand>(dst, value, bytes));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipEventRecordCommandCreate(HwCommandHandle *cmd, void *event)
+{
+    if (cmd == nullptr || event == nullptr) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipEventRecordCommand>((hipEvent_t)event));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipEventWaitCommandCreate(HwCommandHandle *cmd, void *event, uint32_t flags)
+{
+    if (cmd == nullptr || event == nullptr) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipEventWaitCommand>((hipEvent_t)event, flags));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipKernelCommandCreate(HwCommandHandle *cmd, const void *host_func,
+                                             uint32_t gx, uint32_t gy, uint32_t gz,
+                                             uint32_t bx, uint32_t by, uint32_t bz,
+                                             void **args, const size_t *arg_sizes, size_t n_args,
+                                             uint32_t shared_mem_bytes)
+{
+    if (cmd == nullptr || host_func == nullptr || (n_args != 0 && (args == nullptr || arg_sizes == nullptr))) {
+        return kXSchedErrorInvalidValue;
+    }
+    if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || by == 0 || bz == 0 ||
+        (uint64_t)bx * by * bz > 1024) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipKernelCommand>(
+        host_func, dim3(gx, gy, gz), dim3(bx, by, bz), args, arg_sizes, n_args, shared_mem_bytes));
+    return kXSchedSuccess;
+}

@@ -1,0 +1,176 @@
+// MI355X HIP hardware-queue adapter (internal declarations).
+//
+// HipQueue  - HwQueue over one hipStream_t: Level-1 launch and marker sync,
+//             Level-2 deactivate / reactivate through the device-side guard.
+// HipCommand - HwCommand with an optional completion marker (hipEvent).
+// Replaces reference platforms/hip/hal/src/{hip_queue,hip_command}.cpp, which are
+// Level-1 only. Calls the HIP runtime directly (no dlopen'd driver table).
+#pragma once
+
+#include <atomic>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "xsched/hip/guard.h"
+#include "xsched/types.h"
+#include "xsched/utils/xassert.h"
+#include "xsched/preempt/hal/hw_command.h"
+#include "xsched/preempt/hal/hw_queue.h"
+
+#define HIP_ASSERT(expr) \
+    do { hipError_t e_ = (expr); \
+         XASSERT(e_ == hipSuccess, "HIP error %d (%s) at %s", (int)e_, hipGetErrorString(e_), #expr); \
+    } while (0)
+
+namespace xsched::hip
+{
+
+/// Process-wide pool of timing-less events used as completion markers. Grows by
+/// small chunks on demand (the reference creates 513 at the first use:
+/// event_pool.h:26-32, utils/pool.h:15-24).
+class EventPool
+{
+public:
+    static EventPool &Instance();
+    hipEvent_t Pop();
+    void Push(hipEvent_t ev);
+private:
+    std::mutex mtx_;
+    std::vector<hipEvent_t> free_;
+};
+
+/// Level-2 state of one queue: the preempt word and the progress-bitmap slots.
+class GuardState
+{
+public:
+    static constexpr uint32_t kMaxWorkGroups = 1u << 18;          // per guarded command
+    static constexpr uint32_t kSlotWords = kMaxWorkGroups / 32;   // 32 KiB per slot
+    static constexpr uint32_t kSlotsPerArena = 32;
+
+    explicit GuardState(int device);
+    ~GuardState();
+
+    /// Device-visible address of the preempt word.
+    const uint32_t *FlagDevPtr() const { return flag_dev_; }
+    uint32_t Epoch() const { return epoch_.load(std::memory_order_acquire); }
+
+    /// Bump the preempt word; visible to running kernels within a memory round trip.
+    void Deactivate(hipStream_t op_stream);
+    /// Returns once the latest Deactivate() is visible to the device.
+    void WaitFlagWritten(hipStream_t op_stream);
+
+    /// A bitmap slot (device memory, NOT cleared). Never blocks on the device except
+    /// when a new arena has to be allocated.
+    uint32_t *AcquireSlot();
+    void ReleaseSlot(uint32_t *slot);
+    uint64_t SlotsInUse();
+
+private:
+    const int device_;
+    bool flag_on_host_ = true;
+    uint32_t *flag_host_ = nullptr;  // CPU address (host placement) / staging word
+    uint32_t *flag_dev_ = nullptr;   // GPU address
+    std::atomic<uint32_t> epoch_ { 0 };
+
+    std::mutex mtx_;
+    std::vector<uint32_t *> arenas_;
+    std::vector<uint32_t *> free_slots_;
+    uint64_t in_use_ = 0;
+};
+
+class HipQueue;
+
+class HipCommand : public preempt::HwCommand
+{
+public:
+    explicit HipCommand(preempt::XCommandProperties props = preempt::kCommandPropertyNone)
+        : HwCommand(props) {}
+    virtual ~HipCommand();
+
+    virtual void Synchronize() override;
+    virtual bool Synchronizable() override { return marker_ != nullptr; }
+    virtual bool EnableSynchronization() override;
+
+    /// Enqueue on the queue's stream and (re-)record the marker behind it.
+    /// `replay` is true when called from Reactivate().
+    hipError_t LaunchWrapper(HipQueue &q, bool replay);
+
+    /// Whether Reactivate() must enqueue this command again.
+    virtual bool ReplayOnReactivate() const { return false; }
+
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool replay) = 0;
+    hipEvent_t marker_ = nullptr;
+
+private:
+    HipQueue *queue_ = nullptr; // for wait statistics; set at launch
+};
+
+/// Base of the guarded victim kernels.
+class HipGuardedCommand : public HipCommand
+{
+public:
+    /// guard_mode: 0 plain, 1 guarded at level >= 2, 2 guarded always.
+    HipGuardedCommand(uint32_t n_wg, int guard_mode)
+        : HipCommand(guard_mode ? preempt::kCommandPropertyDeactivatable : preempt::kCommandPropertyNone)
+        , n_wg_(n_wg), guard_mode_(guard_mode) {}
+    virtual ~HipGuardedCommand();
+
+    virtual bool ReplayOnReactivate() const override { return guard_mode_ != 0; }
+    uint32_t WorkGroups() const { return n_wg_; }
+
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool replay) override final;
+    /// Launch the kernel. `guarded` selects the variant with the guard compiled in.
+    virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) = 0;
+
+    const uint32_t n_wg_;
+    const int guard_mode_;
+
+private:
+    std::shared_ptr<GuardState> guard_state_; // keeps the slot's arena alive
+    uint32_t *slot_ = nullptr;
+};
+
+class HipQueue : public preempt::HwQueue
+{
+public:
+    explicit HipQueue(hipStream_t stream);
+    virtual ~HipQueue();
+
+    virtual void Launch(std::shared_ptr<preempt::HwCommand> hw_cmd) override;
+    virtual void Synchronize() override;
+    virtual void Deactivate() override;
+    virtual void Reactivate(const preempt::CommandLog &log) override;
+
+    virtual XDevice       GetDevice()            override { return xdevice_; }
+    virtual HwQueueHandle GetHandle()            override { return (HwQueueHandle)stream_; }
+    virtual bool          SupportDynamicLevel()  override { return true; }
+    virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
+    virtual void OnPreemptLevelChange(XPreemptLevel level) override;
+    virtual void OnXQueueCreate() override;
+
+    hipStream_t Stream() const { return stream_; }
+    XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }
+    const std::shared_ptr<GuardState> &Guard() const { return guard_; }
+
+    // statistics (see HipQueueGetStats)
+    std::atomic<uint64_t> n_launch { 0 }, n_replay { 0 }, n_deactivate { 0 }, n_reactivate { 0 };
+    std::atomic<uint64_t> n_wait_polled { 0 }, n_wait_blocked { 0 };
+
+private:
+    const hipStream_t stream_;
+    int device_ = 0;
+    XDevice xdevice_ = 0;
+    std::atomic<XPreemptLevel> level_ { kPreemptLevelUnknown };
+    std::shared_ptr<GuardState> guard_;
+    hipStream_t op_stream_ = nullptr; // flag writes when the word lives in device memory
+};
+
+/// Microseconds a marker wait polls before it blocks in the driver.
+int64_t SyncSpinMicros();
+
+} // namespace xsched::hip

@@ -1,0 +1,319 @@
+// HipQueue, its Level-2 guard state, the marker pool and the command base classes.
+#include <chrono>
+#include <thread>
+
+#include "hip_hal.h"
+#include "xsched/hip/hal.h"
+#include "xsched/utils/env.h"
+#include "xsched/protocol/def.h"
+#include "xsched/protocol/device.h"
+
+using namespace xsched::preempt;
+using namespace xsched::protocol;
+
+namespace xsched::hip
+{
+
+int64_t SyncSpinMicros()
+{
+    static const int64_t us = []() {
+        int64_t v = 200;
+        GetEnvInt64(XSCHED_HIP_SYNC_SPIN_US_ENV_NAME, v);
+        return v < 0 ? (int64_t)0 : v;
+    }();
+    return us;
+}
+
+// ---- EventPool ---------------------------------------------------------------
+
+EventPool &EventPool::Instance()
+{
+    static EventPool *pool = new EventPool(); // never destroyed: commands may outlive main()
+    return *pool;
+}
+
+hipEvent_t EventPool::Pop()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    if (free_.empty()) {
+        for (int i = 0; i < 16; ++i) {
+            hipEvent_t ev = nullptr;
+            HIP_ASSERT(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+            free_.push_back(ev);
+        }
+    }
+    hipEvent_t ev = free_.back();
+    free_.pop_back();
+    return ev;
+}
+
+void EventPool::Push(hipEvent_t ev)
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    free_.push_back(ev);
+}
+
+// ---- GuardState --------------------------------------------------------------
+// Placement of the preempt word (XSCHED_HIP_FLAG_MEM):
+//   host   (default) pinned, coherent host memory mapped into the device. The CPU
+//          flips it with one store; the device reads it across the host link.
+//   device fine-grained device memory; the CPU flips it with a 4-byte stream write
+//          on a side stream; the device reads it from local memory.
+
+GuardState::GuardState(int device): device_(device)
+{
+    flag_on_host_ = GetEnv(XSCHED_HIP_FLAG_MEM_ENV_NAME) != "device";
+    HIP_ASSERT(hipHostMalloc((void **)&flag_host_, 64, hipHostMallocMapped | hipHostMallocCoherent));
+    *flag_host_ = 0;
+    if (flag_on_host_) {
+        HIP_ASSERT(hipHostGetDevicePointer((void **)&flag_dev_, flag_host_, 0));
+    } else {
+        HIP_ASSERT(hipExtMallocWithFlags((void **)&flag_dev_, 64, hipDeviceMallocFinegrained));
+        HIP_ASSERT(hipMemset(flag_dev_, 0, 64));
+    }
+}
+
+GuardState::~GuardState()
+{
+    // Arenas and the word are only released here, when no command holds the state
+    // any more (each guarded command keeps a reference while it owns a slot).
+    for (uint32_t *a : arenas_) (void)hipFree(a);
+    if (!flag_on_host_ && flag_dev_) (void)hipFree(flag_dev_);
+    if (flag_host_) (void)hipHostFree(flag_host_);
+}
+
+void GuardState::Deactivate(hipStream_t op_stream)
+{
+    const uint32_t e = epoch_.fetch_add(1, std::memory_order_acq_rel) + 1;
+    if (flag_on_host_) {
+        __atomic_store_n(flag_host_, e, __ATOMIC_RELEASE);
+    } else {
+        HIP_ASSERT(hipStreamWriteValue32(op_stream, flag_dev_, e, 0));
+    }
+}
+
+void GuardState::WaitFlagWritten(hipStream_t op_stream)
+{
+    if (!flag_on_host_) HIP_ASSERT(hipStreamSynchronize(op_stream));
+}
+
+uint32_t *GuardState::AcquireSlot()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    if (free_slots_.empty()) {
+        uint32_t *arena = nullptr;
+        HIP_ASSERT(hipMalloc((void **)&arena, (size_t)kSlotsPerArena * kSlotWords * sizeof(uint32_t)));
+        arenas_.push_back(arena);
+        for (uint32_t i = 0; i < kSlotsPerArena; ++i) free_slots_.push_back(arena + (size_t)i * kSlotWords);
+    }
+    uint32_t *slot = free_slots_.back();
+    free_slots_.pop_back();
+    in_use_++;
+    return slot;
+}
+
+void GuardState::ReleaseSlot(uint32_t *slot)
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    free_slots_.push_back(slot);
+    in_use_--;
+}
+
+uint64_t GuardState::SlotsInUse()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    return in_use_;
+}
+
+// ---- HipCommand --------------------------------------------------------------
+
+HipCommand::~HipCommand()
+{
+    if (marker_ != nullptr) EventPool::Instance().Push(marker_);
+}
+
+bool HipCommand::EnableSynchronization()
+{
+    if (marker_ == nullptr) marker_ = EventPool::Instance().Pop();
+    return marker_ != nullptr;
+}
+
+hipError_t HipCommand::LaunchWrapper(HipQueue &q, bool replay)
+{
+    queue_ = &q;
+    hipError_t err = Enqueue(q, replay);
+    if (UNLIKELY(err != hipSuccess)) return err;
+    // Recording again after a replay moves the marker behind the replayed work,
+    // which is what a later Synchronize() has to wait for.
+    if (marker_ != nullptr) err = hipEventRecord(marker_, q.Stream());
+    return err;
+}
+
+// Marker wait, sized for device work in the 10 us .. 1 ms range: poll the event
+// for a bounded time (no system call, no sleep/wake latency), then fall back to
+// the driver's blocking wait so that a long wait does not burn a core.
+void HipCommand::Synchronize()
+{
+    XASSERT(marker_ != nullptr, "Synchronize() needs EnableSynchronization() before launch");
+    const int64_t spin_us = SyncSpinMicros();
+    if (spin_us > 0) {
+        const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_us);
+        int probes = 0;
+        while (true) {
+            hipError_t err = hipEventQuery(marker_);
+            if (err == hipSuccess) {
+                if (queue_) queue_->n_wait_polled.fetch_add(1, std::memory_order_relaxed);
+                return;
+            }
+            XASSERT(err == hipErrorNotReady, "hipEventQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
+            if ((++probes & 7) == 0 && std::chrono::steady_clock::now() >= deadline) break;
+            __builtin_ia32_pause();
+        }
+    }
+    if (queue_) queue_->n_wait_blocked.fetch_add(1, std::memory_order_relaxed);
+    HIP_ASSERT(hipEventSynchronize(marker_));
+}
+
+// ---- HipGuardedCommand -------------------------------------------------------
+
+HipGuardedCommand::~HipGuardedCommand()
+{
+    if (slot_ != nullptr) guard_state_->ReleaseSlot(slot_);
+}
+
+// Level 1 (or guard_mode 0): the plain kernel, nothing else on the stream.
+// Level 2: first launch takes a bitmap slot and clears it in stream order; every
+// launch (first or replay) carries the epoch current at enqueue time.
+hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
+{
+    const bool level2 = q.Level() >= kPreemptLevelDeactivate;
+    const bool guarded = guard_mode_ == 2 || (guard_mode_ == 1 && level2);
+
+    XGuardArgs g;
+    g.flag = q.Guard()->FlagDevPtr();
+    g.bitmap = nullptr;
+    g.epoch = q.Guard()->Epoch();
+    g.resume = replay ? 1u : 0u;
+
+    if (guarded && level2) {
+        if (slot_ == nullptr) {
+            XASSERT(n_wg_ <= GuardState::kMaxWorkGroups, "too many work-groups for a guarded command");
+            guard_state_ = q.Guard();
+            slot_ = guard_state_->AcquireSlot();
+            hipError_t err = hipMemsetAsync(slot_, 0, ((size_t)n_wg_ + 31) / 32 * sizeof(uint32_t), q.Stream());
+            if (err != hipSuccess) return err;
+        }
+        g.bitmap = slot_;
+    }
+    return LaunchKernel(q.Stream(), guarded, g);
+}
+
+// ---- HipQueue ----------------------------------------------------------------
+
+HipQueue::HipQueue(hipStream_t stream): stream_(stream)
+{
+    HIP_ASSERT(hipGetDevice(&device_));
+    hipDeviceProp_t prop;
+    HIP_ASSERT(hipGetDeviceProperties(&prop, device_));
+    xdevice_ = MakeDevice(kDeviceTypeGPU, MakePciId(prop.pciDomainID, prop.pciBusID, prop.pciDeviceID, 0));
+    guard_ = std::make_shared<GuardState>(device_);
+    HIP_ASSERT(hipStreamCreateWithFlags(&op_stream_, hipStreamNonBlocking)); // default priority
+    // Nothing of the application may still be running on the stream (hip_queue.cpp:35-36).
+    HIP_ASSERT(hipStreamSynchronize(stream_));
+}
+
+HipQueue::~HipQueue()
+{
+    if (op_stream_) (void)hipStreamDestroy(op_stream_);
+}
+
+void HipQueue::OnXQueueCreate() { HIP_ASSERT(hipSetDevice(device_)); }
+
+void HipQueue::OnPreemptLevelChange(XPreemptLevel level)
+{
+    XASSERT(level <= kPreemptLevelDeactivate, "unsupported level: %d", level);
+    level_.store(level, std::memory_order_release);
+}
+
+void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
+{
+    auto *cmd = dynamic_cast<HipCommand *>(hw_cmd.get());
+    XASSERT(cmd != nullptr, "hw_cmd is not a HipCommand");
+    hipError_t err = cmd->LaunchWrapper(*this, false);
+    XASSERT(err == hipSuccess, "failed to enqueue command: %d (%s)", (int)err, hipGetErrorString(err));
+    n_launch.fetch_add(1, std::memory_order_relaxed);
+}
+
+void HipQueue::Synchronize() { HIP_ASSERT(hipStreamSynchronize(stream_)); }
+
+void HipQueue::Deactivate()
+{
+    XASSERT(Level() >= kPreemptLevelDeactivate, "Deactivate() not supported on level-%d", Level());
+    guard_->Deactivate(op_stream_);
+    n_deactivate.fetch_add(1, std::memory_order_relaxed);
+}
+
+// No device synchronisation and no read-back: flushed launches are still draining
+// on the stream; the replays are queued behind them with the new epoch and sort
+// out, work-group by work-group, what is left to do. Commands that cannot be
+// flushed (plain kernels, copies) are never behind an in-flight flushable command,
+// so they have run to completion and are skipped; marker-only commands (event
+// records) that follow a replayed kernel are recorded again to keep their place.
+void HipQueue::Reactivate(const CommandLog &log)
+{
+    XASSERT(Level() >= kPreemptLevelDeactivate, "Reactivate() not supported on level-%d", Level());
+    HIP_ASSERT(hipSetDevice(device_));
+    n_reactivate.fetch_add(1, std::memory_order_relaxed);
+    // A replay carries the new epoch; the word must already show it, or the replay
+    // would flush itself.
+    guard_->WaitFlagWritten(op_stream_);
+
+    bool replaying = false;
+    for (auto &hw_cmd : log) {
+        auto *cmd = dynamic_cast<HipCommand *>(hw_cmd.get());
+        if (cmd == nullptr) continue;
+        const bool flushable = cmd->ReplayOnReactivate();
+        const bool idempotent = cmd->GetProps(kCommandPropertyIdempotent) != 0;
+        if (!flushable && !(replaying && idempotent)) continue;
+        replaying = true;
+        hipError_t err = cmd->LaunchWrapper(*this, true);
+        XASSERT(err == hipSuccess, "failed to replay command: %d (%s)", (int)err, hipGetErrorString(err));
+        n_replay.fetch_add(1, std::memory_order_relaxed);
+    }
+}
+
+} // namespace xsched::hip
+
+using namespace xsched::hip;
+
+EXPORT_C_FUNC XResult HipQueueCreate(HwQueueHandle *hwq, void *stream)
+{
+    if (hwq == nullptr) {
+        XWARN("HipQueueCreate failed: hwq is nullptr");
+        return kXSchedErrorInvalidValue;
+    }
+    if (stream == nullptr) {
+        XWARN("HipQueueCreate failed: the default stream is not supported");
+        return kXSchedErrorNotSupported;
+    }
+    const HwQueueHandle h = (HwQueueHandle)stream;
+    XResult res = HwQueueManager::Add(h, [&]() { return std::make_shared<HipQueue>((hipStream_t)stream); });
+    if (res == kXSchedSuccess) *hwq = h;
+    return res;
+}
+
+EXPORT_C_FUNC XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out)
+{
+    if (out == nullptr) return kXSchedErrorInvalidValue;
+    auto q = std::dynamic_pointer_cast<HipQueue>(HwQueueManager::Get(hwq));
+    if (q == nullptr) return kXSchedErrorNotFound;
+    out[0] = q->n_launch.load();
+    out[1] = q->n_replay.load();
+    out[2] = q->n_deactivate.load();
+    out[3] = q->n_reactivate.load();
+    out[4] = q->n_wait_polled.load();
+    out[5] = q->n_wait_blocked.load();
+    out[6] = q->Guard()->SlotsInUse();
+    out[7] = q->Guard()->Epoch();
+    return kXSchedSuccess;
+}

@@ -1,0 +1,183 @@
+// Guarded streaming AXPY for gfx950: y = fma(alpha, x, y), fp32, in place.
+//
+// HBM-bound: 12 bytes of traffic per element (read x, read y, write y). One
+// work-group is one wavefront; it owns a contiguous chunk of `steps` x 1024
+// elements and walks it in steps of 4 x 128-bit accesses per lane and stream,
+// lane-contiguous so that every access of a wave covers 1 KiB. Loads and stores
+// are non-temporal: nothing is reused. The preempt word is read after the first
+// step's loads have been issued, so its latency overlaps theirs. Because the
+// update is in place, a work-group must run exactly once: it commits its bit in
+// the progress bitmap after its last store.
+#include "hip_hal.h"
+#include "xsched/hip/hal.h"
+#include "xsched/utils/env.h"
+
+using namespace xsched::preempt;
+
+namespace xsched::hip
+{
+
+namespace axpy
+{
+
+constexpr uint32_t kLanes = 64;
+constexpr uint32_t kVecPerStep = 4;                        // float4 per lane per step
+constexpr uint32_t kStepVecs = kLanes * kVecPerStep;       // 256 float4 = 4 KiB per stream
+constexpr uint32_t kStepElems = kStepVecs * 4;             // 1024 floats
+
+typedef float float4 __attribute__((ext_vector_type(4))); // 128-bit access unit
+
+__device__ __forceinline__ float4 ld_nt(const float4 *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st_nt(float4 *p, float4 v) { __builtin_nontemporal_store(v, p); }
+
+__device__ __forceinline__ float4 fma4(float a, float4 x, float4 y)
+{
+    float4 r;
+    r.x = __builtin_fmaf(a, x.x, y.x);
+    r.y = __builtin_fmaf(a, x.y, y.y);
+    r.z = __builtin_fmaf(a, x.z, y.z);
+    r.w = __builtin_fmaf(a, x.w, y.w);
+    return r;
+}
+
+// n4: number of whole float4 in the arrays; tail: the 0..3 trailing scalars, done by
+// the last work-group.
+template <bool kGuard>
+__global__ __launch_bounds__(64)
+void AxpyVec4Kernel(float alpha, const float4 *x, float4 *y,
+                    uint64_t n4, uint32_t tail, uint32_t steps, XGuardArgs g)
+{
+    const uint32_t wg = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint64_t wg_base = (uint64_t)wg * steps * kStepVecs;
+    XGuardWave guard(g, wg);
+
+    const bool full = wg_base + (uint64_t)steps * kStepVecs <= n4;
+    if (full) {
+        for (uint32_t s = 0; s < steps; ++s) {
+            const uint64_t base = wg_base + (uint64_t)s * kStepVecs + lane;
+            float4 xv[kVecPerStep], yv[kVecPerStep];
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                xv[u] = ld_nt(&x[base + u * kLanes]);
+                yv[u] = ld_nt(&y[base + u * kLanes]);
+            }
+            if (kGuard && s == 0) {
+                if (!guard.Enter()) return;
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                st_nt(&y[base + u * kLanes], fma4(alpha, xv[u], yv[u]));
+            }
+        }
+    } else {
+        if (kGuard) {
+            if (!guard.Enter()) return;
+        }
+        const uint64_t end = wg_base + (uint64_t)steps * kStepVecs;
+        for (uint64_t i = wg_base + lane; i < end && i < n4; i += kLanes) {
+            st_nt(&y[i], fma4(alpha, ld_nt(&x[i]), ld_nt(&y[i])));
+        }
+        if (wg == gridDim.x - 1 && lane < tail) {
+            const float *xs = (const float *)(x + n4);
+            float *ys = (float *)(y + n4);
+            ys[lane] = __builtin_fmaf(alpha, xs[lane], ys[lane]);
+        }
+    }
+    if (kGuard) guard.Commit();
+}
+
+// Fallback for pointers that are not 16-byte aligned: same chunking, 32-bit accesses.
+template <bool kGuard>
+__global__ __launch_bounds__(64)
+void AxpyScalarKernel(float alpha, const float *__restrict__ x, float *__restrict__ y,
+                      uint64_t n, uint32_t steps, XGuardArgs g)
+{
+    const uint32_t wg = blockIdx.x;
+    XGuardWave guard(g, wg);
+    if (kGuard) {
+        if (!guard.Enter()) return;
+    }
+    const uint64_t begin = (uint64_t)wg * steps * kStepElems;
+    const uint64_t end = begin + (uint64_t)steps * kStepElems;
+    for (uint64_t i = begin + threadIdx.x; i < end && i < n; i += kLanes) {
+        y[i] = __builtin_fmaf(alpha, x[i], y[i]);
+    }
+    if (kGuard) guard.Commit();
+}
+
+class HipAxpyCommand final : public HipGuardedCommand
+{
+public:
+    HipAxpyCommand(float alpha, const float *x, float *y, size_t n, uint32_t steps, uint32_t n_wg,
+                   int guard_mode)
+        : HipGuardedCommand(n_wg, guard_mode), alpha_(alpha), x_(x), y_(y), n_(n), steps_(steps) {}
+
+protected:
+    virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
+    {
+        if (n_ == 0) return hipSuccess;
+        const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
+        const dim3 grid(n_wg_), block(kLanes);
+        if (aligned) {
+            const uint64_t n4 = n_ / 4;
+            const uint32_t tail = (uint32_t)(n_ % 4);
+            if (guarded) {
+                hipLaunchKernelGGL(AxpyVec4Kernel<true>, grid, block, 0, stream, alpha_,
+                                   (const float4 *)x_, (float4 *)y_, n4, tail, steps_, g);
+            } else {
+                hipLaunchKernelGGL(AxpyVec4Kernel<false>, grid, block, 0, stream, alpha_,
+                                   (const float4 *)x_, (float4 *)y_, n4, tail, steps_, g);
+            }
+        } else {
+            if (guarded) {
+                hipLaunchKernelGGL(AxpyScalarKernel<true>, grid, block, 0, stream, alpha_, x_, y_,
+                                   (uint64_t)n_, steps_, g);
+            } else {
+                hipLaunchKernelGGL(AxpyScalarKernel<false>, grid, block, 0, stream, alpha_, x_, y_,
+                                   (uint64_t)n_, steps_, g);
+            }
+        }
+        return hipGetLastError();
+    }
+
+private:
+    const float alpha_;
+    const float *x_;
+    float *y_;
+    const size_t n_;
+    const uint32_t steps_;
+};
+
+} // namespace axpy
+
+using namespace axpy;
+
+/// Steps (of 1024 elements) per work-group: small enough that the device drains in
+/// tens of microseconds after a flush, large enough that the grid fits the progress
+/// bitmap.
+uint32_t AxpyStepsFor(size_t n)
+{
+    static const int64_t dflt = []() { int64_t v = 4; GetEnvInt64("XSCHED_HIP_AXPY_STEPS", v); return v < 1 ? (int64_t)1 : v; }();
+    uint64_t steps = (uint64_t)dflt;
+    while (((uint64_t)n + steps * kStepElems - 1) / (steps * kStepElems) > GuardState::kMaxWorkGroups) steps *= 2;
+    return (uint32_t)steps;
+}
+
+} // namespace xsched::hip
+
+using namespace xsched::hip;
+
+EXPORT_C_FUNC XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, void *y,
+                                           size_t n, int guard)
+{
+    if (cmd == nullptr || (n != 0 && (x == nullptr || y == nullptr)) || guard < 0 || guard > 2) {
+        return kXSchedErrorInvalidValue;
+    }
+    const uint32_t steps = AxpyStepsFor(n);
+    const uint64_t per_wg = (uint64_t)steps * 1024;
+    const uint32_t n_wg = n == 0 ? 1 : (uint32_t)((n + per_wg - 1) / per_wg);
+    *cmd = HwCommandManager::Add(std::make_shared<axpy::HipAxpyCommand>(
+        alpha, (const float *)x, (float *)y, n, steps, n_wg, guard));
+    return kXSchedSuccess;
+}
