@@ -14,35 +14,52 @@
 // (`epoch`). A work-group may run only while word == epoch: Deactivate() bumps
 // the word, so every work-group that has not yet passed Enter() returns at once
 // and the device drains in about the time of one work-group. Work-groups that did
-// pass Enter() run to their end and set their bit in `bitmap`. Reactivate()
-// enqueues the same kernel again with the new epoch and `resume` set; the
-// work-groups whose bit is set return immediately, the others run. Each
+// pass Enter() run to their end and record themselves in the progress map `done`
+// (one byte per work-group, holding the generation tag of the command).
+// Reactivate() enqueues the same kernel again with the new epoch and `resume`
+// set; the work-groups already recorded return immediately, the others run. Each
 // work-group therefore executes exactly once, which makes in-place and atomic
 // kernels safe to flush. Stream order guarantees that a replay starts only after
-// the flushed launch has left the device, so the bitmap it reads is final.
+// the flushed launch has left the device, so the progress map it reads is final.
+// The generation tag makes a recycled map valid without clearing it: bytes left by
+// an earlier command carry another tag.
 //
 // This is the role of the guardian prologue that XSched injects into CUDA kernels
 // by binary instrumentation (reference platforms/cuda/hal/inject/inject.cu:43-83
 // check_preempt, :124-140 restore_exec; preempt buffer layout
 // platforms/cuda/hal/src/level2/instrument.cpp:177-180). Differences: it is
 // compiled into hand-written kernels instead of injected; the flag is an epoch
-// counter, so nothing has to be cleared or read back on resume; one bit per
+// counter, so nothing has to be cleared or read back on resume; one byte per
 // work-group instead of two words.
 //
-// Cost: one scalar load per work-group whose latency hides behind the first
-// input loads, one compare, and one atomic OR per work-group.
+// Cost: one uncached scalar load per work-group whose latency hides behind the first
+// input loads, one compare, and one byte store per work-group.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// The preempt word is replicated: copy c lives at flag[c * kXGuardFlagStrideWords],
+// c in [0, flag_mask]. Uncached reads of ONE address are served one after the other by
+// a single memory channel (about 27 ns each on MI355X), which would cap a kernel at
+// some 37 M work-groups per second; work-group w reads copy (w & flag_mask), so the
+// reads spread over many channels. The host rewrites all copies on a deactivation.
+#define kXGuardFlagStrideWords 64u /* 256 bytes between copies */
+
 struct XGuardArgs
 {
-    const uint32_t *flag;   // the queue's preempt word (deactivation count)
-    uint32_t       *bitmap; // 1 bit per work-group, set at Commit(); may be null
-    uint32_t        epoch;  // deactivation count this launch was enqueued under
-    uint32_t        resume; // nonzero: skip work-groups whose bit is already set
+    const uint32_t *flag;      // the queue's preempt word, copy 0 (deactivation count)
+    uint8_t        *done;      // progress map: done[w] == gen once work-group w has committed; may be null
+    uint32_t        epoch;     // deactivation count this launch was enqueued under
+    uint32_t        resume;    // nonzero: skip work-groups that have already committed
+    uint32_t        flag_mask; // number of copies of the preempt word minus one (2^k - 1)
+    uint32_t        gen;       // generation tag of this command in its progress map (1..255)
 };
+
+__device__ __forceinline__ const uint32_t *xguard_flag_copy(const XGuardArgs &g, uint32_t wg)
+{
+    return g.flag + (size_t)(wg & g.flag_mask) * kXGuardFlagStrideWords;
+}
 
 #ifndef XGUARD_SCALAR_LOAD
 #define XGUARD_SCALAR_LOAD 1
@@ -68,10 +85,18 @@ __device__ __forceinline__ uint32_t xguard_read_flag(const uint32_t *flag)
     return v;
 }
 
-__device__ __forceinline__ bool xguard_bit_set(const uint32_t *bitmap, uint32_t wg)
+__device__ __forceinline__ bool xguard_committed(const XGuardArgs &g, uint32_t wg)
 {
-    const uint32_t word = __builtin_amdgcn_readfirstlane(__builtin_nontemporal_load(&bitmap[wg >> 5]));
-    return ((word >> (wg & 31)) & 1u) != 0;
+    const uint32_t tag = __builtin_amdgcn_readfirstlane((uint32_t)__builtin_nontemporal_load(&g.done[wg]));
+    return tag == g.gen;
+}
+
+// A plain (cached) byte store: the L2 merges the bytes of neighbouring work-groups
+// into whole lines. A non-temporal store or an atomic OR here costs 3-4 % of a
+// streaming kernel's bandwidth on MI355X, the cached store well under 1 %.
+__device__ __forceinline__ void xguard_commit(const XGuardArgs &g, uint32_t wg)
+{
+    g.done[wg] = (uint8_t)g.gen;
 }
 
 /// Guard of a work-group that is ONE wavefront (blockDim == 64): the decision is
@@ -84,18 +109,15 @@ public:
     /// False: this work-group must not run (flushed, or finished by an earlier launch).
     __device__ __forceinline__ bool Enter() const
     {
-        if (xguard_read_flag(g_.flag) != g_.epoch) return false;
-        if (g_.resume && g_.bitmap && xguard_bit_set(g_.bitmap, wg_)) return false;
+        if (xguard_read_flag(xguard_flag_copy(g_, wg_)) != g_.epoch) return false;
+        if (g_.resume && g_.done && xguard_committed(g_, wg_)) return false;
         return true;
     }
 
     /// Call after the last store of the work-group.
     __device__ __forceinline__ void Commit() const
     {
-        if (g_.bitmap && (threadIdx.x & 63) == 0) {
-            __hip_atomic_fetch_or(&g_.bitmap[wg_ >> 5], 1u << (wg_ & 31),
-                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (g_.done && (threadIdx.x & 63) == 0) xguard_commit(g_, wg_);
     }
 
 private:
@@ -114,8 +136,8 @@ public:
     __device__ __forceinline__ bool Enter() const
     {
         if (threadIdx.x < 64) {
-            bool go = xguard_read_flag(g_.flag) == g_.epoch;
-            if (go && g_.resume && g_.bitmap && xguard_bit_set(g_.bitmap, wg_)) go = false;
+            bool go = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+            if (go && g_.resume && g_.done && xguard_committed(g_, wg_)) go = false;
             if (threadIdx.x == 0) *lds_ = go ? 1u : 0u;
         }
         __syncthreads();
@@ -124,12 +146,12 @@ public:
 
     /// Mid-work re-check for a work-group whose results so far live only in
     /// registers / LDS: when it returns false the work-group abandons itself (its
-    /// bit stays clear, a replay redoes it). Every wave of the group must call it
+    /// byte stays untagged, a replay redoes it). Every wave of the group must call it
     /// at the same point; it contains two barriers.
     __device__ __forceinline__ bool StillCurrent() const
     {
         __syncthreads();
-        if (threadIdx.x == 0) *lds_ = xguard_read_flag(g_.flag) == g_.epoch ? 1u : 0u;
+        if (threadIdx.x == 0) *lds_ = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch ? 1u : 0u;
         __syncthreads();
         return *lds_ != 0;
     }
@@ -138,10 +160,7 @@ public:
     __device__ __forceinline__ void Commit() const
     {
         __syncthreads();
-        if (g_.bitmap && threadIdx.x == 0) {
-            __hip_atomic_fetch_or(&g_.bitmap[wg_ >> 5], 1u << (wg_ & 31),
-                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (g_.done && threadIdx.x == 0) xguard_commit(g_, wg_);
     }
 
 private:

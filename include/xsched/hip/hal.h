@@ -34,13 +34,13 @@ XResult HipQueueCreate(HwQueueHandle *hwq, void *stream);
 /* Counters of one queue, for tests and benches. `out` receives 8 values:
  * [0] launches, [1] replayed launches, [2] deactivations, [3] reactivations,
  * [4] marker waits that returned while polling, [5] marker waits that had to
- * block in the driver, [6] bitmap slots in use, [7] current preempt epoch. */
+ * block in the driver, [6] progress-map slots in use, [7] current preempt epoch. */
 XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
 
 /* ---- guarded victim kernels: flushable at level 2 ---------------------------
  * `guard`: 0 = plain kernel (never flushable, property None),
  *          1 = guarded kernel, property Deactivatable: at level 2 it carries the
- *              work-group entry guard and a progress bitmap; at level 1 the same
+ *              work-group entry guard and a progress map; at level 1 the same
  *              command launches the plain variant.
  *          2 = always launch the guarded variant, even at level 1 (for measuring
  *              the cost of the guard). */

@@ -42,19 +42,23 @@ private:
     std::vector<hipEvent_t> free_;
 };
 
-/// Level-2 state of one queue: the preempt word and the progress-bitmap slots.
+/// Level-2 state of one queue: the preempt word and the progress-map slots.
 class GuardState
 {
 public:
-    static constexpr uint32_t kMaxWorkGroups = 1u << 18;          // per guarded command
-    static constexpr uint32_t kSlotWords = kMaxWorkGroups / 32;   // 32 KiB per slot
-    static constexpr uint32_t kSlotsPerArena = 32;
+    static constexpr uint32_t kMaxWorkGroups = 1u << 18;   // per guarded command
+    static constexpr uint32_t kSlotBytes = kMaxWorkGroups; // one byte per work-group
+    static constexpr uint32_t kSlotsPerArena = 16;         // 4 MiB per arena
+
+    /// A progress map and the generation tag its current owner writes into it.
+    struct Slot { uint8_t *done = nullptr; uint32_t gen = 0; uint32_t index = 0; bool needs_clear = false; };
 
     explicit GuardState(int device);
     ~GuardState();
 
-    /// Device-visible address of the preempt word.
+    /// Device-visible address of copy 0 of the preempt word, and copies - 1.
     const uint32_t *FlagDevPtr() const { return flag_dev_; }
+    uint32_t FlagMask() const { return copies_ - 1; }
     uint32_t Epoch() const { return epoch_.load(std::memory_order_acquire); }
 
     /// Bump the preempt word; visible to running kernels within a memory round trip.
@@ -62,22 +66,28 @@ public:
     /// Returns once the latest Deactivate() is visible to the device.
     void WaitFlagWritten(hipStream_t op_stream);
 
-    /// A bitmap slot (device memory, NOT cleared). Never blocks on the device except
-    /// when a new arena has to be allocated.
-    uint32_t *AcquireSlot();
-    void ReleaseSlot(uint32_t *slot);
+    /// A progress map with a fresh generation tag. The map is not cleared: bytes of
+    /// earlier owners carry other tags. Only when the 8-bit tag wraps does the caller
+    /// have to clear it (needs_clear). Blocks on the device only when a new arena has
+    /// to be allocated.
+    Slot AcquireSlot();
+    void ReleaseSlot(const Slot &slot);
     uint64_t SlotsInUse();
 
 private:
     const int device_;
-    bool flag_on_host_ = true;
-    uint32_t *flag_host_ = nullptr;  // CPU address (host placement) / staging word
-    uint32_t *flag_dev_ = nullptr;   // GPU address
+    bool flag_on_host_ = false;
+    uint32_t copies_ = 1;            // power of two
+    uint32_t *flag_host_ = nullptr;  // pinned image of all copies (the word itself when on host)
+    uint32_t *flag_dev_ = nullptr;   // GPU address of copy 0
     std::atomic<uint32_t> epoch_ { 0 };
 
+    bool write_through_bar_ = false; // CPU stores straight into device memory
     std::mutex mtx_;
-    std::vector<uint32_t *> arenas_;
-    std::vector<uint32_t *> free_slots_;
+    std::vector<uint8_t *> arenas_;
+    std::vector<uint8_t *> slot_ptr_;   // by slot index
+    std::vector<uint32_t> slot_gen_;    // last generation handed out, by slot index
+    std::vector<uint32_t> free_slots_;  // slot indices
     uint64_t in_use_ = 0;
 };
 
@@ -132,7 +142,7 @@ protected:
 
 private:
     std::shared_ptr<GuardState> guard_state_; // keeps the slot's arena alive
-    uint32_t *slot_ = nullptr;
+    GuardState::Slot slot_;
 };
 
 class HipQueue : public preempt::HwQueue

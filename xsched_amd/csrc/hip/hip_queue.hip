@@ -1,5 +1,8 @@
 // HipQueue, its Level-2 guard state, the marker pool and the command base classes.
 #include <chrono>
+#include <csetjmp>
+#include <csignal>
+#include <cstring>
 #include <thread>
 
 #include "hip_hal.h"
@@ -55,21 +58,67 @@ void EventPool::Push(hipEvent_t ev)
 
 // ---- GuardState --------------------------------------------------------------
 // Placement of the preempt word (XSCHED_HIP_FLAG_MEM):
-//   host   (default) pinned, coherent host memory mapped into the device. The CPU
-//          flips it with one store; the device reads it across the host link.
-//   device fine-grained device memory; the CPU flips it with a 4-byte stream write
-//          on a side stream; the device reads it from local memory.
+//   device (default) fine-grained device memory, read by kernels from local memory.
+//          How the CPU rewrites the copies (XSCHED_HIP_FLAG_WRITE):
+//            bar   (default when the device exposes all of its memory to the CPU)
+//                  plain CPU stores through the PCIe aperture: posted writes, no
+//                  runtime call, visible to the device about a microsecond later
+//            copy  one small host-to-device copy on a side stream
+//   host   pinned, coherent host memory mapped into the device. The CPU flips the
+//          copies with plain stores; kernels read them across the host link,
+//          which limits them to a few tens of millions of work-groups per second.
+// XSCHED_HIP_FLAG_COPIES: number of copies (power of two, default 64).
+
+namespace
+{
+thread_local sigjmp_buf g_probe_jmp;
+void ProbeFault(int) { siglongjmp(g_probe_jmp, 1); }
+
+// Whether the CPU can load and store `p`. A fault is caught, not fatal.
+bool CpuCanAccess(volatile uint32_t *p)
+{
+    struct sigaction sa {}, old_segv {}, old_bus {};
+    sa.sa_handler = ProbeFault;
+    sigemptyset(&sa.sa_mask);
+    sigaction(SIGSEGV, &sa, &old_segv);
+    sigaction(SIGBUS, &sa, &old_bus);
+    bool ok = false;
+    if (sigsetjmp(g_probe_jmp, 1) == 0) {
+        const uint32_t v = *p;
+        *p = v;
+        ok = true;
+    }
+    sigaction(SIGSEGV, &old_segv, nullptr);
+    sigaction(SIGBUS, &old_bus, nullptr);
+    return ok;
+}
+} // namespace
 
 GuardState::GuardState(int device): device_(device)
 {
-    flag_on_host_ = GetEnv(XSCHED_HIP_FLAG_MEM_ENV_NAME) != "device";
-    HIP_ASSERT(hipHostMalloc((void **)&flag_host_, 64, hipHostMallocMapped | hipHostMallocCoherent));
-    *flag_host_ = 0;
+    flag_on_host_ = GetEnv(XSCHED_HIP_FLAG_MEM_ENV_NAME) == "host";
+    int64_t copies = 64;
+    GetEnvInt64("XSCHED_HIP_FLAG_COPIES", copies);
+    copies_ = 1;
+    while ((int64_t)copies_ * 2 <= copies && copies_ < 4096) copies_ *= 2;
+
+    const size_t bytes = (size_t)copies_ * kXGuardFlagStrideWords * sizeof(uint32_t);
+    HIP_ASSERT(hipHostMalloc((void **)&flag_host_, bytes, hipHostMallocMapped | hipHostMallocCoherent));
+    memset(flag_host_, 0, bytes);
     if (flag_on_host_) {
         HIP_ASSERT(hipHostGetDevicePointer((void **)&flag_dev_, flag_host_, 0));
-    } else {
-        HIP_ASSERT(hipExtMallocWithFlags((void **)&flag_dev_, 64, hipDeviceMallocFinegrained));
-        HIP_ASSERT(hipMemset(flag_dev_, 0, 64));
+        return;
+    }
+    HIP_ASSERT(hipExtMallocWithFlags((void **)&flag_dev_, bytes, hipDeviceMallocFinegrained));
+    HIP_ASSERT(hipMemset(flag_dev_, 0, bytes));
+    HIP_ASSERT(hipDeviceSynchronize());
+
+    const std::string how = GetEnv("XSCHED_HIP_FLAG_WRITE");
+    int large_bar = 0;
+    (void)hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device_);
+    if (how != "copy" && large_bar != 0) write_through_bar_ = CpuCanAccess(flag_dev_);
+    if (how == "bar" && !write_through_bar_) {
+        XWARN("XSCHED_HIP_FLAG_WRITE=bar, but device memory is not CPU-accessible; using copies");
     }
 }
 
@@ -77,45 +126,63 @@ GuardState::~GuardState()
 {
     // Arenas and the word are only released here, when no command holds the state
     // any more (each guarded command keeps a reference while it owns a slot).
-    for (uint32_t *a : arenas_) (void)hipFree(a);
+    for (uint8_t *a : arenas_) (void)hipFree(a);
     if (!flag_on_host_ && flag_dev_) (void)hipFree(flag_dev_);
     if (flag_host_) (void)hipHostFree(flag_host_);
 }
 
 void GuardState::Deactivate(hipStream_t op_stream)
 {
+    std::lock_guard<std::mutex> lock(mtx_);
     const uint32_t e = epoch_.fetch_add(1, std::memory_order_acq_rel) + 1;
-    if (flag_on_host_) {
-        __atomic_store_n(flag_host_, e, __ATOMIC_RELEASE);
-    } else {
-        HIP_ASSERT(hipStreamWriteValue32(op_stream, flag_dev_, e, 0));
+    uint32_t *target = (flag_on_host_ || !write_through_bar_) ? flag_host_ : flag_dev_;
+    for (uint32_t c = 0; c < copies_; ++c) {
+        __atomic_store_n(&target[(size_t)c * kXGuardFlagStrideWords], e, __ATOMIC_RELEASE);
+    }
+    if (!flag_on_host_ && write_through_bar_) {
+        __builtin_ia32_sfence(); // push the write-combined stores out now
+    } else if (!flag_on_host_) {
+        const size_t bytes = (size_t)copies_ * kXGuardFlagStrideWords * sizeof(uint32_t);
+        HIP_ASSERT(hipMemcpyAsync(flag_dev_, flag_host_, bytes, hipMemcpyHostToDevice, op_stream));
     }
 }
 
 void GuardState::WaitFlagWritten(hipStream_t op_stream)
 {
-    if (!flag_on_host_) HIP_ASSERT(hipStreamSynchronize(op_stream));
+    if (!flag_on_host_ && !write_through_bar_) HIP_ASSERT(hipStreamSynchronize(op_stream));
 }
 
-uint32_t *GuardState::AcquireSlot()
+GuardState::Slot GuardState::AcquireSlot()
 {
     std::lock_guard<std::mutex> lock(mtx_);
     if (free_slots_.empty()) {
-        uint32_t *arena = nullptr;
-        HIP_ASSERT(hipMalloc((void **)&arena, (size_t)kSlotsPerArena * kSlotWords * sizeof(uint32_t)));
+        uint8_t *arena = nullptr;
+        const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
+        HIP_ASSERT(hipMalloc((void **)&arena, bytes));
+        HIP_ASSERT(hipMemset(arena, 0, bytes));
         arenas_.push_back(arena);
-        for (uint32_t i = 0; i < kSlotsPerArena; ++i) free_slots_.push_back(arena + (size_t)i * kSlotWords);
+        for (uint32_t i = 0; i < kSlotsPerArena; ++i) {
+            free_slots_.push_back((uint32_t)slot_ptr_.size());
+            slot_ptr_.push_back(arena + (size_t)i * kSlotBytes);
+            slot_gen_.push_back(0);
+        }
     }
-    uint32_t *slot = free_slots_.back();
+    Slot slot;
+    slot.index = free_slots_.back();
     free_slots_.pop_back();
+    slot.done = slot_ptr_[slot.index];
+    uint32_t gen = slot_gen_[slot.index] + 1;
+    if (gen > 255) { gen = 1; slot.needs_clear = true; } // tags of 255 owners ago could collide
+    slot_gen_[slot.index] = gen;
+    slot.gen = gen;
     in_use_++;
     return slot;
 }
 
-void GuardState::ReleaseSlot(uint32_t *slot)
+void GuardState::ReleaseSlot(const Slot &slot)
 {
     std::lock_guard<std::mutex> lock(mtx_);
-    free_slots_.push_back(slot);
+    free_slots_.push_back(slot.index);
     in_use_--;
 }
 
@@ -178,12 +245,12 @@ void HipCommand::Synchronize()
 
 HipGuardedCommand::~HipGuardedCommand()
 {
-    if (slot_ != nullptr) guard_state_->ReleaseSlot(slot_);
+    if (slot_.done != nullptr) guard_state_->ReleaseSlot(slot_);
 }
 
 // Level 1 (or guard_mode 0): the plain kernel, nothing else on the stream.
-// Level 2: first launch takes a bitmap slot and clears it in stream order; every
-// launch (first or replay) carries the epoch current at enqueue time.
+// Level 2: the first launch takes a progress map (no clearing: its generation tag is
+// new); every launch (first or replay) carries the epoch current at enqueue time.
 hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
 {
     const bool level2 = q.Level() >= kPreemptLevelDeactivate;
@@ -191,19 +258,24 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
 
     XGuardArgs g;
     g.flag = q.Guard()->FlagDevPtr();
-    g.bitmap = nullptr;
+    g.done = nullptr;
+    g.gen = 0;
     g.epoch = q.Guard()->Epoch();
     g.resume = replay ? 1u : 0u;
+    g.flag_mask = q.Guard()->FlagMask();
 
     if (guarded && level2) {
-        if (slot_ == nullptr) {
+        if (slot_.done == nullptr) {
             XASSERT(n_wg_ <= GuardState::kMaxWorkGroups, "too many work-groups for a guarded command");
             guard_state_ = q.Guard();
             slot_ = guard_state_->AcquireSlot();
-            hipError_t err = hipMemsetAsync(slot_, 0, ((size_t)n_wg_ + 31) / 32 * sizeof(uint32_t), q.Stream());
-            if (err != hipSuccess) return err;
+            if (slot_.needs_clear) {
+                hipError_t err = hipMemsetAsync(slot_.done, 0, GuardState::kSlotBytes, q.Stream());
+                if (err != hipSuccess) return err;
+            }
         }
-        g.bitmap = slot_;
+        g.done = slot_.done;
+        g.gen = slot_.gen;
     }
     return LaunchKernel(q.Stream(), guarded, g);
 }

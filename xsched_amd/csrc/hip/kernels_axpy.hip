@@ -7,7 +7,7 @@
 // are non-temporal: nothing is reused. The preempt word is read after the first
 // step's loads have been issued, so its latency overlaps theirs. Because the
 // update is in place, a work-group must run exactly once: it commits its bit in
-// the progress bitmap after its last store.
+// the progress map after its last store.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 #include "xsched/utils/env.h"
@@ -21,9 +21,7 @@ namespace axpy
 {
 
 constexpr uint32_t kLanes = 64;
-constexpr uint32_t kVecPerStep = 4;                        // float4 per lane per step
-constexpr uint32_t kStepVecs = kLanes * kVecPerStep;       // 256 float4 = 4 KiB per stream
-constexpr uint32_t kStepElems = kStepVecs * 4;             // 1024 floats
+constexpr uint32_t kStepElems = 1024;                      // unit in which chunk sizes are counted
 
 typedef float float4 __attribute__((ext_vector_type(4))); // 128-bit access unit
 
@@ -42,11 +40,14 @@ __device__ __forceinline__ float4 fma4(float a, float4 x, float4 y)
 
 // n4: number of whole float4 in the arrays; tail: the 0..3 trailing scalars, done by
 // the last work-group.
-template <bool kGuard>
+// kVecPerStep float4 per lane and stream are requested before anything is stored:
+// 4 -> steps of 1024 elements, 8 -> steps of 2048 elements.
+template <bool kGuard, uint32_t kVecPerStep>
 __global__ __launch_bounds__(64)
 void AxpyVec4Kernel(float alpha, const float4 *x, float4 *y,
                     uint64_t n4, uint32_t tail, uint32_t steps, XGuardArgs g)
 {
+    constexpr uint32_t kStepVecs = kLanes * kVecPerStep;
     const uint32_t wg = blockIdx.x;
     const uint32_t lane = threadIdx.x;
     const uint64_t wg_base = (uint64_t)wg * steps * kStepVecs;
@@ -109,6 +110,7 @@ void AxpyScalarKernel(float alpha, const float *__restrict__ x, float *__restric
 class HipAxpyCommand final : public HipGuardedCommand
 {
 public:
+    /// steps: chunk size per work-group in units of 1024 elements.
     HipAxpyCommand(float alpha, const float *x, float *y, size_t n, uint32_t steps, uint32_t n_wg,
                    int guard_mode)
         : HipGuardedCommand(n_wg, guard_mode), alpha_(alpha), x_(x), y_(y), n_(n), steps_(steps) {}
@@ -119,16 +121,21 @@ protected:
         if (n_ == 0) return hipSuccess;
         const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
         const dim3 grid(n_wg_), block(kLanes);
+        int64_t lds = 0;
+        GetEnvInt64("XSCHED_HIP_AXPY_LDS_BYTES", lds);
         if (aligned) {
             const uint64_t n4 = n_ / 4;
             const uint32_t tail = (uint32_t)(n_ % 4);
-            if (guarded) {
-                hipLaunchKernelGGL(AxpyVec4Kernel<true>, grid, block, 0, stream, alpha_,
-                                   (const float4 *)x_, (float4 *)y_, n4, tail, steps_, g);
-            } else {
-                hipLaunchKernelGGL(AxpyVec4Kernel<false>, grid, block, 0, stream, alpha_,
-                                   (const float4 *)x_, (float4 *)y_, n4, tail, steps_, g);
-            }
+            // An even chunk is walked in steps of 2048 elements (8 accesses in flight
+            // per lane and stream), an odd one in steps of 1024.
+            const bool wide = (steps_ % 2) == 0;
+            const uint32_t steps = wide ? steps_ / 2 : steps_;
+            const float4 *xv = (const float4 *)x_;
+            float4 *yv = (float4 *)y_;
+            if (guarded && wide)       hipLaunchKernelGGL((AxpyVec4Kernel<true, 8>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (guarded)          hipLaunchKernelGGL((AxpyVec4Kernel<true, 4>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (wide)             hipLaunchKernelGGL((AxpyVec4Kernel<false, 8>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else                       hipLaunchKernelGGL((AxpyVec4Kernel<false, 4>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
         } else {
             if (guarded) {
                 hipLaunchKernelGGL(AxpyScalarKernel<true>, grid, block, 0, stream, alpha_, x_, y_,
@@ -155,11 +162,12 @@ using namespace axpy;
 
 /// Steps (of 1024 elements) per work-group: small enough that the device drains in
 /// tens of microseconds after a flush, large enough that the grid fits the progress
-/// bitmap.
+/// map.
 uint32_t AxpyStepsFor(size_t n)
 {
-    static const int64_t dflt = []() { int64_t v = 4; GetEnvInt64("XSCHED_HIP_AXPY_STEPS", v); return v < 1 ? (int64_t)1 : v; }();
-    uint64_t steps = (uint64_t)dflt;
+    int64_t dflt = 1;
+    GetEnvInt64("XSCHED_HIP_AXPY_STEPS", dflt);
+    uint64_t steps = (uint64_t)(dflt < 1 ? 1 : dflt);
     while (((uint64_t)n + steps * kStepElems - 1) / (steps * kStepElems) > GuardState::kMaxWorkGroups) steps *= 2;
     return (uint32_t)steps;
 }

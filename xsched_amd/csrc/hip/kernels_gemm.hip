@@ -158,7 +158,7 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     for (int t = 0; t < steps; ++t) {
         store_lds();
         if (kGuard && t != 0 && (t % kPollSteps) == 0 && tid == 0) {
-            guard_word = xguard_read_flag(g.flag) == g.epoch ? 1u : 0u;
+            guard_word = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch ? 1u : 0u;
         }
         __syncthreads();
         if (kGuard && t != 0 && (t % kPollSteps) == 0) {

@@ -16,7 +16,7 @@
 //
 // Guard: work-group entry. Tier-2 atomics go to global memory while the group is
 // running, so a group that has started must finish (exactly-once); it commits its
-// bit in the progress bitmap after the flush.
+// byte in the progress map after the flush.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 

@@ -1,5 +1,6 @@
 // XCommand state machine and the HwCommand / HwQueue handle tables.
 // reference preempt/src/xqueue/xcommand.cpp, preempt/src/hal/{hw_command,hw_queue}.cpp
+#include <chrono>
 #include <unordered_map>
 
 #include "xsched/xqueue.h"
@@ -12,6 +13,8 @@ namespace xsched::preempt
 {
 
 // ---- XCommand --------------------------------------------------------------
+
+static constexpr int64_t kWaitSpinMicros = 150;
 
 void XCommand::SetState(XCommandState new_state)
 {
@@ -29,9 +32,19 @@ void XCommand::SetState(XCommandState new_state)
     if (new_state == kCommandStateCompleted && on_completed_ != nullptr) on_completed_(this);
 }
 
+// Short waits (a command of a few microseconds) are polled: sleeping on the state
+// word costs a wake-up through the kernel, which is several times such a command.
 void XCommand::WaitUntil(XCommandState state)
 {
     int32_t cur = state_.load(std::memory_order_acquire);
+    if (cur >= (int32_t)state) return;
+    const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(kWaitSpinMicros);
+    for (int probes = 1; ; ++probes) {
+        cur = state_.load(std::memory_order_acquire);
+        if (cur >= (int32_t)state) return;
+        if ((probes & 63) == 0 && std::chrono::steady_clock::now() >= deadline) break;
+        __builtin_ia32_pause();
+    }
     while (cur < (int32_t)state) {
         state_.wait(cur, std::memory_order_acquire);
         cur = state_.load(std::memory_order_acquire);
