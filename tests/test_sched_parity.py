@@ -1,0 +1,196 @@
+"""Scheduling policies, wire records and name tables of this repository against
+(a) golden vectors produced by the reference's own sources (tests/golden/sched_vectors.json,
+    written by tests/golden/make_sched_vectors.py from oracle/_ref/libsched_ref.so), and
+(b) the live reference build, when oracle/_ref is present in this checkout.
+Decisions are compared exactly; records byte for byte on every byte that carries a field
+(the reference leaves alignment padding uninitialised, this repository zeroes it)."""
+import json
+import os
+import random
+import struct
+import time
+
+import pytest
+
+import sched_driver_api as api
+
+HPF, LAX = 1, 8
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "sched_vectors.json")
+
+
+@pytest.fixture(scope="module")
+def golden():
+    with open(GOLDEN) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="module")
+def probe():
+    if not os.path.exists(api.PROBE_LIB):
+        pytest.fail("oracle/libsched_probe.so missing: run __graft_entry__.build()")
+    return api.probe()
+
+
+@pytest.fixture(scope="module")
+def ref():
+    r = api.ref()
+    if r is None:
+        pytest.skip("oracle/_ref not built here (reference tree absent)")
+    os.environ["XLOG_LEVEL"] = "ERRO"
+    return r
+
+
+def patch_pid(name, data, pid):
+    """Events carry the producer's pid at offset 4; operations at offset 12."""
+    b = bytearray(data)
+    if name.startswith("event_") and name != "event_process_destroy":
+        b[4:8] = struct.pack("<i", pid)
+    if name == "operation_terminate":
+        b[12:16] = struct.pack("<i", pid)
+    return bytes(b)
+
+
+def run_hpf(drv, sc):
+    p = drv.policy(HPF)
+    for h, prio in sc["hints"]:
+        p.priority(h, prio)
+    dec, timers = p.sched([tuple(q) for q in sc["queues"]])
+    p.close()
+    return dec, timers
+
+
+def run_lax(drv, queues, hints):
+    p = drv.policy(LAX)
+    for h, lax, lp, cp in hints:
+        p.laxity(h, lax, lp, cp)
+    out = p.sched(queues)
+    p.close()
+    return out
+
+
+def test_hpf_decisions_match_golden(probe, golden):
+    for sc in golden["hpf"]:
+        dec, timers = run_hpf(probe, sc)
+        assert dec == sc["decisions"]
+        assert timers == sc["timers"] == []
+
+
+def test_lax_decisions_match_golden(probe, golden):
+    now = int(time.time() * 1e6)
+    for sc in golden["lax"]:
+        queues = [(h, d, r, now + rel) for (h, d, r, rel) in sc["queues_rel"]]
+        dec, timers = run_lax(probe, queues, sc["hints"])
+        assert dec == sc["decisions"]
+        assert [t - now for t in timers] == sc["timers_rel"]
+
+
+def test_records_match_golden(probe, golden):
+    me = os.getpid()
+    for name, rec in golden["records"].items():
+        want = bytes.fromhex(rec["hex"])
+        if name.startswith("operation_sched"):
+            op_id, pid, running, suspended = rec["args"]
+            got = probe.sched_operation(op_id, pid, running, suspended)
+            assert got == want, name
+            continue
+        args = [a.encode() if isinstance(a, str) else a for a in rec["args"]]
+        got = api.masked(name, probe.record(name, *args))
+        want = patch_pid(name, want, me) if name != "operation_config" else want
+        assert got == want, name
+
+
+def test_name_tables_match_golden(probe, golden):
+    names = golden["names"]
+    for t, n in names["policy"].items():
+        assert probe.policy_name(int(t)) == n
+    for n, t in names["policy_by_name"].items():
+        assert probe.policy_type_by_name(n) == t
+    for t, n in names["scheduler"].items():
+        assert probe.scheduler_name(int(t)) == n
+    for n, t in names["scheduler_by_name"].items():
+        assert probe.scheduler_type_by_name(n) == t
+    for t, n in names["level"].items():
+        assert probe.level_name(int(t)) == n
+    for t, n in names["platform"].items():
+        assert probe.platform_name(int(t)) == n
+    assert probe.make_device(2, 193) == names["make_device"]["2,193"] == (2 << 32) | 193
+    assert probe.make_device(1, 0) == names["make_device"]["1,0"]
+
+
+def test_policies_against_live_reference(probe, ref):
+    """Fresh random scenarios through both builds."""
+    rnd = random.Random(int.from_bytes(os.urandom(4), "little"))
+    now = int(time.time() * 1e6)
+    far = 3600 * 10**6
+    for _ in range(300):
+        n = rnd.randint(1, 10)
+        handles = rnd.sample(range(1, 10**6), n)
+        queues = [(h, rnd.choice([1, 2, 3]), rnd.random() < 0.5, 0) for h in handles]
+        sc = {"queues": queues, "hints": [(h, rnd.randint(-300, 300)) for h in handles if rnd.random() < 0.7]}
+        assert run_hpf(probe, sc) == run_hpf(ref, sc)
+        lq = [(h, 1, rnd.random() < 0.6, now + rnd.choice([-far, far])) for h in handles]
+        lh = [(h, rnd.choice([-1, 0, 500, 10**5]), rnd.randint(-9, 9), rnd.randint(-9, 9))
+              for h in handles if rnd.random() < 0.7]
+        assert run_lax(probe, lq, lh) == run_lax(ref, lq, lh)
+
+
+def test_records_against_live_reference(probe, ref):
+    rnd = random.Random(3)
+    for _ in range(50):
+        xq, dev = rnd.getrandbits(64), rnd.getrandbits(40)
+        cases = {
+            "hint_priority": [xq, rnd.randint(-256, 255)],
+            "hint_utilization": [rnd.randint(1, 99999), xq, rnd.randint(0, 100)],
+            "hint_timeslice": [rnd.randint(100, 10**7)],
+            "hint_deadline": [xq, rnd.randint(-1, 10**9)],
+            "hint_kdeadline": [rnd.randint(1, 64)],
+            "hint_laxity": [xq, rnd.randint(-1, 10**9), rnd.randint(-255, 255), rnd.randint(-255, 255)],
+            "event_hint_priority": [xq, rnd.randint(-256, 255)],
+            "event_process_create": [bytes(rnd.choice(b"abc xyz-/") for _ in range(rnd.randint(0, 300)))],
+            "event_process_destroy": [rnd.randint(1, 99999)],
+            "event_terminate": [],
+            "event_xqueue_create": [xq, dev, rnd.randint(1, 3), rnd.randint(1, 64), rnd.randint(1, 64)],
+            "event_xqueue_config": [xq, dev, rnd.randint(1, 3), rnd.randint(1, 64), rnd.randint(1, 64)],
+            "event_xqueue_destroy": [xq],
+            "event_xqueue_idle": [xq],
+            "event_xqueue_ready": [xq, rnd.randint(0, 2 * 10**15)],
+            "event_operation_complete": [rnd.getrandbits(60)],
+            "operation_config": [rnd.getrandbits(60), rnd.randint(1, 99999), xq, rnd.randint(0, 3),
+                                 rnd.randint(-1, 64), rnd.randint(-1, 64)],
+            "operation_terminate": [],
+        }
+        for name, args in cases.items():
+            a = api.masked(name, probe.record(name, *args))
+            b = api.masked(name, ref.record(name, *args))
+            assert a == b, name
+        running = [rnd.getrandbits(64) for _ in range(rnd.randint(0, 20))]
+        suspended = [rnd.getrandbits(64) for _ in range(rnd.randint(0, 20))]
+        a = probe.sched_operation(7, 11, running, suspended)
+        assert a == ref.sched_operation(7, 11, running, suspended)
+        # each side re-reads the other's bytes with its own CopyConstructor
+        assert probe.operation_roundtrip(a) == a == ref.operation_roundtrip(a)
+        ev = ref.record("event_xqueue_ready", xq, 123456789)
+        assert api.masked("event_xqueue_ready", probe.event_roundtrip(ev)) == api.masked("event_xqueue_ready", ev)
+        hev = ref.record("event_hint_priority", xq, 5)
+        assert api.masked("event_hint_priority", probe.event_roundtrip(hev)) == api.masked("event_hint_priority", hev)
+
+
+def test_hpf_closed_form(probe):
+    """What HPF is, stated independently of either implementation: per device the bar is
+    the highest priority among ready queues (clamped to [-255, 255], default 0); a queue
+    is suspended iff its priority is below its device's bar; no ready queue, no bar."""
+    rnd = random.Random(11)
+    for _ in range(200):
+        n = rnd.randint(1, 9)
+        handles = list(range(100, 100 + n))
+        dev = {h: rnd.choice([10, 20]) for h in handles}
+        ready = {h: rnd.random() < 0.5 for h in handles}
+        raw = {h: rnd.randint(-400, 400) for h in handles if rnd.random() < 0.8}
+        prio = {h: max(-255, min(255, raw[h])) if h in raw else 0 for h in handles}
+        bar = {}
+        for h in handles:
+            if ready[h]:
+                bar[dev[h]] = max(bar.get(dev[h], -10**9), prio[h])
+        want = [1 if prio[h] < bar.get(dev[h], -255) else 0 for h in handles]
+        sc = {"queues": [(h, dev[h], ready[h], 0) for h in handles], "hints": list(raw.items())}
+        assert run_hpf(probe, sc)[0] == want
