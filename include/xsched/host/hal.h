@@ -38,8 +38,8 @@ XResult HostKernelCommandCreate(HwCommandHandle *cmd, HostKernelFn fn, void *arg
 XResult HostVecAddCommandCreate(HwCommandHandle *cmd, const float *a, const float *b,
                                 float *c, size_t n, int guarded);
 
-/* y[i] = alpha * x[i] + y[i] (one multiply, one add, each rounded to fp32), in
- * place, work-groups of 16384 elements. */
+/* y[i] = fma(alpha, x[i], y[i]) (one rounding per element), in place, work-groups
+ * of 16384 elements. */
 XResult HostAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const float *x, float *y,
                               size_t n, int guarded);
 

@@ -1,5 +1,6 @@
 // Host (CPU) hardware-queue adapter; see include/xsched/host/hal.h.
 #include <atomic>
+#include <cmath>
 #include <condition_variable>
 #include <deque>
 #include <mutex>
@@ -27,7 +28,6 @@ struct Ticket
     std::shared_ptr<class HostKernelCommand> cmd;
     uint32_t epoch;   // deactivation count at launch time
     uint64_t seq;     // position in this queue's launch order
-    bool mark;        // completion of this ticket completes the command's marker
 };
 
 class HostKernelCommand : public HwCommand
@@ -144,7 +144,7 @@ private:
         {
             std::lock_guard<std::mutex> lock(mtx_);
             const uint32_t epoch = epoch_.load(std::memory_order_acquire);
-            tickets_.push_back(Ticket { std::move(cmd), epoch, ++launched_, true });
+            tickets_.push_back(Ticket { std::move(cmd), epoch, ++launched_ });
         }
         cv_.notify_one();
     }
@@ -243,11 +243,8 @@ static void AxpyWg(void *p, uint32_t wg, uint32_t)
 {
     const VecArgs &v = *(const VecArgs *)p;
     const size_t lo = (size_t)wg * kWgElems, hi = std::min(v.n, lo + kWgElems);
-    for (size_t i = lo; i < hi; ++i) {
-        // Two roundings on purpose (no fused multiply-add), matching the device kernel.
-        volatile float prod = v.alpha * v.a[i];
-        v.c[i] = prod + v.c[i];
-    }
+    // One rounding per element (fused multiply-add), like the device kernel.
+    for (size_t i = lo; i < hi; ++i) v.c[i] = std::fmaf(v.alpha, v.a[i], v.c[i]);
 }
 
 } // namespace xsched::host
