@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 os.environ.setdefault("XLOG_LEVEL", "WARN")
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
+# Background in-flight window: one kernel running and one queued behind it keeps the
+# device busy (a 2^28 AXPY runs ~0.5 ms, a launch costs ~10 us) and bounds what a
+# suspended queue still has on the device to two kernels.
+BG_THRESHOLD, BG_BATCH = 2, 1
 
 
 class QueueSpec(Structure):
@@ -80,7 +84,7 @@ def axpy_bytes(n):
 
 def run_config2(lib, steps, warmup, bg_n, fg_n, bg_level=1, bg_guard=1):
     cfg = Config(HPF, 1,
-                 spec(AXPY, bg_n, bg_guard, bg_level, 4, 2, 1),
+                 spec(AXPY, bg_n, bg_guard, bg_level, BG_THRESHOLD, BG_BATCH, 1),
                  spec(AXPY, fg_n, 0, 1, 8, 4, 2, period_us=20000),
                  64, 0)
     b = lib.XBenchCreate(byref(cfg))
@@ -115,7 +119,7 @@ def run_config2(lib, steps, warmup, bg_n, fg_n, bg_level=1, bg_guard=1):
 
 def run_bg_variant(lib, bg_n, level, guard, commands=40):
     """Average device time per background launch for one guard variant."""
-    cfg = Config(0, 1, spec(AXPY, bg_n, guard, level, 4, 2, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
+    cfg = Config(0, 1, spec(AXPY, bg_n, guard, level, BG_THRESHOLD, BG_BATCH, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
     b = lib.XBenchCreate(byref(cfg))
     assert b
     try:
@@ -128,7 +132,7 @@ def run_bg_variant(lib, bg_n, level, guard, commands=40):
 
 
 def run_preempt(lib, bg_n, level, samples=200):
-    cfg = Config(0, 1, spec(AXPY, bg_n, 1, level, 4, 2, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
+    cfg = Config(0, 1, spec(AXPY, bg_n, 1, level, BG_THRESHOLD, BG_BATCH, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
     b = lib.XBenchCreate(byref(cfg))
     assert b
     try:
@@ -147,7 +151,7 @@ def cpu_baseline(seconds_budget=15.0):
         from oracle import cpu_baseline as cb
     except Exception as e:  # oracle not built
         return {"value": None, "unit": "us", "cores": 0, "kind": "port", "sample": f"unavailable: {e}"}
-    return cb.run_config2_sample(seconds_budget)
+    return cb.run_config2_sample(seconds_budget, samples=300)
 
 
 def main():
@@ -216,7 +220,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "cfg2: L1 HPF, bg AXPY 2^%d back-to-back, fg AXPY 2^%d every 20 ms"
                                % (a.bg_log2, a.fg_log2),
-                   "bg_threshold": 4, "bg_batch": 2, "fg_threshold": 8, "fg_batch": 4,
+                   "bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4,
                    "percentile_rule": "sorted[floor(p*n)]"},
         "fg_latency_us": {"alone_p50": p50a, "alone_p99": p99a, "contended_p50": p50c,
                           "contended_p99": p99c, "p99_ratio": p99c / p99a if p99a else None},

@@ -40,7 +40,7 @@ class NativeLibraryMissing(RuntimeError):
     """Raised when a native library has not been built; there is no fallback."""
 
 
-def _load(name, mode=ctypes.RTLD_GLOBAL):
+def _load(name, mode=ctypes.RTLD_LOCAL):
     path = os.path.join(_LIB_DIR, name)
     if not os.path.exists(path):
         raise NativeLibraryMissing(
