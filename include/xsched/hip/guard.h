@@ -4,8 +4,7 @@
 // XGuardArgs, and brackets the work of each work-group with the calls below:
 //
 //     XGuardWave guard(g, wg);      // or XGuardBlock for multi-wave work-groups
-//     ... issue the loads of the work-group's inputs ...
-//     if (!guard.Enter()) return;   // flushed (or already done): store nothing
+//     if (!guard.Enter()) return;   // flushed (or already done): touch nothing
 //     ... compute, store ...
 //     guard.Commit();               // mark the work-group done
 //
@@ -32,8 +31,8 @@
 // counter, so nothing has to be cleared or read back on resume; one byte per
 // work-group instead of two words.
 //
-// Cost: one uncached scalar load per work-group whose latency hides behind the first
-// input loads, one compare, and one byte store per work-group.
+// Cost: one uncached scalar load per work-group (hidden by the other resident
+// waves), one compare, and one byte store per work-group.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -70,8 +69,7 @@ __device__ __forceinline__ const uint32_t *xguard_flag_copy(const XGuardArgs &g,
 // with the GLC bit always fetches memory-side data (the word lives in fine-grained
 // memory). Load and wait form one asm statement so the compiler never touches the
 // destination register while the load is in flight. Vector loads issued before
-// this call stay in flight across it (it waits on the scalar counter only), which
-// is how a kernel hides the latency of the word: inputs first, then Enter().
+// this call stay in flight across it (it waits on the scalar counter only).
 __device__ __forceinline__ uint32_t xguard_read_flag(const uint32_t *flag)
 {
     uint32_t v;

@@ -8,6 +8,7 @@ Produces, under xsched_amd/lib/:
     libhalhip.so    MI355X HIP adapter: Level-1/Level-2 queue, guarded
                     kernels, benchmark harness                         (hipcc, gfx950)
     xserver         scheduler daemon                                   (g++)
+    traffic_probe   counter-run driver for the AXPY kernel             (hipcc)
 and, under oracle/, the checker libraries (see oracle/Makefile).
 
 Everything is compiled for gfx950 only; hipcc cross-compiles without a GPU.
@@ -94,6 +95,10 @@ def build_hip(extra, jobs):
         return
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-o", os.path.join(LIB, "libhalhip.so")]
          + objs + ["-L", LIB, "-Wl,-rpath,$ORIGIN", "-lpreempt", "-pthread"])
+    probe = os.path.join(CSRC, "bench", "traffic_probe.hip")
+    if os.path.exists(probe):
+        _run(["hipcc"] + HIPFLAGS + extra + [probe, "-o", os.path.join(LIB, "traffic_probe"),
+             "-L", LIB, "-Wl,-rpath,$ORIGIN", "-lhalhip", "-lpreempt", "-pthread"])
 
 
 def build_oracle():

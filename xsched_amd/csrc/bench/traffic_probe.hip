@@ -1,0 +1,69 @@
+// Small driver for hardware-counter runs: launches a plain copy kernel of known size
+// (1 GiB read + 1 GiB written) and then the AXPY victim kernel through an XQueue in
+// its three forms (plain, guarded at level 1, guarded at level 2), a few times each.
+// Run it under `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`: the copy kernel's
+// counters give the scale factor of the counter, the AXPY rows the kernel's real HBM
+// traffic per launch.
+#include <cstdio>
+#include <cstdlib>
+
+#include <hip/hip_runtime.h>
+
+#include "xsched/hip/hal.h"
+#include "xsched/xsched.h"
+
+#define CHECK_HIP(e) do { hipError_t r_ = (e); if (r_ != hipSuccess) { \
+    fprintf(stderr, "HIP error %s at %s\n", hipGetErrorString(r_), #e); exit(1); } } while (0)
+#define CHECK_X(e) do { XResult r_ = (e); if (r_ != kXSchedSuccess) { \
+    fprintf(stderr, "XSched error %d at %s\n", (int)r_, #e); exit(1); } } while (0)
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+__global__ void PlainCopyKernel(const f4 *src, f4 *dst, size_t n4)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+        dst[i] = src[i];
+    }
+}
+
+int main(int argc, char **argv)
+{
+    const size_t n = argc > 1 ? (size_t)atoll(argv[1]) : (size_t)1 << 28;
+    const int reps = argc > 2 ? atoi(argv[2]) : 5;
+    float *x = nullptr, *y = nullptr;
+    CHECK_HIP(hipMalloc((void **)&x, n * 4));
+    CHECK_HIP(hipMalloc((void **)&y, n * 4));
+    CHECK_HIP(hipMemset(x, 0, n * 4));
+    CHECK_HIP(hipMemset(y, 0, n * 4));
+    hipStream_t stream;
+    CHECK_HIP(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+
+    for (int i = 0; i < reps; ++i) {
+        hipLaunchKernelGGL(PlainCopyKernel, dim3(8192), dim3(256), 0, stream, (const f4 *)x, (f4 *)y, n / 4);
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+
+    CHECK_X(XHintSetScheduler(kSchedulerAppManaged, kPolicyUnknown));
+    HwQueueHandle hwq;
+    XQueueHandle xq;
+    CHECK_X(HipQueueCreate(&hwq, stream));
+    CHECK_X(XQueueCreate(&xq, hwq, kPreemptLevelBlock, kQueueCreateFlagNone));
+    CHECK_X(XQueueSetLaunchConfig(xq, 2, 1));
+    auto run = [&](int guard) {
+        for (int i = 0; i < reps; ++i) {
+            HwCommandHandle cmd;
+            CHECK_X(HipAxpyCommandCreate(&cmd, 0.5f, x, y, n, guard));
+            CHECK_X(XQueueSubmit(xq, cmd));
+        }
+        CHECK_X(XQueueWaitAll(xq));
+    };
+    run(0);                                                   // AxpyVec4Kernel<false, 4>
+    run(2);                                                   // AxpyVec4Kernel<true, 4>, no progress map
+    CHECK_X(XQueueSetPreemptLevel(xq, kPreemptLevelDeactivate));
+    run(1);                                                   // AxpyVec4Kernel<true, 4> with progress map
+    CHECK_X(XQueueDestroy(xq));
+    CHECK_X(HwQueueDestroy(hwq));
+    printf("traffic_probe: n=%zu reps=%d copy_bytes_read=%zu copy_bytes_written=%zu axpy_algorithmic_bytes=%zu\n",
+           n, reps, n * 4, n * 4, n * 12);
+    return 0;
+}
