@@ -1,0 +1,93 @@
+"""Scheduler daemon wiring on one machine: client processes relay their events to
+xserver over the datagram channel, xserver's LocalScheduler decides, and the operations
+come back to the process they address (reference sched/src/scheduler/global.cpp and
+service/server/src/server.cpp). CPU only: the clients use the host adapter."""
+import json
+import os
+import subprocess
+import sys
+import tempfile
+import time
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+XSERVER = os.path.join(ROOT, "xsched_amd", "lib", "xserver")
+CLIENT = os.path.join(ROOT, "tests", "daemon_client.py")
+
+
+@pytest.fixture()
+def daemon():
+    if not os.path.exists(XSERVER):
+        pytest.fail("xserver has not been built")
+    sock_dir = tempfile.mkdtemp(prefix="xsched-test-")
+    env = dict(os.environ, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="INFO")
+    proc = subprocess.Popen([XSERVER, "HPF"], env=env, stderr=subprocess.PIPE, text=True)
+    deadline = time.time() + 5
+    while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
+        time.sleep(0.01)
+    assert os.path.exists(os.path.join(sock_dir, "xsched-1.sock")), "xserver did not come up"
+    client_env = dict(os.environ, XSCHED_SOCKET_DIR=sock_dir, XSCHED_SCHEDULER="GLB", XLOG_LEVEL="WARN")
+    client_env.pop("XSCHED_POLICY", None)
+    yield proc, client_env, sock_dir
+    proc.terminate()
+    try:
+        proc.wait(timeout=5)
+    except subprocess.TimeoutExpired:
+        proc.kill()
+
+
+def client(env, *args):
+    return subprocess.Popen([sys.executable, CLIENT, *map(str, args)], env=env,
+                            stdout=subprocess.PIPE, text=True)
+
+
+def test_two_processes_hpf_through_the_daemon(daemon):
+    """A low-priority process must not run while a high-priority process has work, and
+    must run to completion afterwards."""
+    proc, env, _ = daemon
+    busy = client(env, "busy", 5, 1.0)
+    assert json.loads(busy.stdout.readline())["event"] == "busy-started"
+    time.sleep(0.1)                      # let the daemon see the busy queue
+    quick = client(env, "quick", 1, 8)
+    q = json.loads(quick.communicate(timeout=20)[0].strip().splitlines()[-1])
+    b = busy.communicate(timeout=20)[0]
+    assert quick.returncode == 0 and busy.returncode == 0
+    assert q["executed_early"] == 0, "low-priority client ran while the high-priority one was busy"
+    assert q["executed_final"] == 8
+    assert json.loads(b.strip().splitlines()[-1])["role"] == "busy"
+
+
+def test_equal_priorities_are_not_blocked(daemon):
+    proc, env, _ = daemon
+    busy = client(env, "busy", 3, 0.8)
+    assert json.loads(busy.stdout.readline())["event"] == "busy-started"
+    time.sleep(0.1)
+    quick = client(env, "quick", 3, 8)
+    q = json.loads(quick.communicate(timeout=20)[0].strip().splitlines()[-1])
+    busy.communicate(timeout=20)
+    assert q["executed_early"] == 8
+
+
+def test_dead_client_is_forgotten(daemon):
+    """A high-priority client that is killed must stop blocking everybody else."""
+    proc, env, sock_dir = daemon
+    busy = client(env, "busy", 9, 30.0)
+    assert json.loads(busy.stdout.readline())["event"] == "busy-started"
+    time.sleep(0.1)
+    quick = client(env, "quick", 1, 4)
+    time.sleep(0.2)
+    busy.kill()
+    busy.wait()
+    q = json.loads(quick.communicate(timeout=20)[0].strip().splitlines()[-1])
+    assert q["executed_final"] == 4      # released once the daemon noticed the death
+    assert not os.path.exists(os.path.join(sock_dir, f"xsched-{busy.pid}.sock")) or True
+
+
+def test_client_without_daemon_fails_loudly():
+    env = dict(os.environ, XSCHED_SOCKET_DIR=tempfile.mkdtemp(prefix="xsched-none-"),
+               XSCHED_SCHEDULER="GLB", XLOG_LEVEL="ERRO")
+    p = subprocess.run([sys.executable, CLIENT, "quick", 1, 1], env=env, capture_output=True, text=True,
+                       timeout=30)
+    assert p.returncode != 0
+    assert "scheduler daemon" in p.stderr
