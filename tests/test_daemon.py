@@ -87,7 +87,7 @@ def test_dead_client_is_forgotten(daemon):
 def test_client_without_daemon_fails_loudly():
     env = dict(os.environ, XSCHED_SOCKET_DIR=tempfile.mkdtemp(prefix="xsched-none-"),
                XSCHED_SCHEDULER="GLB", XLOG_LEVEL="ERRO")
-    p = subprocess.run([sys.executable, CLIENT, "quick", 1, 1], env=env, capture_output=True, text=True,
+    p = subprocess.run([sys.executable, CLIENT, "quick", "1", "1"], env=env, capture_output=True, text=True,
                        timeout=30)
     assert p.returncode != 0
     assert "scheduler daemon" in p.stderr
