@@ -154,6 +154,20 @@ def cpu_baseline(seconds_budget=15.0):
     return cb.run_config2_sample(seconds_budget, samples=300)
 
 
+def recorded_traffic(bg_n):
+    """HBM bytes per launch of the plain 2^28 AXPY kernel as recorded by the two
+    rocprofv3 counter runs summarised under profiles/ (counters cannot be read from
+    inside this process); None for any other size or when the summary is absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                        "axpy_2p28_hbm_traffic.md")
+    if bg_n != 1 << 28 or not os.path.exists(path):
+        return None
+    for ln in open(path):
+        if ln.startswith("traffic_bytes_per_launch_plain:"):
+            return int(ln.split(":")[1])
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -227,7 +241,7 @@ def main():
         "bg": {"alone_GBs": axpy_bytes(bg_n) / r["bg_alone_ms"] / 1e6, "contended_GBs": bg_kept,
                "commands_in_timed_region": r["bg_cont_cmds"]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(bg_n),
                      "kernel": "AxpyVec4Kernel", "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
                      "avg_launch_ms": per_launch_ms},
     }

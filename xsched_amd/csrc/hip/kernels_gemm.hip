@@ -250,6 +250,10 @@ EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void 
         return kXSchedErrorInvalidValue;
     }
     if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) return kXSchedErrorInvalidValue;
+    // one progress-map byte per tile
+    if ((uint64_t)(M / gemm::kTile) * (uint64_t)(N / gemm::kTile) > GuardState::kMaxWorkGroups) {
+        return kXSchedErrorInvalidValue;
+    }
     *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, guard));
     return kXSchedSuccess;
 }
