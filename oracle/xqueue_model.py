@@ -9,9 +9,12 @@ and resumes. It restates, step for step,
     preempt/src/xqueue/command_buffer.cpp  (Dequeue :39-97: the synthetic batch-sync then
                                             drain marker when the buffer runs empty)
     preempt/src/xqueue/async_xqueue.cpp    (Suspend :91-113, Resume :115-150)
-of the reference. The reference's own build of these files needs the un-vendored `ipc`
-library, so the model is pinned by facts read off that code (tests/test_xqueue_model.py)
-rather than by running it.
+of the reference. Pinned two ways: by the traces the reference's own build of these files
+produces for fixed and seeded random scripts (tests/golden/xqueue_traces.json, written by
+tests/golden/make_xqueue_traces.py from oracle/_ref/libxqueue_ref.so; compared call for
+call in tests/test_xqueue_trace.py), and by facts read off the code
+(tests/test_xqueue_model.py). Not pinned: which thread wins a race inside the reference's
+launch thread when the scripts do not serialise it; the scripts here always do.
 
 Trace tokens (what a hardware adapter observes):
     L<idx>     HwQueue::Launch of command idx      L<idx>*  ... with a completion marker

@@ -1,8 +1,10 @@
 // ORACLE - test infrastructure only. A recording hardware queue: an HwQueue whose
 // "device" is a watermark the test advances by hand, and which writes down every call
-// the XQueue core makes on it. Tests drive the shipped XQueue core (libpreempt.so)
-// through the public C API with this adapter and compare the recorded trace with the
-// launch-loop model in oracle/xqueue_model.py (same token vocabulary).
+// the XQueue core makes on it. It is compiled twice: against this repository's headers
+// (libxqueue_probe.so, driving the shipped libpreempt.so) and against the reference's
+// headers together with the reference's own XQueue sources (_ref/libxqueue_ref.so). Tests
+// drive both through the public C API and compare the recorded traces with each other and
+// with the launch-loop model in oracle/xqueue_model.py (same token vocabulary).
 #include <condition_variable>
 #include <cstring>
 #include <mutex>
