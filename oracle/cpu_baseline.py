@@ -1,6 +1,8 @@
-"""ORACLE - test infrastructure only: runs the CPU port of the headline workload
-(oracle/xsched_port.cpp) on a bounded sample and reports it in bench.py's
-`cpu_baseline` format."""
+"""ORACLE - test infrastructure only: runs the headline workload on CPU cores, on a
+bounded sample, and reports it in bench.py's `cpu_baseline` format. Preferred: the
+reference's own XQueue core, scheduler and policy (oracle/_ref/libxqueue_ref.so, kind
+"reference") driving scalar CPU kernels through oracle/host_bench.cpp; without that build,
+the compact port of the host loop in oracle/xsched_port.cpp (kind "port")."""
 import ctypes
 import os
 from ctypes import POINTER, byref, c_double, c_int, c_int64, c_uint64
@@ -13,34 +15,50 @@ def _pct(samples, p):
     return s[min(int(p * len(s)), len(s) - 1)]
 
 
-def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100):
+def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100, which="auto"):
     """Same structure as the GPU run (bg AXPY back to back at priority 1, fg AXPY every
     20 ms at priority 2, level 1, HPF), with both arrays scaled down by 2^scale_log2 so
     that the sample takes on the order of ten seconds of CPU work."""
+    ref_path = os.path.join(_DIR, "_ref", "libxqueue_ref.so")
     path = os.path.join(_DIR, "libxsched_port.so")
-    if not os.path.exists(path):
-        raise RuntimeError(f"{path} missing: run `make -C oracle`")
-    lib = ctypes.CDLL(path)
-    lib.port_run_fg_bg_axpy.argtypes = [c_uint64, c_uint64, c_int64, c_int, c_int, c_int,
-                                        POINTER(c_double), POINTER(c_double), POINTER(c_uint64),
-                                        POINTER(c_double), POINTER(c_uint64)]
+    if which == "auto":
+        which = "reference" if os.path.exists(ref_path) else "port"
+    if which == "reference":
+        os.environ.setdefault("XLOG_LEVEL", "ERRO")
+        fn = ctypes.CDLL(ref_path, mode=ctypes.RTLD_LOCAL).hostbench_run_fg_bg_axpy
+    elif which == "shipped":
+        fn = ctypes.CDLL(os.path.join(_DIR, "libhostbench.so"), mode=ctypes.RTLD_LOCAL).hostbench_run_fg_bg_axpy
+    else:
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} missing: run `make -C oracle`")
+        fn = ctypes.CDLL(path).port_run_fg_bg_axpy
+    fn.restype = c_int
+    fn.argtypes = [c_uint64, c_uint64, c_int64, c_int, c_int, c_int, POINTER(c_double), POINTER(c_double),
+                   POINTER(c_uint64), POINTER(c_double), POINTER(c_uint64)]
     bg_n, fg_n = (1 << 28) >> scale_log2, (1 << 22) >> scale_log2
     alone = (c_double * samples)()
     cont = (c_double * samples)()
     bg_cmds, secs, chk = c_uint64(), c_double(), c_uint64()
-    lib.port_run_fg_bg_axpy(bg_n, fg_n, 20000, samples, 4, 2, alone, cont, byref(bg_cmds), byref(secs),
-                            byref(chk))
+    rc = fn(bg_n, fg_n, 20000, samples, 4, 2, alone, cont, byref(bg_cmds), byref(secs), byref(chk))
+    if rc != 0:
+        raise RuntimeError(f"CPU baseline run failed with XResult {rc}")
     alone, cont = list(alone)[5:], list(cont)[5:]
     bg_gbs = 12.0 * bg_n * bg_cmds.value / secs.value / 1e9 if secs.value else 0.0
     return {
         "value": _pct(cont, 0.99),
         "unit": "us",
         "cores": 7,
-        "kind": "port",
-        "sample": ("oracle/xsched_port.cpp: CPU restatement of XSched's host loop (2 XQueues, level 1, HPF), "
-                   "scalar single-threaded fmaf AXPY per queue; bg 2^%d and fg 2^%d elements (1/%d of the GPU "
-                   "sizes), fg every 20 ms, %d fg samples; threads: 2 executors + 2 launch workers + 1 "
-                   "scheduler + 2 submitters" % (28 - scale_log2, 22 - scale_log2, 1 << scale_log2, len(cont))),
+        "kind": "port" if which == "port" else "reference" if which == "reference" else "shipped-host",
+        "sample": ("%s (2 XQueues, level 1, HPF, bg window 4/2, fg 8/4), scalar single-threaded fmaf AXPY per "
+                   "queue; bg 2^%d and fg 2^%d elements (1/%d of the GPU sizes), fg every 20 ms, %d fg samples; "
+                   "threads: 2 executors + 2 launch workers + 1 scheduler + 2 submitters"
+                   % ({"port": "oracle/xsched_port.cpp: CPU restatement of XSched's host loop",
+                       "reference": "oracle/_ref/libxqueue_ref.so: XSched's own XQueue core, local scheduler and "
+                                    "HPF policy compiled from the reference sources, driving this repository's "
+                                    "host adapter through oracle/host_bench.cpp",
+                       "shipped-host": "shipped libpreempt.so + libhalhost.so through oracle/host_bench.cpp"}
+                      ["port" if which == "port" else "reference" if which == "reference" else "shipped-host"],
+                      28 - scale_log2, 22 - scale_log2, 1 << scale_log2, len(cont))),
         "fg_alone_p50_us": _pct(alone, 0.5), "fg_alone_p99_us": _pct(alone, 0.99),
         "fg_contended_p50_us": _pct(cont, 0.5), "fg_contended_p99_us": _pct(cont, 0.99),
         "bg_GBs": bg_gbs,
@@ -49,4 +67,5 @@ def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100):
 
 if __name__ == "__main__":
     import json
-    print(json.dumps(run_config2_sample()))
+    import sys
+    print(json.dumps(run_config2_sample(which=sys.argv[1] if len(sys.argv) > 1 else "auto")))
