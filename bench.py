@@ -1,165 +1,115 @@
 #!/usr/bin/env python3
 """Headline benchmark: foreground latency under a saturating background on one MI355X.
 
-Workload (BASELINE.json configs[1]): background XQueue streams fp32 AXPY y = 0.5*x + y
-over 2^28 elements back to back (Level-1, HPF policy, priority 1); foreground XQueue
-submits the same kernel over 2^22 elements every 20 ms (priority 2). One "step" is one
-foreground command under contention (submit -> XQueueWaitAll returns).
+Default workload (BASELINE.json configs[1], `--config 2`): a background XQueue streams fp32
+AXPY y = 0.5*x + y over 2^28 elements back to back (Level-1, HPF policy, priority 1); a
+foreground XQueue submits the same kernel over 2^22 elements every 20 ms (priority 2). One
+"step" is one foreground command under contention (submit -> XQueueWaitAll returns).
 
 Prints ONE JSON line. `value` is the foreground p99 latency under contention in
-microseconds (percentile rule sorted[floor(p*n)], as XSched's own DataProcessor). The
-same line carries the background's achieved HBM bandwidth against the 8 TB/s peak
-(`roofline`), the guard overhead, the Level-2 preemption latency, and a CPU baseline of
-the same workload run through a CPU restatement of XSched's host loop (`cpu_baseline`).
+microseconds (percentile rule sorted[floor(p*n)], as XSched's own DataProcessor). The same
+line carries the background kernel's achieved rate against the MI355X peak (`roofline`),
+the guard overhead, the Level-2 preemption latency, and a CPU baseline of the same workload
+(`cpu_baseline`).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+The other single-GPU configurations print a line of the same shape:
+    --config 3   Level-2 guarded bf16 GEMM 8192^3 back to back, foreground GEMM 1024^3
+                 every 5 ms (MFMA roofline, guard on/off, preemption latency)
+    --config 4   laxity policy: 4 background XQueues histogramming 2^26 Zipf keys,
+                 foreground 2^20 keys every 2 ms with a 1 ms deadline (deadline-miss rate)
+    --config 5   16 XQueues, priorities 0-15, cycling AXPY 2^24 / GEMM 2048^3 / histogram
+                 2^24, exponential arrivals (mean 5 ms, seed 7), HPF, Level-2
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
 """
 import argparse
-import ctypes
 import json
 import os
 import sys
 import time
-from ctypes import POINTER, Structure, byref, c_double, c_int32, c_int64, c_uint64, c_void_p
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 os.environ.setdefault("XLOG_LEVEL", "WARN")
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, vendor figure
+MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 # Background in-flight window: one kernel running and one queued behind it keeps the
 # device busy (a 2^28 AXPY runs ~0.5 ms, a launch costs ~10 us) and bounds what a
 # suspended queue still has on the device to two kernels.
 BG_THRESHOLD, BG_BATCH = 2, 1
 
 
-class QueueSpec(Structure):
-    _fields_ = [("kind", c_int32), ("guard", c_int32), ("n", c_uint64), ("level", c_int32),
-                ("threshold", c_int32), ("batch", c_int32), ("priority", c_int32),
-                ("laxity_us", c_int64), ("period_us", c_int64)]
-
-
-class Config(Structure):
-    _fields_ = [("policy", c_int32), ("n_bg", c_int32), ("bg", QueueSpec), ("fg", QueueSpec),
-                ("bg_burst", c_int32), ("seed", c_uint64)]
-
-
-class PhaseResult(Structure):
-    _fields_ = [("elapsed_s", c_double), ("bg_commands", c_uint64), ("bg_stream_ms", c_double),
-                ("bg_stream_cmds", c_uint64), ("fg_samples", c_uint64), ("fg_deadline_miss", c_uint64),
-                ("stats", c_uint64 * 8)]
-
-
-def bind_harness(lib):
-    lib.XBenchCreate.restype = c_void_p
-    lib.XBenchCreate.argtypes = [POINTER(Config)]
-    lib.XBenchDestroy.argtypes = [c_void_p]
-    lib.XBenchRunForegroundAlone.argtypes = [c_void_p, ctypes.c_int, POINTER(c_double), POINTER(PhaseResult)]
-    lib.XBenchRunBackgroundAlone.argtypes = [c_void_p, ctypes.c_int, POINTER(PhaseResult)]
-    lib.XBenchRunContended.argtypes = [c_void_p, ctypes.c_int, POINTER(c_double), POINTER(PhaseResult)]
-    lib.XBenchRunPreempt.argtypes = [c_void_p, ctypes.c_int, POINTER(c_double), POINTER(c_double),
-                                     POINTER(PhaseResult)]
-    lib.XBenchReadOutput.argtypes = [c_void_p, ctypes.c_int, ctypes.c_int, c_uint64, c_uint64, c_void_p,
-                                     POINTER(c_uint64)]
-    return lib
-
-
-def pct(samples, p):
-    """XSched's percentile rule: sorted[floor(p*n)] (utils/data.h:57-65)."""
-    s = sorted(samples)
-    return s[min(int(p * len(s)), len(s) - 1)] if s else 0.0
-
-
-AXPY, GEMM, HIST = 0, 1, 2
-HPF, LAX = 1, 8
-
-
-def spec(kind, n, guard, level, threshold, batch, priority, laxity_us=-1, period_us=0):
-    return QueueSpec(kind, guard, n, level, threshold, batch, priority, laxity_us, period_us)
-
-
 def axpy_bytes(n):
     return 12.0 * n  # read x, read y, write y
 
 
-def run_config2(lib, steps, warmup, bg_n, fg_n, bg_level=1, bg_guard=1):
-    cfg = Config(HPF, 1,
-                 spec(AXPY, bg_n, bg_guard, bg_level, BG_THRESHOLD, BG_BATCH, 1),
-                 spec(AXPY, fg_n, 0, 1, 8, 4, 2, period_us=20000),
-                 64, 0)
-    b = lib.XBenchCreate(byref(cfg))
-    assert b, "XBenchCreate failed"
-    out = {}
-    try:
-        res = PhaseResult()
-        lat = (c_double * (steps + warmup))()
-        # foreground alone
-        assert lib.XBenchRunForegroundAlone(b, steps + warmup, lat, byref(res)) == 0
-        alone = list(lat)[warmup:]
-        # background alone
-        assert lib.XBenchRunBackgroundAlone(b, 8, byref(res)) == 0      # warm-up
-        assert lib.XBenchRunBackgroundAlone(b, 40, byref(res)) == 0
-        bg_alone_ms = res.bg_stream_ms / res.bg_stream_cmds
-        # contended: exactly `steps` timed foreground steps after `warmup` untimed ones
-        assert lib.XBenchRunContended(b, warmup, lat, byref(res)) == 0 if warmup else True
-        t0 = time.perf_counter()
-        assert lib.XBenchRunContended(b, steps, lat, byref(res)) == 0
-        wall = time.perf_counter() - t0
-        cont = list(lat)[:steps]
-        out.update(
-            fg_alone=alone, fg_contended=cont, wall_s=wall,
-            bg_alone_ms=bg_alone_ms,
-            bg_cont_ms=(res.bg_stream_ms / res.bg_stream_cmds) if res.bg_stream_cmds else None,
-            bg_cont_cmds=int(res.bg_commands), bg_cont_elapsed=res.elapsed_s,
-            stats=list(res.stats))
-    finally:
-        lib.XBenchDestroy(b)
-    return out
+def gemm_flops(n):
+    return 2.0 * n * n * n
 
 
-def run_bg_variant(lib, bg_n, level, guard, commands=40):
-    """Average device time per background launch for one guard variant."""
-    cfg = Config(0, 1, spec(AXPY, bg_n, guard, level, BG_THRESHOLD, BG_BATCH, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
-    b = lib.XBenchCreate(byref(cfg))
-    assert b
-    try:
-        res = PhaseResult()
-        assert lib.XBenchRunBackgroundAlone(b, 8, byref(res)) == 0
-        assert lib.XBenchRunBackgroundAlone(b, commands, byref(res)) == 0
+def hist_bytes(n):
+    return 4.0 * n  # one int32 key read
+
+
+def fg_summary(H, alone, cont):
+    p50a, p99a = H.pct(alone, 0.50), H.pct(alone, 0.99)
+    p50c, p99c = H.pct(cont, 0.50), H.pct(cont, 0.99)
+    return {"alone_p50": p50a, "alone_p99": p99a, "contended_p50": p50c, "contended_p99": p99c,
+            "p99_ratio": p99c / p99a if p99a else None}
+
+
+def bg_ms_per_launch(H, kind, n, level, guard, commands=40, warm=8):
+    """Average device time per background launch for one guard variant, no foreground."""
+    cfg = H.Config(0, 1, H.spec(kind, n, guard, level, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(kind, 0, 0, 1, 8, 4, 2), 64, 0)
+    with H.Bench(cfg) as b:
+        b.bg_alone(warm)
+        res = b.bg_alone(commands)
         return res.bg_stream_ms / res.bg_stream_cmds
-    finally:
-        lib.XBenchDestroy(b)
 
 
-def run_preempt(lib, bg_n, level, samples=200):
-    cfg = Config(0, 1, spec(AXPY, bg_n, 1, level, BG_THRESHOLD, BG_BATCH, 1), spec(AXPY, 0, 0, 1, 8, 4, 2), 64, 0)
-    b = lib.XBenchCreate(byref(cfg))
-    assert b
-    try:
-        res = PhaseResult()
-        sus = (c_double * samples)()
-        resume = (c_double * samples)()
-        assert lib.XBenchRunPreempt(b, samples, sus, resume, byref(res)) == 0
-        return list(sus), list(resume), list(res.stats)
-    finally:
-        lib.XBenchDestroy(b)
+def preempt_latency(H, kind, n, level, samples):
+    cfg = H.Config(0, 1, H.spec(kind, n, 1, level, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(kind, 0, 0, 1, 8, 4, 2), 64, 0)
+    with H.Bench(cfg) as b:
+        sus, resume, res = b.preempt(samples)
+        return sus, resume, list(res.stats)
 
 
-def cpu_baseline(seconds_budget=15.0):
-    """CPU restatement of the same workload (oracle port), bounded sample."""
-    try:
-        from oracle import cpu_baseline as cb
-    except Exception as e:  # oracle not built
-        return {"value": None, "unit": "us", "cores": 0, "kind": "port", "sample": f"unavailable: {e}"}
-    return cb.run_config2_sample(seconds_budget, samples=300)
+def preempt_block(H, kind, n, quick):
+    sus2, res2, st2 = preempt_latency(H, kind, n, 2, 60 if quick else 200)
+    sus1, _, _ = preempt_latency(H, kind, n, 1, 30 if quick else 60)
+    return {"level2_suspend_sync_p50": H.pct(sus2, 0.5), "level2_suspend_sync_p99": H.pct(sus2, 0.99),
+            "level2_resume_p50": H.pct(res2, 0.5), "level2_resume_p99": H.pct(res2, 0.99),
+            "level1_suspend_sync_p50": H.pct(sus1, 0.5), "level1_suspend_sync_p99": H.pct(sus1, 0.99),
+            "level2_stats": st2}
+
+
+def contended_run(H, cfg, steps, warmup, bg_warm=8, bg_cmds=40):
+    """fg alone -> bg alone -> contended (warm-up, then exactly `steps` timed steps)."""
+    with H.Bench(cfg) as b:
+        alone, _ = b.fg_alone(steps + warmup)
+        b.bg_alone(bg_warm)
+        res = b.bg_alone(bg_cmds)
+        bg_alone_ms = res.bg_stream_ms / res.bg_stream_cmds
+        if warmup:
+            b.contended(warmup)
+        t0 = time.perf_counter()
+        cont, res = b.contended(steps)
+        wall = time.perf_counter() - t0
+        return {"fg_alone": alone[warmup:], "fg_contended": cont, "wall_s": wall,
+                "bg_alone_ms": bg_alone_ms,
+                "bg_cont_ms": (res.bg_stream_ms / res.bg_stream_cmds) if res.bg_stream_cmds else None,
+                "bg_cont_cmds": int(res.bg_commands), "bg_cont_elapsed": res.elapsed_s,
+                "deadline_miss": int(res.fg_deadline_miss), "stats": list(res.stats)}
 
 
 def recorded_traffic(bg_n):
     """HBM bytes per launch of the plain 2^28 AXPY kernel as recorded by the two
     rocprofv3 counter runs summarised under profiles/ (counters cannot be read from
     inside this process); None for any other size or when the summary is absent."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
-                        "axpy_2p28_hbm_traffic.md")
+    path = os.path.join(ROOT, "profiles", "axpy_2p28_hbm_traffic.md")
     if bg_n != 1 << 28 or not os.path.exists(path):
         return None
     for ln in open(path):
@@ -168,11 +118,176 @@ def recorded_traffic(bg_n):
     return None
 
 
+def cpu_baseline(seconds_budget=15.0):
+    """The same workload on host cores: XSched's own host loop where its build is present
+    (kind "reference"), else the compact port; bounded sample."""
+    try:
+        from oracle import cpu_baseline as cb
+        return cb.run_config2_sample(seconds_budget, samples=300)
+    except Exception as e:  # checker libraries not built
+        return {"value": None, "unit": "us", "cores": 0, "kind": "port", "sample": f"unavailable: {e}"}
+
+
+def base_line(a, value, wall_s, workload, extra_cfg):
+    cfg = {"workload": workload, "percentile_rule": "sorted[floor(p*n)]"}
+    cfg.update(extra_cfg)
+    return {"metric": "fg_p99_latency_us_under_contention", "value": value, "unit": "us", "n_gpus": 1,
+            "steps": a.steps, "warmup": a.warmup, "ms_per_step": wall_s * 1e3 / a.steps,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "data": "synthetic",
+            "config": cfg}
+
+
+# ---- configurations ------------------------------------------------------------------
+
+def config2(H, a):
+    bg_n, fg_n = 1 << a.bg_log2, 1 << a.fg_log2
+    cfg = H.Config(H.HPF, 1, H.spec(H.AXPY, bg_n, 1, 1, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(H.AXPY, fg_n, 0, 1, 8, 4, 2, period_us=20000), 64, 0)
+    r = contended_run(H, cfg, a.steps, a.warmup)
+    fg = fg_summary(H, r["fg_alone"], r["fg_contended"])
+    per_launch_ms = r["bg_cont_ms"] or r["bg_alone_ms"]
+    achieved = axpy_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
+    line = base_line(a, fg["contended_p99"], r["wall_s"],
+                     "cfg2: L1 HPF, bg AXPY 2^%d back-to-back, fg AXPY 2^%d every 20 ms" % (a.bg_log2, a.fg_log2),
+                     {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
+    line["dtype"] = "f32"
+    line["fg_latency_us"] = fg
+    line["bg"] = {"alone_GBs": axpy_bytes(bg_n) / r["bg_alone_ms"] / 1e6,
+                  "contended_GBs": axpy_bytes(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e9,
+                  "commands_in_timed_region": r["bg_cont_cmds"]}
+    line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(bg_n),
+                        "kernel": "AxpyVec4Kernel", "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
+                        "avg_launch_ms": per_launch_ms}
+    if not a.quick:
+        ms_plain = bg_ms_per_launch(H, H.AXPY, bg_n, 1, 0)
+        ms_guard = bg_ms_per_launch(H, H.AXPY, bg_n, 1, 2)
+        ms_l2 = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 1)
+        line["guard"] = {"plain_GBs": axpy_bytes(bg_n) / ms_plain / 1e6,
+                         "guarded_GBs": axpy_bytes(bg_n) / ms_guard / 1e6,
+                         "level2_GBs": axpy_bytes(bg_n) / ms_l2 / 1e6,
+                         "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
+                         "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
+        line["preempt_us"] = preempt_block(H, H.AXPY, bg_n, False)
+    return line
+
+
+def config3(H, a):
+    bg_n, fg_n = 8192, 1024
+    cfg = H.Config(H.HPF, 1, H.spec(H.GEMM, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(H.GEMM, fg_n, 0, 1, 8, 4, 2, period_us=5000), 64, 0)
+    r = contended_run(H, cfg, a.steps, a.warmup, bg_warm=4, bg_cmds=20)
+    fg = fg_summary(H, r["fg_alone"], r["fg_contended"])
+    per_launch_ms = r["bg_alone_ms"]
+    achieved = gemm_flops(bg_n) / (per_launch_ms * 1e-3) / 1e12
+    line = base_line(a, fg["contended_p99"], r["wall_s"],
+                     "cfg3: L2 HPF, bg bf16 GEMM 8192^3 guarded back-to-back, fg GEMM 1024^3 every 5 ms",
+                     {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
+    line["dtype"] = "bf16"
+    line["fg_latency_us"] = fg
+    line["bg"] = {"alone_TFLOPs": achieved,
+                  "contended_TFLOPs": gemm_flops(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e12,
+                  "commands_in_timed_region": r["bg_cont_cmds"], "level2_stats": r["stats"]}
+    line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
+                        "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": None, "kernel": "GemmBf16Kernel",
+                        "algorithmic_flops_per_launch": gemm_flops(bg_n), "avg_launch_ms": per_launch_ms}
+    if not a.quick:
+        ms_plain = bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 20, 4)
+        ms_guard = bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 20, 4)
+        ms_l2 = bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 20, 4)
+
+        def tf(ms):
+            return gemm_flops(bg_n) / ms / 1e9
+        line["guard"] = {"plain_TFLOPs": tf(ms_plain), "guarded_TFLOPs": tf(ms_guard), "level2_TFLOPs": tf(ms_l2),
+                         "plain_mfma_util": tf(ms_plain) / MFMA_BF16_PEAK_TF,
+                         "guarded_mfma_util": tf(ms_guard) / MFMA_BF16_PEAK_TF,
+                         "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
+                         "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
+        line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, False)
+    return line
+
+
+def config4(H, a):
+    bg_n, fg_n, deadline = 1 << 26, 1 << 20, 1000
+    laxities = [300] if a.quick else [0, 300, 600, 900]
+    runs = {}
+    for lax in laxities:
+        # Background queues run at constant priority 0. The foreground runs beside them at
+        # priority 0 until `lax` us after it became ready, then at priority 1, which
+        # deactivates the four background queues.
+        cfg = H.Config(H.LAX, 4, H.spec(H.HIST, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 0),
+                       H.spec(H.HIST, fg_n, 0, 1, 8, 4, 1, laxity_us=lax, period_us=2000, lax_priority=0,
+                              deadline_us=deadline), 16, 0)
+        runs[lax] = contended_run(H, cfg, a.steps, a.warmup, bg_warm=2, bg_cmds=6)
+    head = runs[300]
+    fg = fg_summary(H, head["fg_alone"], head["fg_contended"])
+    per_launch_ms = head["bg_alone_ms"]
+    achieved = hist_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
+    line = base_line(a, fg["contended_p99"], head["wall_s"],
+                     "cfg4: L2 LAX, 4 bg XQueues histogram 2^26 Zipf(1.1) keys, fg 2^20 keys every 2 ms, "
+                     "deadline 1 ms, laxity hint 300 us",
+                     {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
+    line["dtype"] = "u32"
+    line["fg_latency_us"] = fg
+    line["deadline_miss_rate"] = head["deadline_miss"] / a.steps
+    line["by_laxity_us"] = {
+        str(lax): {"deadline_miss_rate": r["deadline_miss"] / a.steps,
+                   "fg_p50": H.pct(r["fg_contended"], 0.5), "fg_p99": H.pct(r["fg_contended"], 0.99),
+                   "bg_GBs": hist_bytes(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e9,
+                   "bg_deactivations_q0": r["stats"][2]}
+        for lax, r in runs.items()}
+    line["bg"] = {"alone_GBs_4_queues": 4 * achieved,
+                  "contended_GBs": hist_bytes(bg_n) * head["bg_cont_cmds"] / head["bg_cont_elapsed"] / 1e9}
+    line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "HistogramKernel",
+                        "algorithmic_bytes_per_launch": hist_bytes(bg_n), "avg_launch_ms": per_launch_ms,
+                        "note": "per launch while the 4 queues run side by side"}
+    if not a.quick:
+        line["preempt_us"] = preempt_block(H, H.HIST, bg_n, True)
+    return line
+
+
+def config5(H, a):
+    axpy_n, gemm_n, hist_n, nq = 1 << 24, 2048, 1 << 24, 16
+    duration = a.steps / 100.0  # default 150 steps -> 1.5 s of arrivals, ~300 commands per queue
+    cfg = H.StressConfig(H.HPF, nq, 2, 1, 4, 2, axpy_n, gemm_n, hist_n, 5000.0, 7)
+    with H.Bench(cfg) as b:
+        b.stress(0.2)  # warm-up
+        t0 = time.perf_counter()
+        lat, res = b.stress(duration)
+        wall = time.perf_counter() - t0
+        stats = list(res.stats)
+    counts = [len(x) for x in lat]
+    kinds = ["axpy", "gemm", "hist"]
+    by_prio = {str(i): {"kernel": kinds[i % 3], "commands": counts[i], "p50": H.pct(lat[i], 0.5),
+                        "p99": H.pct(lat[i], 0.99)} for i in range(nq)}
+    hbm_bytes = sum(counts[i] * (axpy_bytes(axpy_n) if i % 3 == 0 else hist_bytes(hist_n) if i % 3 == 2 else 0)
+                    for i in range(nq))
+    flops = sum(counts[i] * gemm_flops(gemm_n) for i in range(nq) if i % 3 == 1)
+    line = base_line(a, H.pct(lat[nq - 1], 0.99), wall,
+                     "cfg5: 16 XQueues prio 0-15, AXPY 2^24 / GEMM 2048^3 / histogram 2^24 by queue index mod 3, "
+                     "exponential arrivals mean 5 ms seed 7, HPF, L2; value = p99 of priority 15",
+                     {"threshold": 4, "batch": 2, "arrival_seconds": duration})
+    line["dtype"] = "mixed f32/bf16/u32"
+    line["per_priority_latency_us"] = by_prio
+    line["aggregate"] = {"commands": sum(counts), "elapsed_s": res.elapsed_s,
+                         "hbm_GBs": hbm_bytes / res.elapsed_s / 1e9,
+                         "hbm_frac_of_peak": hbm_bytes / res.elapsed_s / 1e9 / HBM_PEAK_GBS,
+                         "mfma_TFLOPs": flops / res.elapsed_s / 1e12,
+                         "mfma_frac_of_peak": flops / res.elapsed_s / 1e12 / MFMA_BF16_PEAK_TF,
+                         "queue0_stats": stats}
+    line["roofline"] = {"bound": "hbm", "achieved": hbm_bytes / res.elapsed_s / 1e9, "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": hbm_bytes / res.elapsed_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "note": "aggregate of an arrival-limited workload (offered load, not a kernel rate)"}
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=150)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--bg-log2", type=int, default=28)
     ap.add_argument("--fg-log2", type=int, default=22)
     ap.add_argument("--skip-cpu", action="store_true")
@@ -187,67 +302,14 @@ def main():
     if not torch.cuda.is_available():
         print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)
         sys.exit(1)
-    import xsched_amd
-    lib = bind_harness(xsched_amd.halhip())
+    from xsched_amd import harness as H
 
-    bg_n, fg_n = 1 << a.bg_log2, 1 << a.fg_log2
-    r = run_config2(lib, a.steps, a.warmup, bg_n, fg_n)
-    p50a, p99a = pct(r["fg_alone"], 0.50), pct(r["fg_alone"], 0.99)
-    p50c, p99c = pct(r["fg_contended"], 0.50), pct(r["fg_contended"], 0.99)
-    per_launch_ms = r["bg_cont_ms"] or r["bg_alone_ms"]
-    achieved = axpy_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
-    bg_kept = axpy_bytes(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e9
-
-    extra = {}
-    if not a.quick:
-        ms_plain = run_bg_variant(lib, bg_n, 1, 0)
-        ms_guard = run_bg_variant(lib, bg_n, 1, 2)
-        ms_l2 = run_bg_variant(lib, bg_n, 2, 1)
-        extra["guard"] = {
-            "plain_GBs": axpy_bytes(bg_n) / ms_plain / 1e6,
-            "guarded_GBs": axpy_bytes(bg_n) / ms_guard / 1e6,
-            "level2_GBs": axpy_bytes(bg_n) / ms_l2 / 1e6,
-            "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
-            "level2_overhead_frac": 1.0 - ms_plain / ms_l2,
-        }
-        sus2, res2, st2 = run_preempt(lib, bg_n, 2)
-        sus1, res1, _ = run_preempt(lib, bg_n, 1, samples=60)
-        extra["preempt_us"] = {
-            "level2_suspend_sync_p50": pct(sus2, 0.5), "level2_suspend_sync_p99": pct(sus2, 0.99),
-            "level2_resume_p50": pct(res2, 0.5), "level2_resume_p99": pct(res2, 0.99),
-            "level1_suspend_sync_p50": pct(sus1, 0.5), "level1_suspend_sync_p99": pct(sus1, 0.99),
-            "level2_stats": st2,
-        }
-
-    line = {
-        "metric": "fg_p99_latency_us_under_contention",
-        "value": p99c,
-        "unit": "us",
-        "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
-        "ms_per_step": r["wall_s"] * 1e3 / a.steps,
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "cfg2: L1 HPF, bg AXPY 2^%d back-to-back, fg AXPY 2^%d every 20 ms"
-                               % (a.bg_log2, a.fg_log2),
-                   "bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4,
-                   "percentile_rule": "sorted[floor(p*n)]"},
-        "fg_latency_us": {"alone_p50": p50a, "alone_p99": p99a, "contended_p50": p50c,
-                          "contended_p99": p99c, "p99_ratio": p99c / p99a if p99a else None},
-        "bg": {"alone_GBs": axpy_bytes(bg_n) / r["bg_alone_ms"] / 1e6, "contended_GBs": bg_kept,
-               "commands_in_timed_region": r["bg_cont_cmds"]},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(bg_n),
-                     "kernel": "AxpyVec4Kernel", "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
-                     "avg_launch_ms": per_launch_ms},
-    }
-    line.update(extra)
-    line["cpu_baseline"] = ({"value": None, "unit": "us", "cores": 0, "kind": "port", "sample": "skipped"}
-                            if a.skip_cpu else cpu_baseline())
+    line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
+    if a.config == 2 and not a.skip_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    else:
+        line["cpu_baseline"] = {"value": None, "unit": "us", "cores": 0, "kind": "port",
+                                "sample": "skipped" if a.config == 2 else "measured for the headline workload only"}
     print(json.dumps(line))
 
 

@@ -28,8 +28,14 @@ typedef struct {
     int32_t  threshold;   /* in-flight window                                           */
     int32_t  batch;       /* marker period                                              */
     int32_t  priority;    /* XHintPriority (HPF) / critical priority (LAX)              */
-    int64_t  laxity_us;   /* >= 0: XHintLaxity(laxity, lax_prio = PRIORITY_MIN, priority) */
+    int64_t  laxity_us;   /* >= 0: XHintLaxity(laxity, lax_priority, priority) under the
+                             laxity policy: the queue runs at lax_priority until laxity_us
+                             after it became ready, then at `priority`                  */
     int64_t  period_us;   /* foreground: one command every period; background: ignored  */
+    int32_t  lax_priority;/* see laxity_us                                              */
+    int32_t  reserved;
+    int64_t  deadline_us; /* > 0: a foreground command that completes later than this
+                             after its submission counts as a deadline miss             */
 } XBenchQueueSpec;
 
 typedef struct {
@@ -49,7 +55,7 @@ typedef struct {
     uint64_t bg_stream_cmds;   /* commands of bg queue 0 inside bg_stream_ms             */
     uint64_t fg_samples;       /* foreground latencies written                           */
     uint64_t fg_deadline_miss; /* foreground commands that completed later than
-                                  ready time + fg.laxity_us (0 when no laxity)           */
+                                  submission + fg.deadline_us (0 when no deadline)       */
     uint64_t stats[8];         /* HipQueueGetStats of bg queue 0 at the end              */
 } XBenchPhaseResult;
 
@@ -75,6 +81,37 @@ XResult XBenchRunContended(XBench *b, int samples, double *latency_us, XBenchPha
  * XQueueResume, each timed on the host (microseconds). */
 XResult XBenchRunPreempt(XBench *b, int samples, double *suspend_us, double *resume_us,
                          XBenchPhaseResult *res);
+
+/* ---- mixed stress: many XQueues, one priority each, random arrivals ------------- */
+
+typedef struct {
+    int32_t  policy;        /* XPolicyType of the local scheduler                        */
+    int32_t  n_queues;      /* <= 64; queue i has priority i and runs kernel i % 3:
+                               0 AXPY over axpy_n elements, 1 GEMM gemm_n^3, 2 histogram
+                               of hist_n keys                                            */
+    int32_t  level;         /* XPreemptLevel of every queue                              */
+    int32_t  guard;         /* guard mode of every command                               */
+    int32_t  threshold;
+    int32_t  batch;
+    uint64_t axpy_n, gemm_n, hist_n;
+    double   mean_interarrival_us; /* per queue, exponential                             */
+    uint64_t seed;          /* arrivals: interval k of queue i = -mean * ln(1 - u),
+                               u = top 53 bits of synthetic stream (seed, 1000 + i)
+                               at index k, as a fraction of 2^53                         */
+} XBenchStressConfig;
+
+/* Creates the queues and their seeded inputs; queue i is "background queue i" for
+ * XBenchReadOutput. */
+XBench *XBenchCreateStress(const XBenchStressConfig *cfg);
+
+/* Runs the arrival processes for `duration_s` seconds of arrivals, one thread per
+ * queue: wait for the arrival time, submit one command, wait for it. The latency of a
+ * command is completion minus ARRIVAL time (so it includes the time the queue was
+ * behind). latency_us holds n_queues rows of `cap` values; counts[i] receives how many
+ * were written for queue i (commands beyond `cap` are still executed and counted in
+ * `applied`). */
+XResult XBenchRunStress(XBench *b, double duration_s, double *latency_us, uint64_t cap,
+                        uint64_t *counts, XBenchPhaseResult *res);
 
 /* Copy `count` elements starting at `first` of a result buffer to the host:
  * which = 0: background queue `q` output (axpy y / gemm C / hist bins),

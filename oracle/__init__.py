@@ -31,6 +31,8 @@ def lib():
         L.oracle_f32_to_bf16.restype = c_uint16
         L.oracle_stream_key.argtypes = [c_uint64, c_uint64]
         L.oracle_stream_key.restype = c_uint64
+        L.oracle_bits.argtypes = [c_uint64, c_uint64]
+        L.oracle_bits.restype = c_uint64
         L.oracle_fill_uniform.argtypes = [c_void_p, c_uint64, c_uint64, c_uint64]
         L.oracle_fill_normal_bf16.argtypes = [c_void_p, c_uint64, c_uint64, c_uint64]
         L.oracle_zipf_table.argtypes = [c_void_p, c_uint32, c_double]
@@ -92,6 +94,11 @@ def f32_to_bf16_bits(x):
 
 def stream_key(seed, stream):
     return lib().oracle_stream_key(seed, stream)
+
+
+def bits(key, i):
+    """Raw 64 bits of the stream with key `key` at index i."""
+    return lib().oracle_bits(key, i)
 
 
 def fill_uniform(seed, stream, first, count):

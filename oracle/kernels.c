@@ -125,6 +125,9 @@ uint64_t oracle_stream_key(uint64_t seed, uint64_t stream)
     return splitmix64(seed ^ (stream * 0xD1B54A32D192ED03ull));
 }
 
+/* raw 64 bits of a stream at index i */
+uint64_t oracle_bits(uint64_t key, uint64_t i) { return splitmix64(key + i); }
+
 /* uniform in [-1, 1): top 24 bits u -> u * 2^-23 - 1 */
 void oracle_fill_uniform(float *dst, uint64_t first, uint64_t count, uint64_t key)
 {

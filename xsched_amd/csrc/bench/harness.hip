@@ -109,6 +109,7 @@ struct Lane
 struct XBench
 {
     XBenchConfig cfg {};
+    XBenchStressConfig stress {};
     std::vector<std::unique_ptr<Lane>> bg;
     std::unique_ptr<Lane> fg;
     uint32_t *zipf_table_dev = nullptr;
@@ -162,7 +163,7 @@ void SetupLane(XBench &b, Lane &lane, const XBenchQueueSpec &spec, uint64_t seed
     BENCH_X(XQueueCreate(&lane.xq, lane.hwq, spec.level, kQueueCreateFlagNone));
     BENCH_X(XQueueSetLaunchConfig(lane.xq, spec.threshold, spec.batch));
     if (b.cfg.policy == kPolicyLaxity && spec.laxity_us >= 0) {
-        BENCH_X(XHintLaxity(lane.xq, spec.laxity_us, PRIORITY_MIN, spec.priority));
+        BENCH_X(XHintLaxity(lane.xq, spec.laxity_us, spec.lax_priority, spec.priority));
     } else if (b.cfg.policy == kPolicyLaxity) {
         // No laxity: a constant priority (lax == crit).
         BENCH_X(XHintLaxity(lane.xq, 0, spec.priority, spec.priority));
@@ -242,7 +243,7 @@ double ForegroundOnce(Lane &fg, bool *missed)
     fg.Submit();
     BENCH_X(XQueueWaitAll(fg.xq));
     const double us = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
-    if (missed) *missed = fg.spec.laxity_us >= 0 && us > (double)fg.spec.laxity_us;
+    if (missed) *missed = fg.spec.deadline_us > 0 && us > (double)fg.spec.deadline_us;
     return us;
 }
 
@@ -435,6 +436,75 @@ EXPORT_C_FUNC XResult XBenchRunPreempt(XBench *b, int samples, double *suspend_u
         *res = XBenchPhaseResult {};
         res->elapsed_s = std::chrono::duration<double>(Clock::now() - t_begin).count();
         res->bg_commands = q0.applied.load();
+        FillStats(b, res);
+    }
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XBench *XBenchCreateStress(const XBenchStressConfig *cfg)
+{
+    if (cfg == nullptr || cfg->n_queues <= 0 || cfg->n_queues > 64 || cfg->mean_interarrival_us <= 0) return nullptr;
+    auto *b = new XBench();
+    b->stress = *cfg;
+    b->cfg.policy = cfg->policy;
+    b->cfg.seed = cfg->seed;
+    if (cfg->policy != kPolicyUnknown) BENCH_X(XHintSetScheduler(kSchedulerLocal, (XPolicyType)cfg->policy));
+    else BENCH_X(XHintSetScheduler(kSchedulerAppManaged, kPolicyUnknown));
+    for (int i = 0; i < cfg->n_queues; ++i) {
+        XBenchQueueSpec spec {};
+        spec.kind = i % 3;
+        spec.guard = cfg->guard;
+        spec.n = spec.kind == kXBenchAxpy ? cfg->axpy_n : spec.kind == kXBenchGemm ? cfg->gemm_n : cfg->hist_n;
+        spec.level = cfg->level;
+        spec.threshold = cfg->threshold;
+        spec.batch = cfg->batch;
+        spec.priority = i;
+        spec.laxity_us = -1;
+        b->bg.emplace_back(std::make_unique<Lane>());
+        SetupLane(*b, *b->bg.back(), spec, cfg->seed, (uint64_t)i + 1);
+    }
+    return b;
+}
+
+EXPORT_C_FUNC XResult XBenchRunStress(XBench *b, double duration_s, double *latency_us, uint64_t cap,
+                                      uint64_t *counts, XBenchPhaseResult *res)
+{
+    if (b == nullptr || b->stress.n_queues <= 0 || (size_t)b->stress.n_queues != b->bg.size() ||
+        duration_s <= 0 || latency_us == nullptr || counts == nullptr || cap == 0) {
+        return kXSchedErrorInvalidValue;
+    }
+    const int nq = b->stress.n_queues;
+    const double mean = b->stress.mean_interarrival_us;
+    uint64_t applied_before = 0;
+    for (auto &lane : b->bg) applied_before += lane->applied.load();
+    const auto t_begin = Clock::now() + std::chrono::milliseconds(5);
+    std::vector<std::thread> threads;
+    for (int i = 0; i < nq; ++i) {
+        counts[i] = 0;
+        threads.emplace_back([&, i]() {
+            Lane &lane = *b->bg[i];
+            const uint64_t key = synth_stream_key(b->stress.seed, 1000 + (uint64_t)i);
+            double t_us = 0; // arrival time since t_begin
+            for (uint64_t k = 0;; ++k) {
+                const double u = (double)(synth_bits(key, k) >> 11) * (1.0 / 9007199254740992.0);
+                t_us += -mean * std::log1p(-u);
+                if (t_us > duration_s * 1e6) break;
+                const auto arrival = t_begin + std::chrono::nanoseconds((int64_t)(t_us * 1e3));
+                SleepUntil(arrival);
+                lane.Submit();
+                BENCH_X(XQueueWaitAll(lane.xq));
+                const double us = std::chrono::duration<double, std::micro>(Clock::now() - arrival).count();
+                if (counts[i] < cap) latency_us[(uint64_t)i * cap + counts[i]++] = us;
+            }
+        });
+    }
+    for (auto &t : threads) t.join();
+    if (res) {
+        *res = XBenchPhaseResult {};
+        res->elapsed_s = std::chrono::duration<double>(Clock::now() - t_begin).count();
+        uint64_t applied_after = 0;
+        for (auto &lane : b->bg) applied_after += lane->applied.load();
+        res->bg_commands = applied_after - applied_before;
         FillStats(b, res);
     }
     return kXSchedSuccess;
