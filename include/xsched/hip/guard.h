@@ -154,6 +154,15 @@ public:
         return *lds_ != 0;
     }
 
+    /// Barrier-free variant of the re-check for the calling wave alone (the result is
+    /// wave-uniform). The kernel has to make the waves of the group agree before any of
+    /// them produces a side effect, e.g. through an LDS word and the barrier it already
+    /// has in front of its write-out.
+    __device__ __forceinline__ bool WaveStillCurrent() const
+    {
+        return xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+    }
+
     /// Call after the last store of the work-group (all waves; one barrier inside).
     __device__ __forceinline__ void Commit() const
     {

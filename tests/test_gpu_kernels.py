@@ -124,6 +124,56 @@ def test_histogram_bit_exact(xs, gpu, n, n_bins, level, guard):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("n_bins,offset", [(65536, 0), (65536, 1), (1001, 0), (40000, 1)])
+def test_histogram_counters_wrap_independently(xs, gpu, n_bins, offset):
+    """Bins that start just below 2^32 wrap on their own, as uint32 counters do in the
+    oracle: the write-out adds two neighbouring counters with one 64-bit atomic and must
+    take back a carry that leaks from the lower into the upper one. Also with a bins array
+    that is only 4-byte aligned (offset 1), where the write-out uses 32-bit atomics."""
+    torch = gpu
+    n = (1 << 20) + 13
+    print(f"case hist-wrap bins={n_bins} offset={offset}", flush=True)
+    table = oracle.zipf_table(n_bins)
+    keys_h = oracle.fill_zipf(3, 1, 0, n, table, n_bins)
+    keys = torch.from_numpy(keys_h).cuda()
+    rnd = np.random.default_rng(5)
+    start = (0xFFFFFFFF - rnd.integers(0, 3, n_bins)).astype(np.uint32)   # 0..2 below wrapping
+    start[rnd.random(n_bins) < 0.3] = 0
+    store = torch.zeros(n_bins + 2, dtype=torch.int32, device="cuda")
+    bins = store[offset:offset + n_bins]
+    bins.copy_(torch.from_numpy(start.view(np.int32)))
+    q = Queue(xs, torch, 2)
+    q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+    q.wait()
+    got = bins.cpu().numpy().view(np.uint32)
+    guard_words = store.cpu().numpy()
+    q.close()
+    want = oracle.histogram(keys_h, n_bins, start)
+    assert np.array_equal(got, want)
+    assert guard_words[offset + n_bins:].tolist() == [0] * (2 - offset), "wrote beyond the bins array"
+    if offset:
+        assert guard_words[0] == 0
+
+
+@pytest.mark.parametrize("lo,hi", [(32768, 65536), (0, 65536), (100, 101), (40000, 40003)])
+def test_histogram_any_distribution(xs, gpu, lo, hi):
+    """Distributions the kernel is not tuned for: every key in the upper half of the key
+    space (the on-chip list of such keys overflows and the work-group re-reads its chunk),
+    uniform keys, one single bin, three neighbouring bins."""
+    torch = gpu
+    n = (1 << 22) + 5
+    print(f"case hist-dist [{lo},{hi})", flush=True)
+    keys_h = np.random.default_rng(lo).integers(lo, hi, n).astype(np.int32)
+    keys = torch.from_numpy(keys_h).cuda()
+    bins = torch.zeros(65536, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, 2)
+    q.submit(hist_cmd(xs, keys, n, bins, 65536, 1))
+    q.wait()
+    got = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    assert np.array_equal(got, oracle.histogram(keys_h, 65536))
+
+
 def _gemm_case(xs, torch, a_bits, b_bits, M, N, K, level, guard):
     a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
     b = torch.from_numpy(b_bits.view(np.int16).reshape(K, N)).cuda()
