@@ -41,10 +41,16 @@ namespace hist
 
 constexpr uint32_t kThreads = 1024;
 constexpr uint32_t kWaves = kThreads / 64;
-constexpr uint32_t kHotBins = 4;
+#ifndef XSCHED_HIST_HOT_BINS
+#define XSCHED_HIST_HOT_BINS 2
+#endif
+constexpr uint32_t kHotBins = XSCHED_HIST_HOT_BINS;
 constexpr uint32_t kLdsBins = 1u << 15;       // 128 KiB of counters
 constexpr uint32_t kTailCap = 14336;          // 16-bit entries, 28 KiB
-constexpr uint32_t kUnits = 4;                // 128-bit loads per thread and iteration
+#ifndef XSCHED_HIST_UNITS
+#define XSCHED_HIST_UNITS 4
+#endif
+constexpr uint32_t kUnits = XSCHED_HIST_UNITS;  // 128-bit loads per thread and iteration
 constexpr uint32_t kUnitKeys = kThreads * 4;
 constexpr uint32_t kIterKeys = kUnitKeys * kUnits;
 constexpr uint32_t kMinChunk = kUnitKeys;
@@ -88,25 +94,18 @@ __device__ __forceinline__ void GlobalAdd(uint32_t *p, uint32_t v)
 /// dst[0] += lo, dst[1] += hi with ONE 64-bit atomic (dst is 8-byte aligned): the
 /// write-out is bound by the number of atomic operations, and this halves it. The two
 /// counters stay independent 32-bit values: should the low one wrap, the returned old
-/// value shows it and the carry that leaked into the high one is taken back.
-__device__ __forceinline__ void PairAdd(uint32_t *dst, uint32_t lo, uint32_t hi)
+/// value shows it and the carry that leaked into the high one is taken back (PairFix).
+/// Issue and check are separate calls so that a sweep has all its atomics in flight
+/// before it looks at the first returned value.
+__device__ __forceinline__ uint32_t PairAdd(uint32_t *dst, uint32_t lo, uint32_t hi)
 {
-    if ((lo | hi) == 0) return;
-    const unsigned long long old = __hip_atomic_fetch_add((unsigned long long *)dst,
-        ((unsigned long long)hi << 32) | lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((uint32_t)((uint32_t)old + lo) < lo) GlobalAdd(dst + 1, 0xFFFFFFFFu);
+    return (uint32_t)__hip_atomic_fetch_add((unsigned long long *)dst, ((unsigned long long)hi << 32) | lo,
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-/// dst[i] += lo, dst[i + 1] += hi, never touching memory at or beyond dst + count.
-__device__ __forceinline__ void AddTwo(uint32_t *dst, uint32_t i, uint32_t lo, uint32_t hi, uint32_t count,
-                                       bool pair_ok)
+__device__ __forceinline__ void PairFix(uint32_t *dst, uint32_t old_lo, uint32_t lo)
 {
-    if (pair_ok && i + 1 < count) {
-        PairAdd(dst + i, lo, hi);
-    } else {
-        if (lo != 0 && i < count) GlobalAdd(dst + i, lo);
-        if (hi != 0 && i + 1 < count) GlobalAdd(dst + i + 1, hi);
-    }
+    if ((uint32_t)(old_lo + lo) < lo) GlobalAdd(dst + 1, 0xFFFFFFFFu);
 }
 
 /// acc += popcount(mask), issued where it is written. Left to the compiler, the
@@ -118,21 +117,44 @@ __device__ __forceinline__ void AddPopcount(uint32_t &acc, uint64_t mask)
     asm volatile("s_bcnt1_i32_b64 %1, %2\n\ts_add_u32 %0, %0, %1" : "+s"(acc), "=&s"(tmp) : "s"(mask) : "scc");
 }
 
-/// Adds the non-zero counters of sh.bins[0, count) to dst[0, count). Wave q of the group
-/// sweeps segments rot + q, rot + q + 16, ... (mod kSegs), so groups that write out at
-/// the same time start on different cache lines.
+/// Adds the non-zero counters of sh.bins[0, count) to dst[0, count), never touching
+/// memory at or beyond dst + count. Wave q of the group sweeps segments rot + q,
+/// rot + q + 16, ... (mod kSegs), so groups that write out at the same time start on
+/// different cache lines.
 __device__ __forceinline__ void SweepOut(Shared &sh, uint32_t *dst, uint32_t count, uint32_t rot)
 {
+    constexpr uint32_t kSteps = kSegs / kWaves;
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool pair_ok = (((uintptr_t)dst) & 7) == 0; // segment starts are even indices
-    for (uint32_t step = 0; step < kSegs / kWaves; ++step) {
+    uint32_t low[kSteps][2], old[kSteps][2];
+#pragma unroll
+    for (uint32_t step = 0; step < kSteps; ++step) {
         const uint32_t seg = (rot + step * kWaves + wave) & (kSegs - 1);
         const uint32_t b4 = seg * kSegBins + lane * 4;
-        if (b4 >= count) continue;
-        const u32x4 c = *(const u32x4 *)&sh.bins[b4];
         // counters at or beyond `count` are never incremented, so they read zero
-        AddTwo(dst, b4 + 0, c.x, c.y, count, pair_ok);
-        AddTwo(dst, b4 + 2, c.z, c.w, count, pair_ok);
+        const u32x4 c = b4 < count ? *(const u32x4 *)&sh.bins[b4] : u32x4 { 0, 0, 0, 0 };
+        const uint32_t v[4] = { c.x, c.y, c.z, c.w };
+#pragma unroll
+        for (uint32_t p = 0; p < 2; ++p) {
+            const uint32_t i = b4 + p * 2, lo = v[p * 2], hi = v[p * 2 + 1];
+            low[step][p] = 0;
+            old[step][p] = 0;
+            if ((lo | hi) == 0) continue;
+            if (pair_ok && i + 1 < count) {
+                low[step][p] = lo;
+                old[step][p] = PairAdd(dst + i, lo, hi);
+            } else {
+                if (lo != 0 && i < count) GlobalAdd(dst + i, lo);
+                if (hi != 0 && i + 1 < count) GlobalAdd(dst + i + 1, hi);
+            }
+        }
+    }
+#pragma unroll
+    for (uint32_t step = 0; step < kSteps; ++step) {
+        const uint32_t seg = (rot + step * kWaves + wave) & (kSegs - 1);
+        const uint32_t b4 = seg * kSegBins + lane * 4;
+#pragma unroll
+        for (uint32_t p = 0; p < 2; ++p) PairFix(dst + b4 + p * 2, old[step][p], low[step][p]);
     }
 }
 
@@ -174,6 +196,27 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 #pragma unroll
     for (uint32_t b = 0; b < kHotBins; ++b) hot[b] = 0;
 
+    // Lists the tail keys among k[0, count) one key vector at a time: one reservation for
+    // the wave, each key placed by its rank among the wave's tail lanes of that vector.
+    // Used when some thread holds more than four tail keys in one iteration.
+    auto list_tail_per_key = [&](const uint32_t *k, uint32_t count) {
+        uint32_t total = 0;
+        for (uint32_t j = 0; j < count; ++j) AddPopcount(total, __ballot(k[j] - kLdsBins < tail_range));
+        uint32_t slot = 0;
+        if (lane == 0) slot = __hip_atomic_fetch_add(&sh.tail_count, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        slot = __builtin_amdgcn_readfirstlane(slot);
+        for (uint32_t j = 0; j < count; ++j) {
+            const bool is_tail = k[j] - kLdsBins < tail_range;
+            const uint64_t m = __ballot(is_tail);
+            if (is_tail) {
+                const uint32_t at = slot + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                           __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                if (at < kTailCap) sh.tail[at] = (uint16_t)k[j];
+            }
+            AddPopcount(slot, m);
+        }
+    };
+
     // Counts kUnitsNow * 4 keys per thread.
     auto process = [&](const i32x4 *v, auto units_tag) {
         constexpr uint32_t kN = decltype(units_tag)::value * 4;
@@ -190,25 +233,46 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j]], 1u);
         }
         if (tail_range != 0) {
-            uint32_t total = 0;
+            // Tail keys are rare for skewed inputs, and VALU issue is what bounds this loop:
+            // each thread first gathers its own tail keys (up to four 16-bit values in two
+            // registers, newest in the low half of `lo`), then the wave places them with at
+            // most four list writes per iteration instead of one per key.
+            uint32_t cnt = 0, lo = 0, hi = 0;
 #pragma unroll
             for (uint32_t j = 0; j < kN; ++j) {
-                AddPopcount(total, __ballot(k[j] - kLdsBins < tail_range));
+                if (k[j] - kLdsBins < tail_range) {
+                    // asm so that the body stays under the branch (three instructions that
+                    // run only for key vectors with a tail lane) instead of becoming selects
+                    asm volatile("v_alignbit_b32 %0, %0, %1, 16\n\t"
+                                 "v_lshl_or_b32 %1, %1, 16, %3\n\t"
+                                 "v_add_u32 %2, 1, %2"
+                                 : "+v"(hi), "+v"(lo), "+v"(cnt) : "v"(k[j]));
+                }
             }
-            if (total != 0) {
-                uint32_t slot = 0;
-                if (lane == 0) slot = __hip_atomic_fetch_add(&sh.tail_count, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                slot = __builtin_amdgcn_readfirstlane(slot);
-#pragma unroll
-                for (uint32_t j = 0; j < kN; ++j) {
-                    const bool is_tail = k[j] - kLdsBins < tail_range;
-                    const uint64_t m = __ballot(is_tail);
-                    if (is_tail) {
-                        const uint32_t at = slot + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
-                                                   __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-                        if (at < kTailCap) sh.tail[at] = (uint16_t)k[j];
+            if (kN > 4 && __ballot(cnt > 4) != 0) {
+                list_tail_per_key(k, kN);
+            } else {
+                const uint64_t l1 = __ballot(cnt >= 1);
+                if (l1 != 0) {
+                    const uint64_t l2 = __ballot(cnt >= 2), l3 = __ballot(cnt >= 3), l4 = __ballot(cnt >= 4);
+                    const uint32_t n1 = (uint32_t)__popcll(l1), n2 = (uint32_t)__popcll(l2);
+                    const uint32_t n3 = (uint32_t)__popcll(l3), n4 = (uint32_t)__popcll(l4);
+                    const uint32_t total = n1 + n2 + n3 + n4;
+                    uint32_t slot = 0;
+                    if (lane == 0) slot = __hip_atomic_fetch_add(&sh.tail_count, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    slot = __builtin_amdgcn_readfirstlane(slot);
+                    if (slot + total <= kTailCap) {
+                        auto rank = [](uint64_t m) {
+                            return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                        };
+                        if (cnt >= 1) sh.tail[slot + rank(l1)] = (uint16_t)lo;
+                        if (cnt >= 2) sh.tail[slot + n1 + rank(l2)] = (uint16_t)(lo >> 16);
+                        if (l3 != 0) {
+                            if (cnt >= 3) sh.tail[slot + n1 + n2 + rank(l3)] = (uint16_t)hi;
+                            if (cnt >= 4) sh.tail[slot + n1 + n2 + n3 + rank(l4)] = (uint16_t)(hi >> 16);
+                        }
                     }
-                    AddPopcount(slot, m);
+                    // else: tail_count has passed the capacity, the write-out re-reads the chunk
                 }
             }
         }
