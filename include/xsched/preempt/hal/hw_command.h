@@ -41,6 +41,10 @@ public:
     /// Process-unique handle.
     virtual HwCommandHandle GetHandle() { return (uint64_t)this ^ ((uint64_t)GetProcessId() << 48); }
 
+    /// Extension, see HwQueue::SupportDirectLaunch(): true when this command may be
+    /// launched on the submitting thread, i.e. its BeforeLaunch() never blocks.
+    virtual bool DirectLaunchable() { return false; }
+
     /// 1-based submission index inside its XQueue; -1 before submission.
     int64_t GetIdx() const { return idx_; }
     void SetIdx(int64_t idx) { idx_ = idx; }

@@ -61,6 +61,15 @@ public:
     /// Called on the submitting thread for each command, before it is buffered.
     virtual void OnHwCommandSubmit(std::shared_ptr<HwCommand> hw_cmd) { UNUSED(hw_cmd); }
 
+    /// Extension (no counterpart in the reference; declared last so that adapters written
+    /// against the reference interface keep their virtual layout and get the default).
+    /// True: Launch() and Synchronize() may be called from ANY thread that holds the
+    /// XQueue's launch lock, not only from the launch thread. The XQueue then launches a
+    /// command on the submitting thread when the launch thread is asleep and nothing is
+    /// queued ahead of it, which takes the wake-up of that thread (tens of microseconds on
+    /// an idle core) out of the submit-to-device path.
+    virtual bool SupportDirectLaunch() { return false; }
+
     std::shared_ptr<XQueue> GetXQueue() { return xq_; }
     void SetXQueue(std::shared_ptr<XQueue> xq) { xq_ = xq; }
 

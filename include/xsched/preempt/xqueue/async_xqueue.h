@@ -12,6 +12,7 @@
 #include <atomic>
 #include <condition_variable>
 #include <deque>
+#include <functional>
 #include <memory>
 #include <mutex>
 #include <thread>
@@ -34,12 +35,22 @@ public:
     std::shared_ptr<XCommand> Dequeue();
     /// Returns a drain marker covering everything enqueued so far (an existing
     /// one when possible; an already completed one when the queue is idle).
-    std::shared_ptr<XQueueWaitAllCommand> EnqueueXQueueWaitAllCommand();
+    /// `consumer_asleep`, when given, tells whether the launch thread was asleep on the
+    /// buffer at that moment (it is woken for the marker either way).
+    std::shared_ptr<XQueueWaitAllCommand> EnqueueXQueueWaitAllCommand(bool *consumer_asleep = nullptr);
     /// Complete and discard everything still buffered.
     void DropAll();
 
     void WaitForNextIdle();
     XQueueState GetXQueueState();
+
+    /// Direct launch (see HwQueue::SupportDirectLaunch): `launch` is tried, with the
+    /// buffer lock held, for a hardware command that arrives while the launch thread
+    /// sleeps on an empty buffer; when it returns true the command has been launched and
+    /// is not queued. The launch thread is still woken, off the submitter's path, to run
+    /// the drain sequence that ends in the Idle event.
+    using DirectLaunch = std::function<bool(const std::shared_ptr<HwCommand> &)>;
+    void SetDirectLaunch(DirectLaunch launch) { direct_launch_ = std::move(launch); }
 
 private:
     const XQueueHandle kXQueueHandle;
@@ -47,6 +58,8 @@ private:
     std::mutex mtx_;
     std::condition_variable cv_;
     bool consumer_waiting_ = false;
+    bool drain_needed_ = false;
+    DirectLaunch direct_launch_;
 
     XQueueState xq_state_ = kQueueStateIdle;
     std::shared_ptr<XCommand> last_enqueued_cmd_;
@@ -77,6 +90,13 @@ public:
     /// `hw_cmd` must be synchronizable and already launched.
     void SyncCmd(std::shared_ptr<HwCommand> hw_cmd);
 
+    /// Launch on the calling thread if that needs no waiting: queue running, window not
+    /// full, no drain point. False: nothing happened, queue the command as usual.
+    bool TryLaunchDirect(const std::shared_ptr<HwCommand> &hw_cmd);
+    /// Index of the last hardware command that has been launched (or dropped).
+    int64_t HandledIdx() const { return handled_idx_.load(std::memory_order_acquire); }
+    int64_t DirectLaunches() const { return direct_launches_.load(std::memory_order_relaxed); }
+
     void SetPreemptLevel(XPreemptLevel level) { level_ = level; }
     void SetLaunchConfig(int64_t threshold, int64_t batch_size)
     { threshold_ = threshold; batch_size_ = batch_size; }
@@ -89,6 +109,10 @@ private:
 
     void Loop();
     void LaunchHwCommand(std::shared_ptr<HwCommand> hw_cmd);
+    /// Drop check, marker rule, Launch(), log. Lock held.
+    void LaunchLocked(const std::shared_ptr<HwCommand> &hw_cmd);
+    bool NeedsDrainBefore(const std::shared_ptr<HwCommand> &hw_cmd, std::shared_ptr<HwCommand> *marker);
+    void RetireUpTo(int64_t idx);
     /// Both return with the lock held. They release it around the blocking
     /// driver wait and start over when a Pause() happened meanwhile.
     void SyncAllLocked(Lock &lock);
@@ -112,6 +136,8 @@ private:
     std::condition_variable cv_;
 
     int64_t drop_idx_ = -1;
+    std::atomic<int64_t> handled_idx_ { 0 };
+    std::atomic<int64_t> direct_launches_ { 0 };
     int64_t pause_count_ = 0;
     WorkerState state_ = kRunning;
     std::unique_ptr<std::thread> thread_;
@@ -131,6 +157,7 @@ public:
     virtual void Wait(std::shared_ptr<HwCommand> hw_cmd) override;
     virtual XQueueState Query() override;
     virtual int64_t GetHwCommandCount() override;
+    virtual int64_t GetDirectLaunchCount() override { return launch_worker_->DirectLaunches(); }
 
     virtual void Suspend(int64_t flags) override;
     virtual void Resume(int64_t flags) override;
@@ -143,6 +170,7 @@ private:
     const std::shared_ptr<CommandBuffer> cmd_buf_;
     const std::shared_ptr<LaunchWorker> launch_worker_;
 
+    bool direct_ = false; // the adapter allows launches and drains on application threads
     std::atomic_bool suspended_ { false };
     std::atomic_bool terminated_ { false };
     std::atomic<int64_t> next_hw_cmd_idx_ { 1 };

@@ -59,6 +59,10 @@ XResult XQueueResume(XQueueHandle xq, int64_t flags);
 /* Number of commands submitted over the queue's lifetime. reference xqueue.h:84 */
 XResult XQueueProfileHwCommandCount(XQueueHandle xq, int64_t *count);
 
+/* How many of them were launched on the submitting thread instead of the launch
+ * thread (see HwQueue::SupportDirectLaunch). No counterpart in the reference. */
+XResult XQueueProfileDirectLaunchCount(XQueueHandle xq, int64_t *count);
+
 /* Unregister a hardware queue; refused (NotAllowed) while an XQueue is attached.
  * reference xqueue.h:90, hw_queue.cpp:30-49 */
 XResult HwQueueDestroy(HwQueueHandle hwq);

@@ -67,6 +67,7 @@ PREEMPT_API = {
     "XQueueSuspend": (XResult, [c_uint64, c_int64]),
     "XQueueResume": (XResult, [c_uint64, c_int64]),
     "XQueueProfileHwCommandCount": (XResult, [c_uint64, POINTER(c_int64)]),
+    "XQueueProfileDirectLaunchCount": (XResult, [c_uint64, POINTER(c_int64)]),
     "HwQueueDestroy": (XResult, [c_uint64]),
     "HwQueueLaunch": (XResult, [c_uint64, c_uint64]),
     "HwQueueSynchronize": (XResult, [c_uint64]),

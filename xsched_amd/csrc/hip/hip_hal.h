@@ -111,6 +111,10 @@ public:
     /// Whether Reactivate() must enqueue this command again.
     virtual bool ReplayOnReactivate() const { return false; }
 
+    /// Every command of this adapter except the host-side event wait only enqueues on
+    /// the stream, so it may be launched on the submitting thread.
+    virtual bool DirectLaunchable() override { return true; }
+
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) = 0;
     hipEvent_t marker_ = nullptr;
@@ -162,6 +166,9 @@ public:
     virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
     virtual void OnPreemptLevelChange(XPreemptLevel level) override;
     virtual void OnXQueueCreate() override;
+    /// Launch() and Synchronize() only issue stream calls under the caller's lock; the
+    /// calling thread's current device is switched for the call and put back.
+    virtual bool SupportDirectLaunch() override { return true; }
 
     hipStream_t Stream() const { return stream_; }
     XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }

@@ -307,16 +307,56 @@ void HipQueue::OnPreemptLevelChange(XPreemptLevel level)
     level_.store(level, std::memory_order_release);
 }
 
+namespace
+{
+
+/// Makes `device` current for the calling thread and restores what was current before.
+/// The launch thread always has it current (OnXQueueCreate); an application thread that
+/// launches directly may not.
+class DeviceScope
+{
+public:
+    explicit DeviceScope(int device)
+    {
+        int cur = device;
+        if (hipGetDevice(&cur) == hipSuccess && cur != device) {
+            previous_ = cur;
+            HIP_ASSERT(hipSetDevice(device));
+        }
+    }
+    ~DeviceScope() { if (previous_ >= 0) (void)hipSetDevice(previous_); }
+
+private:
+    int previous_ = -1;
+};
+
+} // namespace
+
 void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
 {
     auto *cmd = dynamic_cast<HipCommand *>(hw_cmd.get());
     XASSERT(cmd != nullptr, "hw_cmd is not a HipCommand");
+    DeviceScope scope(device_);
     hipError_t err = cmd->LaunchWrapper(*this, false);
     XASSERT(err == hipSuccess, "failed to enqueue command: %d (%s)", (int)err, hipGetErrorString(err));
     n_launch.fetch_add(1, std::memory_order_relaxed);
 }
 
-void HipQueue::Synchronize() { HIP_ASSERT(hipStreamSynchronize(stream_)); }
+// Polls first, like a marker wait: the blocking call costs a sleep and a wake-up
+// through the driver, which is longer than most foreground kernels run.
+void HipQueue::Synchronize()
+{
+    DeviceScope scope(device_);
+    const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(SyncSpinMicros());
+    while (true) {
+        const hipError_t err = hipStreamQuery(stream_);
+        if (err == hipSuccess) return;
+        XASSERT(err == hipErrorNotReady, "hipStreamQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
+        if (std::chrono::steady_clock::now() >= give_up) break;
+        __builtin_ia32_pause();
+    }
+    HIP_ASSERT(hipStreamSynchronize(stream_));
+}
 
 void HipQueue::Deactivate()
 {

@@ -47,6 +47,10 @@ public:
     }
     virtual bool Synchronizable() override { return marked_; }
     virtual bool EnableSynchronization() override { marked_ = true; return true; }
+    // Launching is handing a ticket to the executor thread: any thread may do it. (No
+    // `override`: this file is also compiled against the plugin interface without the
+    // direct-launch extension.)
+    virtual bool DirectLaunchable() { return true; }
 
     bool Finished() const
     {
@@ -120,6 +124,7 @@ public:
     virtual bool SupportDynamicLevel() override { return true; }
     virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
     virtual void OnPreemptLevelChange(XPreemptLevel level) override { level_ = level; }
+    virtual bool SupportDirectLaunch() { return true; }
 
     void GetStats(uint64_t *executed, uint64_t *skipped, uint64_t *replays) const
     {

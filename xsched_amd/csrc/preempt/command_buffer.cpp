@@ -38,7 +38,8 @@ std::shared_ptr<XCommand> CommandBuffer::Dequeue()
 {
     std::unique_lock<std::mutex> lock(mtx_);
 
-    if (cmds_.empty()) {
+    while (cmds_.empty()) {
+        drain_needed_ = false;
         switch (last_enqueued_cmd_->GetType()) {
         case kCommandTypeXQueueWaitAll:
             if (xq_state_ == kQueueStateReady) {
@@ -48,8 +49,10 @@ std::shared_ptr<XCommand> CommandBuffer::Dequeue()
                 SchedAgent::SendEvent(std::make_shared<XQueueIdleEvent>(kXQueueHandle));
             }
             consumer_waiting_ = true;
-            cv_.wait(lock, [this]() { return !cmds_.empty(); });
+            cv_.wait(lock, [this]() { return !cmds_.empty() || drain_needed_; });
             consumer_waiting_ = false;
+            // Woken with an empty buffer: a command was launched directly meanwhile and
+            // is now the last one enqueued, so the next pass starts the drain sequence.
             break;
 
         case kCommandTypeBatchSynchronize:
@@ -84,12 +87,20 @@ void CommandBuffer::Enqueue(std::shared_ptr<XCommand> xcmd)
     bool wake;
     {
         std::lock_guard<std::mutex> lock(mtx_);
-        if (xcmd->GetType() == kCommandTypeHardware && xq_state_ == kQueueStateIdle) {
+        const bool hardware = xcmd->GetType() == kCommandTypeHardware;
+        if (hardware && xq_state_ == kQueueStateIdle) {
             xq_state_ = kQueueStateReady;
             SchedAgent::SendEvent(std::make_shared<XQueueReadyEvent>(kXQueueHandle, ready_time));
         }
         last_enqueued_cmd_ = xcmd;
-        cmds_.emplace_back(std::move(xcmd));
+        // The launch thread sleeps and nothing is queued: submission order is launch
+        // order even if this thread launches, and the lock keeps it so.
+        if (hardware && direct_launch_ && consumer_waiting_ && cmds_.empty() &&
+            direct_launch_(std::static_pointer_cast<HwCommand>(xcmd))) {
+            drain_needed_ = true;
+        } else {
+            cmds_.emplace_back(std::move(xcmd));
+        }
         wake = consumer_waiting_;
     }
     if (wake) cv_.notify_one();
@@ -102,9 +113,10 @@ void CommandBuffer::DropAll()
     cmds_.clear();
 }
 
-std::shared_ptr<XQueueWaitAllCommand> CommandBuffer::EnqueueXQueueWaitAllCommand()
+std::shared_ptr<XQueueWaitAllCommand> CommandBuffer::EnqueueXQueueWaitAllCommand(bool *consumer_asleep)
 {
     std::unique_lock<std::mutex> lock(mtx_);
+    if (consumer_asleep) *consumer_asleep = consumer_waiting_;
 
     // Idle: the tail is the drain marker that made the queue idle (completed).
     // Not idle but the tail is already a drain marker: share it.

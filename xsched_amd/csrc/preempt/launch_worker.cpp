@@ -150,31 +150,18 @@ void LaunchWorker::Loop()
 //  5. Launch, log it.
 void LaunchWorker::LaunchHwCommand(std::shared_ptr<HwCommand> hw_cmd)
 {
-    const bool wait_deactivatable = level_ >= kPreemptLevelDeactivate &&
-        hw_cmd->GetProps(kCommandPropertyDeactivatable | kCommandPropertyIdempotent)
-            == kCommandPropertyNone;
-
     hw_cmd->BeforeLaunch();
     Lock lock(mtx_);
 
-    if (wait_deactivatable) {
-        // Newest to oldest: remember the earliest marker that still lies behind
-        // the newest deactivatable command.
-        bool has_deactivatable = false;
-        std::shared_ptr<HwCommand> marker;
-        for (auto it = cmd_log_.rbegin(); it != cmd_log_.rend(); ++it) {
-            if ((*it)->Synchronizable()) marker = *it;
-            if ((*it)->GetProps(kCommandPropertyDeactivatable)) { has_deactivatable = true; break; }
-        }
-        if (has_deactivatable) {
-            if (marker) SyncCmdLocked(lock, marker);
-            else SyncAllLocked(lock);
-        }
+    std::shared_ptr<HwCommand> marker;
+    if (NeedsDrainBefore(hw_cmd, &marker)) {
+        if (marker) SyncCmdLocked(lock, marker);
+        else SyncAllLocked(lock);
     }
 
     if (cmd_log_.size() >= (size_t)threshold_) {
         const int64_t front_idx = cmd_log_.front()->GetIdx();
-        std::shared_ptr<HwCommand> marker;
+        marker = nullptr;
         for (auto &cmd : sync_cmd_log_) {
             if (cmd->GetIdx() >= front_idx) { marker = cmd; break; }
         }
@@ -185,8 +172,31 @@ void LaunchWorker::LaunchHwCommand(std::shared_ptr<HwCommand> hw_cmd)
         XASSERT(running, "launch thread asked to launch after termination");
     }
 
+    LaunchLocked(hw_cmd);
+}
+
+// Step 1's test. Newest to oldest: remember the earliest marker that still lies behind
+// the newest deactivatable command.
+bool LaunchWorker::NeedsDrainBefore(const std::shared_ptr<HwCommand> &hw_cmd, std::shared_ptr<HwCommand> *marker)
+{
+    if (level_ < kPreemptLevelDeactivate) return false;
+    if (hw_cmd->GetProps(kCommandPropertyDeactivatable | kCommandPropertyIdempotent) != kCommandPropertyNone) {
+        return false;
+    }
+    for (auto it = cmd_log_.rbegin(); it != cmd_log_.rend(); ++it) {
+        if ((*it)->Synchronizable()) *marker = *it;
+        if ((*it)->GetProps(kCommandPropertyDeactivatable)) return true;
+    }
+    *marker = nullptr;
+    return false;
+}
+
+// Steps 3 to 5, lock held.
+void LaunchWorker::LaunchLocked(const std::shared_ptr<HwCommand> &hw_cmd)
+{
     if (hw_cmd->GetIdx() <= drop_idx_) {
         hw_cmd->SetState(kCommandStateCompleted);
+        handled_idx_.store(hw_cmd->GetIdx(), std::memory_order_release);
         return;
     }
 
@@ -208,6 +218,25 @@ void LaunchWorker::LaunchHwCommand(std::shared_ptr<HwCommand> hw_cmd)
         sync_cmd_log_.emplace_back(hw_cmd);
         last_synchronizable_idx_ = hw_cmd->GetIdx();
     }
+    handled_idx_.store(hw_cmd->GetIdx(), std::memory_order_release);
+}
+
+// The same command through the same window on the SUBMITTING thread, but only when none
+// of the steps would have to wait. The caller (CommandBuffer::Enqueue) holds the buffer
+// lock and has seen the launch thread asleep on an empty buffer, so no other command
+// can slip in between.
+bool LaunchWorker::TryLaunchDirect(const std::shared_ptr<HwCommand> &hw_cmd)
+{
+    if (!hw_cmd->DirectLaunchable() || hw_cmd->GetProps(kCommandPropertyCallback)) return false;
+    Lock lock(mtx_);
+    if (state_ != kRunning) return false;
+    if (cmd_log_.size() >= (size_t)threshold_) return false;
+    std::shared_ptr<HwCommand> marker;
+    if (NeedsDrainBefore(hw_cmd, &marker)) return false;
+    hw_cmd->BeforeLaunch(); // never blocks for a command that declares itself DirectLaunchable
+    LaunchLocked(hw_cmd);
+    direct_launches_.fetch_add(1, std::memory_order_relaxed);
+    return true;
 }
 
 // The blocking driver wait happens with the lock released. If a Pause() came in
@@ -220,13 +249,15 @@ void LaunchWorker::SyncAllLocked(Lock &lock)
         if (!WaitWhilePaused(lock)) return;
         if (cmd_log_.empty()) return;
 
+        // With direct launches another thread may add commands while the lock is
+        // released: only what was in flight when the wait began is known to be done.
+        const int64_t last_idx = cmd_log_.back()->GetIdx();
         const int64_t pause_cnt = pause_count_;
         lock.unlock();
         kHwq->Synchronize();
         lock.lock();
-        if (pause_cnt == pause_count_) break;
+        if (pause_cnt == pause_count_) { RetireUpTo(last_idx); return; }
     }
-    RetireAll();
 }
 
 // Same retry rule; in addition the command may be completed by another thread
@@ -254,7 +285,11 @@ void LaunchWorker::SyncCmdLocked(Lock &lock, const std::shared_ptr<HwCommand> &h
         if (pause_cnt == pause_count_) break;
     }
 
-    const int64_t idx = hw_cmd->GetIdx();
+    RetireUpTo(hw_cmd->GetIdx());
+}
+
+void LaunchWorker::RetireUpTo(int64_t idx)
+{
     while (!sync_cmd_log_.empty() && sync_cmd_log_.front()->GetIdx() <= idx) {
         sync_cmd_log_.pop_front();
     }

@@ -299,3 +299,11 @@ EXPORT_C_FUNC XResult XQueueProfileHwCommandCount(XQueueHandle xq, int64_t *coun
     *count = q->GetHwCommandCount();
     return kXSchedSuccess;
 }
+
+EXPORT_C_FUNC XResult XQueueProfileDirectLaunchCount(XQueueHandle xq, int64_t *count)
+{
+    if (count == nullptr) return kXSchedErrorInvalidValue;
+    FIND_XQUEUE_OR_RETURN(q, xq);
+    *count = q->GetDirectLaunchCount();
+    return kXSchedSuccess;
+}
