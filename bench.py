@@ -69,8 +69,8 @@ def bg_ms_per_launch(H, kind, n, level, guard, commands=40, warm=8):
         return res.bg_stream_ms / res.bg_stream_cmds
 
 
-def preempt_latency(H, kind, n, level, samples):
-    cfg = H.Config(0, 1, H.spec(kind, n, 1, level, BG_THRESHOLD, BG_BATCH, 1),
+def preempt_latency(H, kind, n, level, samples, guard=1):
+    cfg = H.Config(0, 1, H.spec(kind, n, guard, level, BG_THRESHOLD, BG_BATCH, 1),
                    H.spec(kind, 0, 0, 1, 8, 4, 2), 64, 0)
     with H.Bench(cfg) as b:
         sus, resume, res = b.preempt(samples)
@@ -169,6 +169,13 @@ def config2(H, a):
                          "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
                          "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
         line["preempt_us"] = preempt_block(H, H.AXPY, bg_n, False)
+        # The other end of the AXPY trade-off (guard mode 3): a few long-lived waves per CU.
+        ms_sd = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 3)
+        sus, res, _ = preempt_latency(H, H.AXPY, bg_n, 2, 200, guard=3)
+        line["short_drain_variant"] = {
+            "level2_GBs": axpy_bytes(bg_n) / ms_sd / 1e6, "level2_overhead_frac": 1.0 - ms_plain / ms_sd,
+            "level2_suspend_sync_p50": H.pct(sus, 0.5), "level2_suspend_sync_p99": H.pct(sus, 0.99),
+            "level2_resume_p50": H.pct(res, 0.5), "level2_resume_p99": H.pct(res, 0.99)}
     return line
 
 

@@ -43,7 +43,11 @@ XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
  *              work-group entry guard and a progress map; at level 1 the same
  *              command launches the plain variant.
  *          2 = always launch the guarded variant, even at level 1 (for measuring
- *              the cost of the guard). */
+ *              the cost of the guard).
+ *          3 = like 1, but prefer the kernel's short-drain variant where it has one
+ *              (AXPY: a few long-lived waves per CU instead of one wave per chunk: the
+ *              device drains in 20-30 us instead of ~190 us after a deactivation, at
+ *              ~8 % less bandwidth). Same as 1 for the other kernels. */
 
 /* y[i] = fma(alpha, x[i], y[i]) in place, fp32, i < n. 128-bit loads/stores when
  * x and y are 16-byte aligned. */

@@ -56,7 +56,7 @@ def hist_cmd(xs, keys, n, bins, n_bins, guard):
 
 
 @pytest.mark.parametrize("n", [0, 1, 3, 5, 1023, 4096, 4097, (1 << 20) + 7, 1 << 22])
-@pytest.mark.parametrize("level,guard", [(1, 0), (1, 2), (2, 1)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (1, 2), (2, 1), (2, 3), (1, 3)])
 def test_axpy_bit_exact(xs, gpu, n, level, guard):
     torch = gpu
     print(f"case axpy n={n} level={level} guard={guard}", flush=True)

@@ -35,11 +35,12 @@ def churn(xs, q, stop, seed, flags=0):
     return cycles
 
 
+@pytest.mark.parametrize("guard", [1, 3])          # 3 = few long-lived waves per CU
 @pytest.mark.parametrize("suspend_flags", [0, 1])  # 1 = kQueueSuspendFlagSyncHwQueue
-def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags):
+def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags, guard):
     torch = gpu
-    n, times = 1 << 24, 60
-    print(f"case axpy-preempt n={n} times={times} flags={suspend_flags}", flush=True)
+    n, times = (1 << 24) + 5, 60
+    print(f"case axpy-preempt n={n} times={times} flags={suspend_flags} guard={guard}", flush=True)
     x_h = oracle.fill_uniform(5, 1, 0, n)
     y_h = oracle.fill_uniform(5, 2, 0, n)
     x = torch.from_numpy(x_h).cuda()
@@ -50,7 +51,7 @@ def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags):
     t = threading.Thread(target=lambda: result.setdefault("cycles", churn(xs, q, stop, 1, suspend_flags)))
     t.start()
     for _ in range(times):
-        q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, guard))
     # Keep churning while the queue drains, then stop and let it finish.
     time.sleep(0.05)
     stop.set()
@@ -181,3 +182,4 @@ def test_null_stream_and_bad_arguments(xs, gpu):
     assert h.HipGemmBf16CommandCreate(byref(cmd), 16, 16, 16, 100, 256, 64, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipHistogramCommandCreate(byref(cmd), 16, 4, 16, 70000, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, None, None, 4, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipAxpyCommandCreate(byref(cmd), 1.0, 16, 16, 4, 4) == xs.kXSchedErrorInvalidValue

@@ -127,7 +127,8 @@ private:
 class HipGuardedCommand : public HipCommand
 {
 public:
-    /// guard_mode: 0 plain, 1 guarded at level >= 2, 2 guarded always.
+    /// guard_mode: 0 plain, 1 guarded at level >= 2, 2 guarded always, 3 like 1 with the
+    /// kernel's short-drain variant where it has one.
     HipGuardedCommand(uint32_t n_wg, int guard_mode)
         : HipCommand(guard_mode ? preempt::kCommandPropertyDeactivatable : preempt::kCommandPropertyNone)
         , n_wg_(n_wg), guard_mode_(guard_mode) {}

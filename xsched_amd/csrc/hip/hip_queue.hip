@@ -254,7 +254,7 @@ HipGuardedCommand::~HipGuardedCommand()
 hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
 {
     const bool level2 = q.Level() >= kPreemptLevelDeactivate;
-    const bool guarded = guard_mode_ == 2 || (guard_mode_ == 1 && level2);
+    const bool guarded = guard_mode_ == 2 || (guard_mode_ != 0 && level2);
 
     XGuardArgs g;
     g.flag = q.Guard()->FlagDevPtr();

@@ -1,12 +1,25 @@
 // Guarded streaming AXPY for gfx950: y = fma(alpha, x, y), fp32, in place.
 //
-// HBM-bound: 12 bytes of traffic per element (read x, read y, write y). One
-// work-group is one wavefront; it owns a contiguous chunk of `steps` x 1024
-// elements and walks it in steps of 4 x 128-bit accesses per lane and stream,
-// lane-contiguous so that every access of a wave covers 1 KiB. Loads and stores
-// are non-temporal: nothing is reused. Because the update is in place, a
-// work-group must run exactly once: it reads the preempt word first, and commits
-// its byte in the progress map after its last store.
+// HBM-bound: 12 bytes of traffic per element (read x, read y, write y). The unit of
+// work is a chunk of `steps` x 1024 contiguous elements, walked by one wavefront in
+// steps of 4 x 128-bit accesses per lane and stream, lane-contiguous so that every
+// access of a wave covers 1 KiB. Loads and stores are non-temporal: nothing is reused.
+// Because the update is in place, a chunk must be applied exactly once: the wave reads
+// the preempt word before it stores anything, and commits the chunk's byte in the
+// progress map after its last store.
+//
+// Two grids:
+//   one single-wave work-group per chunk (default). Short-lived waves give the best
+//       bandwidth (6.2-6.3 TB/s on MI355X) and let a concurrent kernel find free wave
+//       slots within microseconds. After a deactivation the device still has to start
+//       and retire every remaining work-group, empty: ~3.3 waves per nanosecond, so two
+//       launches of 262144 work-groups in flight drain in ~190 us.
+//   guard mode 3: a fixed number of waves per CU, each walking chunks c, c + G,
+//       c + 2G, ... and re-reading the preempt word while the next chunk's loads are in
+//       flight. Every wave stops at its next chunk and a launch queued behind has only G
+//       work-groups to retire: the device drains in 20-30 us. Long-lived waves stream
+//       at 5.3-5.8 TB/s, though (the same loss shows with larger chunks per work-group,
+//       or several waves per work-group), so this is the latency end of a trade-off.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 #include "xsched/utils/env.h"
@@ -87,6 +100,69 @@ void AxpyVec4Kernel(float alpha, const float4 *x, float4 *y,
     if (kGuard) guard.Commit();
 }
 
+// Guarded launches: grid-stride over chunks, see the head of this file. `n_chunks`
+// chunks of `steps` x 1024 elements; the progress map has one byte per chunk.
+__global__ __launch_bounds__(64)
+void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, uint32_t tail,
+                          uint32_t steps, uint32_t n_chunks, XGuardArgs g)
+{
+    constexpr uint32_t kVecPerStep = 4;
+    constexpr uint32_t kStepVecs = kLanes * kVecPerStep;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t *flag = xguard_flag_copy(g, blockIdx.x);
+
+    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const uint64_t chunk_base = (uint64_t)c * steps * kStepVecs;
+        const bool full = chunk_base + (uint64_t)steps * kStepVecs <= n4;
+        const uint64_t base = chunk_base + lane;
+        float4 xv[kVecPerStep], yv[kVecPerStep];
+        if (full) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                xv[u] = ld_nt(&x[base + u * kLanes]);
+                yv[u] = ld_nt(&y[base + u * kLanes]);
+            }
+        }
+        // The scalar read of the preempt word waits for itself only: the vector loads
+        // above stay in flight across it. A flushed wave drops what it has loaded.
+        if (xguard_read_flag(flag) != g.epoch) return;
+        if (g.resume && g.done && xguard_committed(g, c)) continue;
+
+        if (full) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                st_nt(&y[base + u * kLanes], fma4(alpha, xv[u], yv[u]));
+            }
+            // Chunks of more than one step (arrays beyond 2^28 elements): the rest of the
+            // chunk, with registers of its own so that nothing is carried around the loop.
+            for (uint32_t s = 1; s < steps; ++s) {
+                const uint64_t b = base + (uint64_t)s * kStepVecs;
+                float4 xs[kVecPerStep], ys[kVecPerStep];
+#pragma unroll
+                for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                    xs[u] = ld_nt(&x[b + u * kLanes]);
+                    ys[u] = ld_nt(&y[b + u * kLanes]);
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < kVecPerStep; ++u) {
+                    st_nt(&y[b + u * kLanes], fma4(alpha, xs[u], ys[u]));
+                }
+            }
+        } else {
+            const uint64_t end = chunk_base + (uint64_t)steps * kStepVecs;
+            for (uint64_t i = chunk_base + lane; i < end && i < n4; i += kLanes) {
+                st_nt(&y[i], fma4(alpha, ld_nt(&x[i]), ld_nt(&y[i])));
+            }
+            if (c == n_chunks - 1 && lane < tail) {
+                const float *xs = (const float *)(x + n4);
+                float *ys = (float *)(y + n4);
+                ys[lane] = __builtin_fmaf(alpha, xs[lane], ys[lane]);
+            }
+        }
+        if (g.done && lane == 0) xguard_commit(g, c);
+    }
+}
+
 // Fallback for pointers that are not 16-byte aligned: same chunking, 32-bit accesses.
 template <bool kGuard>
 __global__ __launch_bounds__(64)
@@ -120,9 +196,12 @@ protected:
         if (n_ == 0) return hipSuccess;
         const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
         const dim3 grid(n_wg_), block(kLanes);
-        int64_t lds = 0;
-        GetEnvInt64("XSCHED_HIP_AXPY_LDS_BYTES", lds);
-        if (aligned) {
+        if (aligned && guarded && guard_mode_ == 3) {
+            const uint32_t waves = PersistentWaves();
+            const dim3 pgrid(n_wg_ < waves ? n_wg_ : waves);
+            hipLaunchKernelGGL(AxpyPersistentKernel, pgrid, block, 0, stream, alpha_, (const float4 *)x_,
+                               (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
+        } else if (aligned) {
             const uint64_t n4 = n_ / 4;
             const uint32_t tail = (uint32_t)(n_ % 4);
             // An even chunk is walked in steps of 2048 elements (8 accesses in flight
@@ -131,10 +210,10 @@ protected:
             const uint32_t steps = wide ? steps_ / 2 : steps_;
             const float4 *xv = (const float4 *)x_;
             float4 *yv = (float4 *)y_;
-            if (guarded && wide)       hipLaunchKernelGGL((AxpyVec4Kernel<true, 8>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else if (guarded)          hipLaunchKernelGGL((AxpyVec4Kernel<true, 4>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else if (wide)             hipLaunchKernelGGL((AxpyVec4Kernel<false, 8>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else                       hipLaunchKernelGGL((AxpyVec4Kernel<false, 4>), grid, block, (size_t)lds, stream, alpha_, xv, yv, n4, tail, steps, g);
+            if (guarded && wide)       hipLaunchKernelGGL((AxpyVec4Kernel<true, 8>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (guarded)          hipLaunchKernelGGL((AxpyVec4Kernel<true, 4>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (wide)             hipLaunchKernelGGL((AxpyVec4Kernel<false, 8>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else                       hipLaunchKernelGGL((AxpyVec4Kernel<false, 4>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
         } else {
             if (guarded) {
                 hipLaunchKernelGGL(AxpyScalarKernel<true>, grid, block, 0, stream, alpha_, x_, y_,
@@ -148,6 +227,23 @@ protected:
     }
 
 private:
+    /// Work-groups (= waves) of a guarded launch: a fixed number per compute unit.
+    static uint32_t PersistentWaves()
+    {
+        static const uint32_t waves = []() {
+            int64_t per_cu = 8;
+            GetEnvInt64("XSCHED_HIP_AXPY_WAVES_PER_CU", per_cu);
+            if (per_cu < 1) per_cu = 1;
+            if (per_cu > 64) per_cu = 64;
+            int dev = 0, cus = 256;
+            if (hipGetDevice(&dev) == hipSuccess) {
+                (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            }
+            return (uint32_t)(per_cu * (cus > 0 ? cus : 256));
+        }();
+        return waves;
+    }
+
     const float alpha_;
     const float *x_;
     float *y_;
@@ -178,7 +274,7 @@ using namespace xsched::hip;
 EXPORT_C_FUNC XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, void *y,
                                            size_t n, int guard)
 {
-    if (cmd == nullptr || (n != 0 && (x == nullptr || y == nullptr)) || guard < 0 || guard > 2) {
+    if (cmd == nullptr || (n != 0 && (x == nullptr || y == nullptr)) || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
     const uint32_t steps = AxpyStepsFor(n);

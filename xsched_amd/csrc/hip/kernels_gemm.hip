@@ -242,7 +242,7 @@ using namespace xsched::hip;
 EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void *B,
                                                void *C, int M, int N, int K, int guard)
 {
-    if (cmd == nullptr || A == nullptr || B == nullptr || C == nullptr || guard < 0 || guard > 2) {
+    if (cmd == nullptr || A == nullptr || B == nullptr || C == nullptr || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
     if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kTile || N % gemm::kTile || K % gemm::kStepK) {

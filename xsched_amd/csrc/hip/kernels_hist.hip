@@ -403,7 +403,7 @@ using namespace xsched::hip;
 EXPORT_C_FUNC XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t n,
                                                 void *bins, uint32_t n_bins, int guard)
 {
-    if (cmd == nullptr || bins == nullptr || (n != 0 && keys == nullptr) || guard < 0 || guard > 2) {
+    if (cmd == nullptr || bins == nullptr || (n != 0 && keys == nullptr) || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
     if (n_bins == 0 || n_bins > 65536) return kXSchedErrorInvalidValue;
