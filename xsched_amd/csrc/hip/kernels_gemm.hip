@@ -2,11 +2,12 @@
 // accumulation in ascending k, bf16 (round-to-nearest-even) output.
 //
 // MFMA-bound: 2*M*N*K flop. One work-group of 512 threads (8 wavefronts) owns one
-// 256x256 tile of C and walks K in steps of 64:
-//   global -> registers (prefetch of step t+1 while step t is computed)
+// 256x256 tile of C and walks K in steps of 64 through two LDS buffers:
+//   global -> registers (tile t+2 is requested while tile t is computed)
 //   registers -> LDS    A tile as [256 rows][64 k], B tile transposed to [256 cols][64 k],
 //                       both with rows padded to 72 bf16 so that the 128-bit fragment
-//                       reads of 32 consecutive rows fall into distinct banks
+//                       reads of 32 consecutive rows fall into distinct banks; written to
+//                       the buffer that is not being read, one barrier per step
 //   LDS -> MFMA         v_mfma_f32_32x32x16_bf16; wave (wm, wn) of the 2x4 wave grid
 //                       accumulates a 128x64 sub-tile = 4x2 blocks of 32x32
 // B is read from global memory as 32-bit words (two columns) over eight k rows and
@@ -72,28 +73,29 @@ __device__ __forceinline__ void TileOf(uint32_t wg, uint32_t tiles_m, uint32_t t
     tn = in_band / rows;
 }
 
+// Two LDS buffers and ONE barrier per K step: while the MFMAs of step t read buffer
+// t % 2, the registers holding tile t + 1 are written to the other buffer and the global
+// loads of tile t + 2 are issued; the A fragments of the next 16-wide k slice are read from
+// LDS before the MFMAs of the current slice are issued.
 template <bool kGuard>
 __global__ __launch_bounds__(kThreads)
 void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                    uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
+                             uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t As[kTile * kLdsStride];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[kTile * kLdsStride];
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][kTile * kLdsStride];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kTile * kLdsStride];
     __shared__ uint32_t guard_word;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
-    const uint32_t wm = wave >> 2;   // 0..1 : rows 128*wm
-    const uint32_t wn = wave & 3;    // 0..3 : cols 64*wn
+    const uint32_t wm = wave >> 2;
+    const uint32_t wn = wave & 3;
 
     uint32_t tm, tn;
     TileOf(blockIdx.x, (uint32_t)M / kTile, (uint32_t)N / kTile, tm, tn);
     const size_t m0 = (size_t)tm * kTile, n0 = (size_t)tn * kTile;
 
-    // ---- global -> register staging -------------------------------------------------
-    // A: 256 rows x 8 chunks of 8 bf16 = 2048 chunks, 4 per thread.
-    // B: 8 k-groups (of 8 rows) x 128 column pairs = 1024 items, 2 per thread.
     u32x4 a_reg[4];
     uint32_t b_reg[2][8];
 
@@ -114,29 +116,45 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         }
     };
 
-    auto store_lds = [&]() {
+    auto store_lds = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t c = tid + kThreads * i;
             const uint32_t row = c >> 3, kc = c & 7;
-            *(u32x4 *)(As + row * kLdsStride + kc * 8) = a_reg[i];
+            *(u32x4 *)(As[buf] + row * kLdsStride + kc * 8) = a_reg[i];
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t c = tid + kThreads * i;
             const uint32_t npair = c & 127, kg = c >> 7;
-            // b_reg[i][r] = { B[k+r][n] (low half), B[k+r][n+1] (high half) }.
-            // Column n gets the low halves of rows r, r+1 packed; column n+1 the high halves.
             u32x4 col0, col1;
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const uint32_t lo = b_reg[i][2 * p], hi = b_reg[i][2 * p + 1];
-                col0[p] = __builtin_amdgcn_perm(hi, lo, 0x05040100u); // lo.l | hi.l << 16
-                col1[p] = __builtin_amdgcn_perm(hi, lo, 0x07060302u); // lo.h | hi.h << 16
+                col0[p] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                col1[p] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
             }
-            *(u32x4 *)(Bs + (npair * 2 + 0) * kLdsStride + kg * 8) = col0;
-            *(u32x4 *)(Bs + (npair * 2 + 1) * kLdsStride + kg * 8) = col1;
+            *(u32x4 *)(Bs[buf] + (npair * 2 + 0) * kLdsStride + kg * 8) = col0;
+            *(u32x4 *)(Bs[buf] + (npair * 2 + 1) * kLdsStride + kg * 8) = col1;
         }
+    };
+
+    const uint32_t a_row0 = 128 * wm + (lane & 31);
+    const uint32_t b_col0 = 64 * wn + (lane & 31);
+    const uint32_t khalf = 8 * (lane >> 5);
+    auto load_a_frags = [&](int buf, int ks, bf16x8 *fa) {
+        const uint32_t koff = ks * 16 + khalf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = *(const bf16x8 *)(As[buf] + (a_row0 + 32 * i) * kLdsStride + koff);
+    };
+    auto load_b_frags = [&](int buf, int ks, bf16x8 *fb) {
+        const uint32_t koff = ks * 16 + khalf;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[j] = *(const bf16x8 *)(Bs[buf] + (b_col0 + 32 * j) * kLdsStride + koff);
+    };
+    auto load_frags = [&](int buf, int ks, bf16x8 *fa, bf16x8 *fb) {
+        load_a_frags(buf, ks, fa);
+        load_b_frags(buf, ks, fb);
     };
 
     f32x16 acc[4][2];
@@ -155,43 +173,62 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     }
 
     const int steps = K / kStepK;
+    store_lds(0);
+    load_global(steps > 1 ? kStepK : 0);
+    __syncthreads();
+
+    // The loop body is branch-free (loads and LDS stores past the last tile are clamped or
+    // harmless repeats), so that it is one scheduling region. Per step and wave: 32 MFMAs in four k slices of 8; next to them
+    //   slice 0: fragment reads of slice 1
+    //   slice 1: fragment reads of slice 2, registers of tile t+1 -> the other LDS buffer
+    //   slice 2: fragment reads of slice 3, global loads of tile t+2
+    //   barrier  (the other buffer is complete, this one is no longer read)
+    //   slice 3: fragment reads of slice 0 of the NEXT tile from the other buffer
+    // A fragments are double-buffered in registers, the two B fragments are re-read per
+    // slice after the slice's MFMAs have been issued: the register file (256 per wave at two
+    // waves per SIMD) has no room for a second set of both.
+    bf16x8 fa[2][4], fb[2];
+    load_frags(0, 0, fa[0], fb);
+
+    auto mfma_slice = [&](int set) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[j], acc[i][j], 0, 0, 0);
+    };
+
     for (int t = 0; t < steps; ++t) {
-        store_lds();
-        if (kGuard && t != 0 && (t % kPollSteps) == 0 && tid == 0) {
+        const int cur = t & 1;
+        const int k_next = (t + 2 < steps ? t + 2 : steps - 1) * kStepK;
+
+        load_a_frags(cur, 1, fa[1]);
+        mfma_slice(0);
+        load_b_frags(cur, 1, fb);
+
+        load_a_frags(cur, 2, fa[0]);
+        store_lds(cur ^ 1);
+        mfma_slice(1);
+        load_b_frags(cur, 2, fb);
+
+        load_a_frags(cur, 3, fa[1]);
+        load_global(k_next);
+        mfma_slice(0);
+        load_b_frags(cur, 3, fb);
+
+        if (kGuard && (t % kPollSteps) == kPollSteps - 1 && tid == 0) {
             guard_word = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch ? 1u : 0u;
         }
-        __syncthreads();
-        if (kGuard && t != 0 && (t % kPollSteps) == 0) {
+        __syncthreads(); // buffer cur^1 is complete, buffer cur is free to be overwritten
+        if (kGuard && (t % kPollSteps) == kPollSteps - 1) {
             if (guard_word == 0) return; // whole group leaves together; nothing was written
         }
-        if (t + 1 < steps) load_global((t + 1) * kStepK);
 
-#pragma unroll
-        for (int ks = 0; ks < kStepK / 16; ++ks) {
-            const uint32_t koff = ks * 16 + 8 * (lane >> 5);
-            bf16x8 a_frag[4], b_frag[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t row = 128 * wm + 32 * i + (lane & 31);
-                a_frag[i] = *(const bf16x8 *)(As + row * kLdsStride + koff);
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const uint32_t col = 64 * wn + 32 * j + (lane & 31);
-                b_frag[j] = *(const bf16x8 *)(Bs + col * kLdsStride + koff);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[i], b_frag[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads(); // everyone is done reading before the next store_lds()
+        load_a_frags(cur ^ 1, 0, fa[0]);
+        mfma_slice(1);
+        load_b_frags(cur ^ 1, 0, fb);
     }
 
-    // ---- epilogue: fp32 -> bf16, one store per accumulator register ------------------
-    // Accumulator register r of a 32x32 block holds row 8*(r/4) + 4*(lane/32) + r%4,
-    // column lane%32.
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
