@@ -77,10 +77,23 @@ def preempt_latency(H, kind, n, level, samples, guard=1):
         return sus, resume, list(res.stats)
 
 
+def device_drain(H, kind, n, level, samples, guard=1):
+    """Device-side preemption latency (HIP events, see bench.h), microseconds."""
+    cfg = H.Config(0, 1, H.spec(kind, n, guard, level, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(kind, 0, 0, 1, 8, 4, 2), 64, 0)
+    with H.Bench(cfg) as b:
+        drain, _ = b.preempt_device_timed(samples)
+        return drain
+
+
 def preempt_block(H, kind, n, quick):
     sus2, res2, st2 = preempt_latency(H, kind, n, 2, 60 if quick else 200)
     sus1, _, _ = preempt_latency(H, kind, n, 1, 30 if quick else 60)
-    return {"level2_suspend_sync_p50": H.pct(sus2, 0.5), "level2_suspend_sync_p99": H.pct(sus2, 0.99),
+    dev2 = device_drain(H, kind, n, 2, 60 if quick else 200)
+    dev1 = device_drain(H, kind, n, 1, 30 if quick else 60)
+    return {"level2_device_drain_p50": H.pct(dev2, 0.5), "level2_device_drain_p99": H.pct(dev2, 0.99),
+            "level1_device_drain_p50": H.pct(dev1, 0.5), "level1_device_drain_p99": H.pct(dev1, 0.99),
+            "level2_suspend_sync_p50": H.pct(sus2, 0.5), "level2_suspend_sync_p99": H.pct(sus2, 0.99),
             "level2_resume_p50": H.pct(res2, 0.5), "level2_resume_p99": H.pct(res2, 0.99),
             "level1_suspend_sync_p50": H.pct(sus1, 0.5), "level1_suspend_sync_p99": H.pct(sus1, 0.99),
             "level2_stats": st2}
@@ -172,7 +185,9 @@ def config2(H, a):
         # The other end of the AXPY trade-off (guard mode 3): a few long-lived waves per CU.
         ms_sd = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 3)
         sus, res, _ = preempt_latency(H, H.AXPY, bg_n, 2, 200, guard=3)
+        dev = device_drain(H, H.AXPY, bg_n, 2, 200, guard=3)
         line["short_drain_variant"] = {
+            "level2_device_drain_p50": H.pct(dev, 0.5), "level2_device_drain_p99": H.pct(dev, 0.99),
             "level2_GBs": axpy_bytes(bg_n) / ms_sd / 1e6, "level2_overhead_frac": 1.0 - ms_plain / ms_sd,
             "level2_suspend_sync_p50": H.pct(sus, 0.5), "level2_suspend_sync_p99": H.pct(sus, 0.99),
             "level2_resume_p50": H.pct(res, 0.5), "level2_resume_p99": H.pct(res, 0.99)}
@@ -260,7 +275,7 @@ def config4(H, a):
 
 def config5(H, a):
     axpy_n, gemm_n, hist_n, nq = 1 << 24, 2048, 1 << 24, 16
-    duration = a.steps / 100.0  # default 150 steps -> 1.5 s of arrivals, ~300 commands per queue
+    duration = min(a.steps / 100.0, 4.0)  # seconds of arrivals, ~200 commands per queue and second
     cfg = H.StressConfig(H.HPF, nq, 2, 1, 4, 2, axpy_n, gemm_n, hist_n, 5000.0, 7)
     with H.Bench(cfg) as b:
         b.stress(0.2)  # warm-up
@@ -296,8 +311,8 @@ def config5(H, a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=150)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--bg-log2", type=int, default=28)
     ap.add_argument("--fg-log2", type=int, default=22)

@@ -82,6 +82,14 @@ XResult XBenchRunContended(XBench *b, int samples, double *latency_us, XBenchPha
 XResult XBenchRunPreempt(XBench *b, int samples, double *suspend_us, double *resume_us,
                          XBenchPhaseResult *res);
 
+/* The same loop timed on the DEVICE: XQueueSuspend without the hardware-queue sync, then
+ * two timing events recorded back to back, one on an idle helper stream (it completes at
+ * once: the device time at which the deactivation is out) and one on the queue's stream
+ * behind everything in flight (it completes when the flushed launches have left the
+ * device). drain_us[i] is the time between the two as hipEventElapsedTime reports it:
+ * the device-side preemption latency, without any host wake-up in it. */
+XResult XBenchRunPreemptDeviceTimed(XBench *b, int samples, double *drain_us, XBenchPhaseResult *res);
+
 /* ---- mixed stress: many XQueues, one priority each, random arrivals ------------- */
 
 typedef struct {

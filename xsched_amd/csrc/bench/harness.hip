@@ -441,6 +441,55 @@ EXPORT_C_FUNC XResult XBenchRunPreempt(XBench *b, int samples, double *suspend_u
     return kXSchedSuccess;
 }
 
+EXPORT_C_FUNC XResult XBenchRunPreemptDeviceTimed(XBench *b, int samples, double *drain_us, XBenchPhaseResult *res)
+{
+    if (b == nullptr || b->bg.empty() || samples <= 0 || drain_us == nullptr) return kXSchedErrorInvalidValue;
+    Lane &q0 = *b->bg[0];
+    hipStream_t helper = nullptr;
+    hipEvent_t ev_out = nullptr, ev_drained = nullptr;
+    BENCH_HIP(hipStreamCreateWithFlags(&helper, hipStreamNonBlocking));
+    BENCH_HIP(hipEventCreate(&ev_out));
+    BENCH_HIP(hipEventCreate(&ev_drained));
+
+    std::atomic<bool> stop { false };
+    BgDriver driver;
+    driver.lane = &q0;
+    driver.burst = b->cfg.bg_burst > 0 ? b->cfg.bg_burst : 64;
+    driver.stop = &stop;
+    const auto t_begin = Clock::now();
+    driver.Start();
+    std::this_thread::sleep_for(std::chrono::milliseconds(50));
+
+    uint64_t lcg = 0x9E3779B97F4A7C15ull ^ b->cfg.seed;
+    for (int i = 0; i < samples; ++i) {
+        lcg = lcg * 6364136223846793005ull + 1442695040888963407ull;
+        std::this_thread::sleep_for(std::chrono::microseconds(200 + (lcg >> 33) % 800));
+        BENCH_X(XQueueSuspend(q0.xq, kQueueSuspendFlagNone));
+        // The launch thread is paused, so nothing else is enqueued on the stream now.
+        BENCH_HIP(hipEventRecord(ev_out, helper));
+        BENCH_HIP(hipEventRecord(ev_drained, q0.stream));
+        BENCH_HIP(hipEventSynchronize(ev_drained));
+        BENCH_HIP(hipEventSynchronize(ev_out));
+        float ms = 0;
+        BENCH_HIP(hipEventElapsedTime(&ms, ev_out, ev_drained));
+        drain_us[i] = (double)ms * 1e3;
+        std::this_thread::sleep_for(std::chrono::microseconds(300));
+        BENCH_X(XQueueResume(q0.xq, kQueueResumeFlagNone));
+    }
+    stop.store(true, std::memory_order_release);
+    driver.Join();
+    if (res) {
+        *res = XBenchPhaseResult {};
+        res->elapsed_s = std::chrono::duration<double>(Clock::now() - t_begin).count();
+        res->bg_commands = q0.applied.load();
+        FillStats(b, res);
+    }
+    (void)hipEventDestroy(ev_out);
+    (void)hipEventDestroy(ev_drained);
+    (void)hipStreamDestroy(helper);
+    return kXSchedSuccess;
+}
+
 EXPORT_C_FUNC XBench *XBenchCreateStress(const XBenchStressConfig *cfg)
 {
     if (cfg == nullptr || cfg->n_queues <= 0 || cfg->n_queues > 64 || cfg->mean_interarrival_us <= 0) return nullptr;

@@ -51,6 +51,7 @@ def lib():
         h.XBenchRunContended.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
         h.XBenchRunPreempt.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(c_double),
                                        POINTER(PhaseResult)]
+        h.XBenchRunPreemptDeviceTimed.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
         h.XBenchRunStress.argtypes = [c_void_p, c_double, POINTER(c_double), c_uint64, POINTER(c_uint64),
                                       POINTER(PhaseResult)]
         h.XBenchReadOutput.argtypes = [c_void_p, c_int, c_int, c_uint64, c_uint64, c_void_p,
@@ -107,6 +108,11 @@ class Bench:
         sus, resume, res = (c_double * samples)(), (c_double * samples)(), PhaseResult()
         xsched_amd.check(lib().XBenchRunPreempt(self.h, samples, sus, resume, byref(res)))
         return list(sus), list(resume), res
+
+    def preempt_device_timed(self, samples):
+        drain, res = (c_double * samples)(), PhaseResult()
+        xsched_amd.check(lib().XBenchRunPreemptDeviceTimed(self.h, samples, drain, byref(res)))
+        return list(drain), res
 
     def stress(self, duration_s, cap=4096):
         nq = self.cfg.n_queues
