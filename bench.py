@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: foreground latency under a saturating background on one MI355X.
 
-Default workload (BASELINE.json configs[1], `--config 2`): a background XQueue streams fp32
+Default workload (`--config 2`): a background XQueue streams fp32
 AXPY y = 0.5*x + y over 2^28 elements back to back (Level-1, HPF policy, priority 1); a
 foreground XQueue submits the same kernel over 2^22 elements every 20 ms (priority 2). One
 "step" is one foreground command under contention (submit -> XQueueWaitAll returns).

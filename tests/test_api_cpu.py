@@ -207,7 +207,7 @@ def test_host_level2_exactly_once_under_churn(xs):
 
 
 def test_cpu_configuration_two_queues_hpf(xs):
-    """BASELINE configuration 0 on the host adapter: two XQueues, level 1, HPF, threshold 8
+    """The CPU plumbing configuration on the host adapter: two XQueues, level 1, HPF, threshold 8
     and batch 4. Background: 1000 fp32 vector additions of 2^20 elements (uniform [-1,1),
     seed 0); foreground: one 2^16-element addition every 10 ms, higher priority. Outputs
     must be bit-exact; the foreground latency is printed."""
