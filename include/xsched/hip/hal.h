@@ -81,6 +81,15 @@ XResult HipEventRecordCommandCreate(HwCommandHandle *cmd, void *event);
 /* hipStreamWaitEvent(event, flags) in queue order. reference hip_command.h:236-254 */
 XResult HipEventWaitCommandCreate(HwCommandHandle *cmd, void *event, uint32_t flags);
 
+/* Wait, in queue order, until the event-record command `record_cmd` of ANOTHER XQueue has
+ * completed. `record_cmd` must still be owned by the caller (create this command BEFORE
+ * submitting the record command; NotFound otherwise) and must come from
+ * HipEventRecordCommandCreate (InvalidValue otherwise). The wait happens on the host, on the
+ * launch thread of the waiting XQueue, and follows the record command through level-2
+ * flushes and replays of its queue. reference hip_command.h:240-241, hip_command.cpp:174-177,
+ * shim.cpp:242-244 */
+XResult HipRecordedEventWaitCommandCreate(HwCommandHandle *cmd, HwCommandHandle record_cmd);
+
 /* hipLaunchKernel of an arbitrary kernel. `args[i]` points to argument i of
  * `arg_sizes[i]` bytes; the values are copied at creation (the reference gets the
  * sizes from code-object metadata instead: hip_command.cpp:53-73,

@@ -183,3 +183,53 @@ def test_null_stream_and_bad_arguments(xs, gpu):
     assert h.HipHistogramCommandCreate(byref(cmd), 16, 4, 16, 70000, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, None, None, 4, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, 16, 16, 4, 4) == xs.kXSchedErrorInvalidValue
+
+
+def test_cross_queue_wait_on_recorded_event_follows_replays(xs, gpu):
+    """Queue B waits for an event-record command of queue A, which runs at level 2 and is
+    suspended and resumed all the time: B's kernel, which reads A's output, must see it
+    complete, i.e. the wait must follow A's flushes and replays rather than the raw event."""
+    import ctypes
+    torch = gpu
+    hip = ctypes.CDLL("libamdhip64.so")
+    event = ctypes.c_void_p()
+    assert hip.hipEventCreateWithFlags(byref(event), 2) == 0  # hipEventDisableTiming
+    n, times = 1 << 24, 40
+    print(f"case cross-queue-wait n={n} times={times}", flush=True)
+    xa_h = oracle.fill_uniform(21, 1, 0, n); ya_h = oracle.fill_uniform(21, 2, 0, n)
+    yb_h = oracle.fill_uniform(21, 3, 0, n)
+    xa = torch.from_numpy(xa_h).cuda(); ya = torch.from_numpy(ya_h.copy()).cuda()
+    yb = torch.from_numpy(yb_h.copy()).cuda()
+    qa = Queue(xs, torch, level=2, threshold=4, batch=2)
+    qb = Queue(xs, torch, level=1)
+    h = xs.halhip()
+
+    record, wait = c_uint64(), c_uint64()
+    xs.check(h.HipEventRecordCommandCreate(byref(record), event))
+    xs.check(h.HipRecordedEventWaitCommandCreate(byref(wait), record.value))
+    assert h.HipRecordedEventWaitCommandCreate(byref(c_uint64()), 0x1234) == xs.kXSchedErrorNotFound
+
+    # B first: its launch thread has to wait for a command that is not even submitted yet.
+    qb.submit(wait.value)
+    qb.submit(axpy_cmd(xs, 1.0, ya, yb, n, 0))          # yb += ya, once A is done
+    time.sleep(0.01)
+    stop = threading.Event()
+    t = threading.Thread(target=churn, args=(xs, qa, stop, 9))
+    t.start()
+    for _ in range(times):
+        qa.submit(axpy_cmd(xs, 0.5, xa, ya, n, 1))
+    qa.submit(record.value)
+    qb.wait()                                            # returns only after A's work
+    stop.set()
+    t.join()
+    qa.wait()
+    st = hip_stats(xs, qa.hwq)
+    got_a, got_b = ya.cpu().numpy(), yb.cpu().numpy()
+    qa.close(); qb.close()
+    assert hip.hipEventDestroy(event) == 0
+    want_a = oracle.axpy(0.5, xa_h, ya_h, times)
+    want_b = oracle.axpy(1.0, want_a, yb_h, 1)
+    print("stats", st, flush=True)
+    assert st[2] > 0, "queue A was never deactivated: the test did not exercise level 2"
+    assert np.array_equal(got_a.view(np.uint32), want_a.view(np.uint32))
+    assert np.array_equal(got_b.view(np.uint32), want_b.view(np.uint32)), "B ran before A had finished"

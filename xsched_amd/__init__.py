@@ -102,6 +102,7 @@ HALHIP_API = {
     "HipMemsetCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_int, c_size_t]),
     "HipEventRecordCommandCreate": (XResult, [POINTER(c_uint64), c_void_p]),
     "HipEventWaitCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32]),
+    "HipRecordedEventWaitCommandCreate": (XResult, [POINTER(c_uint64), c_uint64]),
     "HipKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32,
                                          c_uint32, c_uint32, c_uint32, POINTER(c_void_p),
                                          POINTER(c_size_t), c_size_t, c_uint32]),

@@ -65,6 +65,31 @@ private:
     hipEvent_t event_; unsigned flags_;
 };
 
+// Cross-queue ordering against an event-record COMMAND of another XQueue (what the
+// interception shim builds for hipStreamWaitEvent on an event it has seen recorded:
+// reference hip_command.h:236-254, hip_command.cpp:174-184, shim.cpp:216-246). The wait is
+// on the host, in BeforeLaunch(), and on the record command's COMPLETION as the XQueue that
+// owns it reports it, not on the raw event: after a level-2 flush the raw event signals
+// although the work in front of it was only flushed, while the owning XQueue repeats that
+// wait after the replay. Until the record command has been submitted there is nothing to
+// wait on, so that comes first. Nothing is enqueued on the stream.
+class HipRecordedEventWaitCommand final : public HipCommand
+{
+public:
+    explicit HipRecordedEventWaitCommand(std::shared_ptr<HwCommand> record)
+        : HipCommand(kCommandPropertyIdempotent), record_(std::move(record)) {}
+    virtual void BeforeLaunch() override
+    {
+        record_->WaitUntil(kCommandStatePending);
+        record_->Wait();
+    }
+    virtual bool DirectLaunchable() override { return false; } // BeforeLaunch() blocks
+protected:
+    virtual hipError_t Enqueue(HipQueue &, bool) override { return hipSuccess; }
+private:
+    const std::shared_ptr<HwCommand> record_;
+};
+
 // Arguments are copied at creation, so the caller's storage may go away before the
 // launch thread gets to the command.
 class HipKernelCommand final : public HipCommand
@@ -126,6 +151,16 @@ EXPORT_C_FUNC XResult HipEventWaitCommandCreate(HwCommandHandle *cmd, void *even
 {
     if (cmd == nullptr || event == nullptr) return kXSchedErrorInvalidValue;
     *cmd = HwCommandManager::Add(std::make_shared<HipEventWaitCommand>((hipEvent_t)event, flags));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipRecordedEventWaitCommandCreate(HwCommandHandle *cmd, HwCommandHandle record_cmd)
+{
+    if (cmd == nullptr) return kXSchedErrorInvalidValue;
+    auto record = HwCommandManager::Get(record_cmd);
+    if (record == nullptr) return kXSchedErrorNotFound;
+    if (dynamic_cast<HipEventRecordCommand *>(record.get()) == nullptr) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipRecordedEventWaitCommand>(std::move(record)));
     return kXSchedSuccess;
 }
 
