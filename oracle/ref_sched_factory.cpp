@@ -1,4 +1,4 @@
-// ORACLE - test infrastructure only; compiled ONLY into oracle/_ref/libxqueue_ref.so.
+// ORACLE - test infrastructure only; compiled ONLY into the libraries under oracle/_ref/.
 //
 // The reference's XQueue core is compiled from its own sources for the launch-trace
 // oracle. Two of its files, sched/src/scheduler/scheduler.cpp and global.cpp, include the

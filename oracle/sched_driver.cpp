@@ -1,5 +1,5 @@
 // ORACLE - test infrastructure only. A C interface over XSched's scheduling classes
-// (Policy, Status, Hint / Event / Operation records, name tables). The SAME source is
+// (Policy, LocalScheduler, Status, Hint / Event / Operation records, name tables). The SAME source is
 // compiled twice:
 //   * against the reference's own headers and sources under /root/reference
 //     (oracle/_ref/libsched_ref.so, symbols ref_*), and
@@ -12,6 +12,7 @@
 #include <cstring>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -23,6 +24,7 @@
 #include "xsched/sched/protocol/hint.h"
 #include "xsched/sched/protocol/operation.h"
 #include "xsched/sched/protocol/status.h"
+#include "xsched/sched/scheduler/local.h"
 
 #ifndef DRV_PREFIX
 #error "define DRV_PREFIX (ref_ or probe_)"
@@ -139,6 +141,14 @@ DRV_EXPORT size_t DRV(bytes_hint_laxity)(uint64_t xq, int64_t lax, int lp, int c
 DRV_EXPORT size_t DRV(bytes_event_hint_priority)(uint64_t xq, int prio, void *out, size_t cap)
 { HintEvent e(std::make_shared<PriorityHint>(xq, prio)); return CopyOut(e.Data(), e.Size(), out, cap); }
 
+DRV_EXPORT size_t DRV(bytes_event_hint)(const void *hint_bytes, void *out, size_t cap)
+{
+    auto hint = Hint::CopyConstructor(hint_bytes);
+    if (hint == nullptr) return 0;
+    HintEvent e(hint);
+    return CopyOut(e.Data(), e.Size(), out, cap);
+}
+
 DRV_EXPORT size_t DRV(bytes_event_process_create)(const char *cmdline, void *out, size_t cap)
 { ProcessCreateEvent e{std::string(cmdline)}; return CopyOut(e.Data(), e.Size(), out, cap); }
 
@@ -201,6 +211,69 @@ DRV_EXPORT size_t DRV(operation_roundtrip)(const void *in, void *out, size_t cap
 {
     auto op = Operation::CopyConstructor(in);
     return op ? CopyOut(op->Data(), op->Size(), out, cap) : 0;
+}
+
+// ---- local scheduler ------------------------------------------------------------
+// The whole LocalScheduler (event queue, worker thread, Status mirror, operation ids)
+// driven through its public interface only. Events go in as wire bytes, so a test can
+// set any process id; every operation the scheduler hands to its executor is kept as
+// wire bytes, in order.
+
+namespace
+{
+
+struct LocalBox
+{
+    std::unique_ptr<LocalScheduler> sched;
+    std::mutex mtx;
+    std::vector<std::vector<char>> ops;
+};
+
+} // namespace
+
+DRV_EXPORT void *DRV(local_create)(int policy)
+{
+    auto *box = new LocalBox();
+    box->sched = std::make_unique<LocalScheduler>((XPolicyType)policy);
+    box->sched->SetExecutor([box](std::shared_ptr<const Operation> op) {
+        const char *bytes = (const char *)op->Data();
+        std::lock_guard<std::mutex> lock(box->mtx);
+        box->ops.emplace_back(bytes, bytes + op->Size());
+    });
+    return box;
+}
+
+DRV_EXPORT void DRV(local_destroy)(void *b) { delete (LocalBox *)b; }
+DRV_EXPORT void DRV(local_run)(void *b) { ((LocalBox *)b)->sched->Run(); }
+DRV_EXPORT void DRV(local_stop)(void *b) { ((LocalBox *)b)->sched->Stop(); }
+DRV_EXPORT void DRV(local_set_policy)(void *b, int policy) { ((LocalBox *)b)->sched->SetPolicy((XPolicyType)policy); }
+
+DRV_EXPORT int DRV(local_recv_event)(void *b, const void *bytes)
+{
+    auto event = Event::CopyConstructor(bytes);
+    if (event == nullptr) return 0;
+    ((LocalBox *)b)->sched->RecvEvent(event);
+    return 1;
+}
+
+/// Moves the recorded operations out as [uint64 size][bytes]... Returns the bytes
+/// needed; nothing is consumed when `cap` is too small.
+DRV_EXPORT size_t DRV(local_take_operations)(void *b, void *out, size_t cap)
+{
+    auto *box = (LocalBox *)b;
+    std::lock_guard<std::mutex> lock(box->mtx);
+    size_t need = 0;
+    for (auto &op : box->ops) need += sizeof(uint64_t) + op.size();
+    if (out == nullptr || need > cap) return need;
+    char *dst = (char *)out;
+    for (auto &op : box->ops) {
+        const uint64_t size = op.size();
+        memcpy(dst, &size, sizeof(size));
+        memcpy(dst + sizeof(size), op.data(), op.size());
+        dst += sizeof(size) + op.size();
+    }
+    box->ops.clear();
+    return need;
 }
 
 // ---- names and devices ----------------------------------------------------------

@@ -2,6 +2,7 @@
 sources, probe_* over this repository's classes). Test helper."""
 import ctypes
 import os
+import struct
 from ctypes import (POINTER, c_char_p, c_int, c_int8, c_int64, c_size_t, c_uint8, c_uint32, c_uint64,
                     c_void_p)
 
@@ -82,6 +83,17 @@ class SchedDriver:
         n = f(data, buf, 4096)
         return buf.raw[:n]
 
+    def hint_event(self, hint_bytes):
+        f = self.fn("bytes_event_hint", c_size_t, [c_char_p, c_void_p, c_size_t])
+        buf = ctypes.create_string_buffer(1024)
+        n = f(hint_bytes, buf, 1024)
+        assert 0 < n <= 1024
+        return buf.raw[:n]
+
+    # ---- local scheduler ----
+    def local(self, ptype):
+        return _Local(self, ptype)
+
     # ---- names ----
     def policy_type_by_name(self, name):
         return self.fn("policy_type_by_name", c_int, [c_char_p])(name.encode())
@@ -155,6 +167,68 @@ class _Policy:
         timers = (c_int64 * 16)()
         nt = f(self.h, n, h, d, r, t, dec, timers, 16)
         return list(dec), list(timers)[:min(nt, 16)]
+
+
+def with_pid(event_bytes, pid):
+    """The same event as sent by process `pid` (EventMeta is {int32 type, int32 pid})."""
+    return event_bytes[:4] + struct.pack("<i", pid) + event_bytes[8:]
+
+
+def parse_sched_operation(data):
+    """(id, type, pid, running list, suspended list) of a SchedOperation's wire bytes:
+    {uint64 id, int32 type, int32 pid, uint64 size, uint64 running_cnt,
+    uint64 suspended_cnt, uint64 handles[]}."""
+    op_id, op_type, pid, size, n_run, n_sus = struct.unpack_from("<QiiQQQ", data)
+    assert size == len(data) == 40 + 8 * (n_run + n_sus)
+    handles = struct.unpack_from("<%dQ" % (n_run + n_sus), data, 40)
+    return op_id, op_type, pid, list(handles[:n_run]), list(handles[n_run:])
+
+
+class _Local:
+    """A LocalScheduler whose executor records operations."""
+
+    def __init__(self, drv, ptype):
+        self.drv = drv
+        self.h = drv.fn("local_create", c_void_p, [c_int])(ptype)
+
+    def close(self):
+        self.drv.fn("local_destroy", None, [c_void_p])(self.h)
+
+    def run(self):
+        self.drv.fn("local_run", None, [c_void_p])(self.h)
+
+    def stop(self):
+        self.drv.fn("local_stop", None, [c_void_p])(self.h)
+
+    def set_policy(self, ptype):
+        self.drv.fn("local_set_policy", None, [c_void_p, c_int])(self.h, ptype)
+
+    def recv(self, event_bytes):
+        assert self.drv.fn("local_recv_event", c_int, [c_void_p, c_char_p])(self.h, event_bytes) == 1
+
+    def take(self):
+        """Wire bytes of the operations executed since the last call, in order."""
+        f = self.drv.fn("local_take_operations", c_size_t, [c_void_p, c_void_p, c_size_t])
+        need = f(self.h, None, 0)
+        buf = ctypes.create_string_buffer(max(1, need))
+        assert f(self.h, buf, need) == need
+        ops, off = [], 0
+        while off < need:
+            (size,) = struct.unpack_from("<Q", buf.raw, off)
+            ops.append(buf.raw[off + 8:off + 8 + size])
+            off += 8 + size
+        return ops
+
+    def round(self, events):
+        """Exactly one scheduling round over `events`: they are queued while no worker
+        runs, followed by a terminate event, so the worker that is then started folds
+        all of them into the status, runs the policy once, executes and exits."""
+        for e in events:
+            self.recv(e)
+        self.recv(self.drv.record("event_terminate"))
+        self.run()
+        self.stop()
+        return self.take()
 
 
 def masked(name, data):
