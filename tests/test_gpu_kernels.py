@@ -102,12 +102,26 @@ def test_axpy_general_alpha_and_unaligned(xs, gpu):
     assert got[0] == y_before[0]
 
 
+@pytest.fixture(params=["sweep", "merge"])
+def hist_layout(request, monkeypatch):
+    """The histogram merges its per-group counts in one of two ways, chosen by the number
+    of keys when the command is created: an atomic sweep by the counting kernel itself
+    (small inputs) or packed partial histograms summed by a second kernel (2^25 keys and
+    more). "merge" forces the second one at every size."""
+    if request.param == "merge":
+        monkeypatch.setenv("XSCHED_HIP_HIST_MERGE_MIN_KEYS", "1")
+    else:
+        monkeypatch.setenv("XSCHED_HIP_HIST_MERGE_MIN_KEYS", str(1 << 40))
+    return request.param
+
+
 @pytest.mark.parametrize("n,n_bins", [(0, 65536), (1, 65536), (1000, 65536), (65536 + 13, 65536),
-                                      (1 << 20, 65536), (300000, 1000), (5000, 7)])
+                                      (1 << 20, 65536), (300000, 1000), (5000, 7), (70000, 32769),
+                                      (4096 * 300 + 1, 65535)])
 @pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
-def test_histogram_bit_exact(xs, gpu, n, n_bins, level, guard):
+def test_histogram_bit_exact(xs, gpu, hist_layout, n, n_bins, level, guard):
     torch = gpu
-    print(f"case hist n={n} bins={n_bins} level={level} guard={guard}", flush=True)
+    print(f"case hist {hist_layout} n={n} bins={n_bins} level={level} guard={guard}", flush=True)
     table = oracle.zipf_table(n_bins)
     keys_h = oracle.fill_zipf(0, 1, 0, max(n, 1), table, n_bins)[:n]
     keys = torch.from_numpy(np.ascontiguousarray(keys_h) if n else np.zeros(1, np.int32)).cuda()
@@ -125,14 +139,14 @@ def test_histogram_bit_exact(xs, gpu, n, n_bins, level, guard):
 
 
 @pytest.mark.parametrize("n_bins,offset", [(65536, 0), (65536, 1), (1001, 0), (40000, 1)])
-def test_histogram_counters_wrap_independently(xs, gpu, n_bins, offset):
+def test_histogram_counters_wrap_independently(xs, gpu, hist_layout, n_bins, offset):
     """Bins that start just below 2^32 wrap on their own, as uint32 counters do in the
     oracle: the write-out adds two neighbouring counters with one 64-bit atomic and must
     take back a carry that leaks from the lower into the upper one. Also with a bins array
     that is only 4-byte aligned (offset 1), where the write-out uses 32-bit atomics."""
     torch = gpu
     n = (1 << 20) + 13
-    print(f"case hist-wrap bins={n_bins} offset={offset}", flush=True)
+    print(f"case hist-wrap {hist_layout} bins={n_bins} offset={offset}", flush=True)
     table = oracle.zipf_table(n_bins)
     keys_h = oracle.fill_zipf(3, 1, 0, n, table, n_bins)
     keys = torch.from_numpy(keys_h).cuda()
@@ -156,13 +170,13 @@ def test_histogram_counters_wrap_independently(xs, gpu, n_bins, offset):
 
 
 @pytest.mark.parametrize("lo,hi", [(32768, 65536), (0, 65536), (100, 101), (40000, 40003)])
-def test_histogram_any_distribution(xs, gpu, lo, hi):
+def test_histogram_any_distribution(xs, gpu, hist_layout, lo, hi):
     """Distributions the kernel is not tuned for: every key in the upper half of the key
     space (the on-chip list of such keys overflows and the work-group re-reads its chunk),
     uniform keys, one single bin, three neighbouring bins."""
     torch = gpu
     n = (1 << 22) + 5
-    print(f"case hist-dist [{lo},{hi})", flush=True)
+    print(f"case hist-dist {hist_layout} [{lo},{hi})", flush=True)
     keys_h = np.random.default_rng(lo).integers(lo, hi, n).astype(np.int32)
     keys = torch.from_numpy(keys_h).cuda()
     bins = torch.zeros(65536, dtype=torch.int32, device="cuda")
@@ -172,6 +186,42 @@ def test_histogram_any_distribution(xs, gpu, lo, hi):
     got = bins.cpu().numpy().view(np.uint32)
     q.close()
     assert np.array_equal(got, oracle.histogram(keys_h, 65536))
+
+
+@pytest.mark.parametrize("case", ["zipf", "one low bin", "one high bin", "both halves of a word", "ballot bin",
+                                  "half heavy"])
+def test_histogram_merge_layout_at_its_own_size(xs, gpu, case):
+    """2^25 keys take the two-kernel layout by themselves, 131072 keys per counting group.
+    Its 16-bit halves overflow when one bin takes 65536 keys of a group: the group must
+    notice and recount. "both halves of a word": bins 7232 and 40000 share a packed word."""
+    torch = gpu
+    n, n_bins = 1 << 25, 65536
+    print(f"case hist-merge {case}", flush=True)
+    rng = np.random.default_rng(11)
+    if case == "zipf":
+        keys_h = oracle.fill_zipf(5, 1, 0, n, oracle.zipf_table(n_bins), n_bins)
+    elif case == "one low bin":
+        keys_h = np.full(n, 100, np.int32)
+    elif case == "one high bin":
+        keys_h = np.full(n, 40000, np.int32)
+    elif case == "both halves of a word":
+        keys_h = np.where(rng.random(n) < 0.5, 7232, 40000).astype(np.int32)
+    elif case == "ballot bin":
+        keys_h = np.where(rng.random(n) < 0.9, 0, rng.integers(0, n_bins, n)).astype(np.int32)
+    else:
+        # groups in the first half of the array overflow, the others do not
+        keys_h = rng.integers(0, n_bins, n).astype(np.int32)
+        keys_h[:n // 2][rng.random(n // 2) < 0.7] = 12345
+    keys = torch.from_numpy(keys_h).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, 2)
+    q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+    q.submit(hist_cmd(xs, keys, n, bins, n_bins, 0))
+    q.wait()
+    got = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    want = oracle.histogram(keys_h, n_bins)
+    assert np.array_equal(got.astype(np.uint64), want.astype(np.uint64) * 2)
 
 
 def _gemm_case(xs, torch, a_bits, b_bits, M, N, K, level, guard):

@@ -66,10 +66,15 @@ def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags, guard):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-def test_histogram_preempt_resume_bit_exact(xs, gpu):
+@pytest.mark.parametrize("layout", ["sweep", "merge"])
+def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
+    """Both ways the histogram merges its per-group counts (see hist_layout in
+    test_gpu_kernels.py); in the second one a flushed launch leaves partial histograms in
+    the queue's scratch buffer for the replay."""
     torch = gpu
+    monkeypatch.setenv("XSCHED_HIP_HIST_MERGE_MIN_KEYS", "1" if layout == "merge" else str(1 << 40))
     n, n_bins, times = 1 << 24, 65536, 40
-    print(f"case hist-preempt n={n} times={times}", flush=True)
+    print(f"case hist-preempt {layout} n={n} times={times}", flush=True)
     table = oracle.zipf_table(n_bins)
     keys_h = oracle.fill_zipf(9, 1, 0, n, table, n_bins)
     keys = torch.from_numpy(keys_h).cuda()

@@ -139,6 +139,9 @@ public:
 
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) override final;
+    /// Called before every LaunchKernel() with the queue the command is launched on, for
+    /// commands that need something of the queue (its scratch buffer).
+    virtual hipError_t PrepareLaunch(HipQueue &) { return hipSuccess; }
     /// Launch the kernel. `guarded` selects the variant with the guard compiled in.
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) = 0;
 
@@ -174,6 +177,12 @@ public:
     hipStream_t Stream() const { return stream_; }
     XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }
     const std::shared_ptr<GuardState> &Guard() const { return guard_; }
+    /// Device memory of at least `bytes` that belongs to this queue until it is destroyed,
+    /// for kernels of its commands that pass data from one launch to the next. The
+    /// commands of a queue run in order, so they can share it; its contents survive a
+    /// deactivation. Grows by allocating anew (earlier buffers stay valid for launches
+    /// that already carry their address). Returns nullptr when the allocation fails.
+    void *Scratch(size_t bytes);
 
     // statistics (see HipQueueGetStats)
     std::atomic<uint64_t> n_launch { 0 }, n_replay { 0 }, n_deactivate { 0 }, n_reactivate { 0 };
@@ -186,6 +195,8 @@ private:
     std::atomic<XPreemptLevel> level_ { kPreemptLevelUnknown };
     std::shared_ptr<GuardState> guard_;
     hipStream_t op_stream_ = nullptr; // flag writes when the word lives in device memory
+    std::mutex scratch_mtx_;
+    std::vector<std::pair<void *, size_t>> scratch_; // last one is current
 };
 
 /// Microseconds a marker wait polls before it blocks in the driver.

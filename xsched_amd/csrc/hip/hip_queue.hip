@@ -277,6 +277,8 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
         g.done = slot_.done;
         g.gen = slot_.gen;
     }
+    hipError_t err = PrepareLaunch(q);
+    if (err != hipSuccess) return err;
     return LaunchKernel(q.Stream(), guarded, g);
 }
 
@@ -297,6 +299,7 @@ HipQueue::HipQueue(hipStream_t stream): stream_(stream)
 HipQueue::~HipQueue()
 {
     if (op_stream_) (void)hipStreamDestroy(op_stream_);
+    for (auto &buf : scratch_) (void)hipFree(buf.first);
 }
 
 void HipQueue::OnXQueueCreate() { HIP_ASSERT(hipSetDevice(device_)); }
@@ -331,6 +334,17 @@ private:
 };
 
 } // namespace
+
+void *HipQueue::Scratch(size_t bytes)
+{
+    std::lock_guard<std::mutex> lock(scratch_mtx_);
+    if (!scratch_.empty() && scratch_.back().second >= bytes) return scratch_.back().first;
+    DeviceScope scope(device_);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    scratch_.emplace_back(ptr, bytes);
+    return ptr;
+}
 
 void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
 {

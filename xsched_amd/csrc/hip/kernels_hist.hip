@@ -1,33 +1,53 @@
 // Guarded integer histogram for gfx950: bins[keys[i]] += 1, keys int32 in
 // [0, n_bins), n_bins <= 65536, bins uint32.
 //
-// The keys are read once (4 bytes per key); what bounds the kernel on MI355X is the
-// LDS atomic unit (a 64-lane ds_add on random addresses retires in ~38 cycles per
-// CU) and, before this layout, VALU issue: a wave64 vector instruction occupies its
-// SIMD for four cycles, so every compare per key counts.
+// The keys are read once (4 bytes per key). What bounds the kernel on MI355X besides
+// that read is the LDS atomic unit (a 64-lane ds_add on random addresses retires in
+// ~38 cycles per CU) and the merge of the per-group counts into the one result array:
+// device-wide atomic adds retire at ~90-110 G/s however they are arranged, and 256
+// groups times 65536 bins is a lot of them.
 //
 // One work-group of 1024 threads per compute unit owns a contiguous chunk of keys
 // (sized so that a launch has about one work-group per CU) and keeps everything it
-// counts on chip until the end:
-//   hot    keys < kHotBins: wave ballot + popcount into scalar registers. For skewed
-//          (Zipf-like) keys these few bins take a quarter of all keys and would
-//          otherwise serialise the LDS atomics of a wave on one address.
-//   main   keys < kLdsBins (32768): LDS-privatised 32-bit counters, 128 KiB.
-//   tail   keys >= kLdsBins: appended as 16-bit values to an LDS list (28 KiB), one
-//          list reservation per wave and iteration.
-// Only then does it touch global memory: a sweep of atomic adds over its non-zero
-// counters (a wave covers 256 consecutive bins, so the adds arrive line by line; each
-// group starts its sweep at a different segment because atomics on ONE cache line
-// retire at only ~0.1 G/s); then the same 128 KiB are cleared, the listed tail keys
-// are counted into them and swept out the same way (scattered global atomics, one per
-// tail key, retire at ~25 G/s device-wide: too slow). If the list overflows (an
-// adversarial distribution), the group re-reads its chunk for the tail keys instead.
+// counts on chip until the end. Keys < kHotBins are counted by wave ballot + popcount
+// into scalar registers: for skewed (Zipf-like) keys these few bins take a quarter of
+// all keys and would otherwise serialise the LDS atomics of a wave on one address.
+// The other keys go to LDS counters, in one of two layouts:
+//
+// Two kernels (kMerge; the layout in use up to 2^28 keys). 32768 LDS words hold all 65536 bins as 16-bit
+// halves: word w counts bin w in its low half and bin w + 32768 in its high half (a
+// hot low bin shares its word with a cold high one), one ds_add of 1 or 65536 per key.
+// The group then stores its words (128 KiB, plain coalesced stores) as one partial
+// histogram into a scratch buffer of the queue, and a second kernel sums the partials
+// (each of its groups reads a 512-byte column of every partial) and adds the totals to
+// the result with one 64-bit atomic per pair of bins. A half overflows only when one
+// bin outside the ballot bins takes 65536 keys of a chunk (at least a quarter of it).
+// Every overflow lowers the sum of all halves by at least 65534 and nothing raises it,
+// so "sum of halves == keys added" proves there was none; a group that fails the
+// test stores an all-zero partial and recounts its chunk the slow way (32-bit
+// counters, two passes over its keys, atomic sweep into the result).
+//
+// One kernel (above 2^28 keys, where the partials would need more than 128 MiB of
+// scratch, when the scratch buffer cannot be allocated, or on request through
+// XSCHED_HIP_HIST_MERGE_MIN_KEYS). The group keeps 32-bit counters for bins < 32768,
+// appends the rarer keys above that as 16-bit values to an LDS list (one list
+// reservation per wave and iteration), and merges by itself: a sweep of atomic adds
+// over its non-zero counters (a wave covers 256 consecutive bins, so the adds arrive
+// line by line; each group starts its sweep at a different segment because atomics on
+// ONE cache line retire at only ~0.1 G/s); then the same 128 KiB are cleared, the
+// listed keys are counted into them and swept out the same way. If the list
+// overflows (an adversarial distribution), the group re-reads its chunk for those
+// keys instead.
 //
 // Guard: entry check, and because a group has no side effects before its write-out,
 // every wave re-reads the preempt word every second iteration and the group abandons
 // itself (its progress byte stays untagged, a replay redoes the chunk). The write-out
-// runs to completion and commits. Integer adds commute, so the result does not depend
-// on the order in which work-groups (or replays) run.
+// runs to completion and commits. The groups of the merge kernel have progress bytes
+// of their own behind those of the counting groups, and run only when every counting
+// group has committed; the scratch buffer belongs to the queue, whose commands run in
+// order, so the partials of a flushed launch are still there for the replay. Integer
+// adds commute, so the result does not depend on the order in which work-groups (or
+// replays) run.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 
@@ -58,14 +78,23 @@ constexpr uint32_t kMaxChunk = 1u << 18;
 constexpr uint32_t kTargetGroups = 256;       // compute units of an MI355X
 constexpr uint32_t kSegBins = 256;            // bins one wave sweeps per step
 constexpr uint32_t kSegs = kLdsBins / kSegBins;
+// merge layout
+constexpr uint32_t kPartialWords = kLdsBins + 64;   // packed words, then the ballot bins' counts
+constexpr uint32_t kMergeGroups = 256;              // groups of the merge kernel
+constexpr uint32_t kMergeWords = kLdsBins / kMergeGroups;  // packed words per merge group (128)
+constexpr uint32_t kMaxPartials = 1024;
+constexpr uint64_t kMergeMinKeys = 1;             // the two-kernel layout wins at every size measured
+constexpr uint32_t kMergeMinChunk = 16384;        // fewer, fuller partials for small inputs
 
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-/// Keys per work-group for a histogram of n keys: a multiple of kMinChunk.
-inline uint32_t ChunkFor(uint64_t n)
+/// Keys per work-group for a histogram of n keys: a multiple of kMinChunk, at least
+/// `floor` (rounded up to one).
+inline uint32_t ChunkFor(uint64_t n, uint64_t floor = kMinChunk)
 {
     uint64_t c = (n + kTargetGroups - 1) / kTargetGroups;
+    if (c < floor) c = floor;
     c = (c + kMinChunk - 1) / kMinChunk * kMinChunk;
     if (c < kMinChunk) c = kMinChunk;
     if (c > kMaxChunk) c = kMaxChunk;
@@ -79,6 +108,9 @@ struct Shared
     uint32_t tail_count;
     uint32_t bailed;
     uint32_t guard_word;
+    uint32_t hot[kHotBins]; // merge layout: ballot counts of the whole group
+    uint32_t added;         // merge layout: keys added to the packed counters
+    uint32_t sum;           // merge layout: sum of all 16-bit halves
 };
 
 __device__ __forceinline__ void LdsAdd(uint32_t *p, uint32_t v)
@@ -163,10 +195,12 @@ __device__ __forceinline__ void ClearBins(Shared &sh)
     for (uint32_t i = threadIdx.x * 4; i < kLdsBins; i += kThreads * 4) *(u32x4 *)&sh.bins[i] = u32x4 { 0, 0, 0, 0 };
 }
 
-template <bool kGuard>
+/// kMerge: the group stores a packed partial histogram at partials + blockIdx.x *
+/// kPartialWords instead of adding its counts to bins itself (HistogramMergeKernel does).
+template <bool kGuard, bool kMerge>
 __global__ __launch_bounds__(kThreads)
 void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__restrict__ bins,
-                     uint32_t n_bins, uint32_t chunk, XGuardArgs g)
+                     uint32_t n_bins, uint32_t chunk, uint32_t *__restrict__ partials, XGuardArgs g)
 {
     __shared__ __attribute__((aligned(16))) Shared sh;
 
@@ -175,12 +209,30 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     const uint32_t lds_used = n_bins < kLdsBins ? n_bins : kLdsBins;
     // unsigned "k - lo < range" tests: one subtract and one compare per tier, and the
     // sentinel 0xFFFFFFFF of an absent key fails all of them
-    const uint32_t main_range = lds_used > kHotBins ? lds_used - kHotBins : 0;
-    const uint32_t tail_range = n_bins > kLdsBins ? n_bins - kLdsBins : 0;
+    const uint32_t main_range = kMerge ? (n_bins > kHotBins ? n_bins - kHotBins : 0)
+                                       : (lds_used > kHotBins ? lds_used - kHotBins : 0);
+    const uint32_t tail_range = !kMerge && n_bins > kLdsBins ? n_bins - kLdsBins : 0;
     XGuardBlock guard(g, blockIdx.x, &sh.guard_word);
 
     ClearBins(sh);
-    if (tid == 0) { sh.tail_count = 0; sh.bailed = 0; }
+    if (tid == 0) { sh.tail_count = 0; sh.bailed = 0; sh.added = 0; sh.sum = 0; }
+    if (tid < kHotBins) sh.hot[tid] = 0;
+
+    const uint64_t begin = (uint64_t)blockIdx.x * chunk;
+    const uint64_t end = begin + chunk < n ? begin + chunk : n;
+    const bool vec_ok = (((uintptr_t)keys) & 15) == 0; // chunk starts are multiples of 4 keys
+    const uint64_t full_end = vec_ok ? begin + (end - begin) / kIterKeys * kIterKeys : begin;
+
+    auto load_iter = [&](i32x4 *v, uint64_t base) {
+#pragma unroll
+        for (uint32_t u = 0; u < kUnits; ++u) {
+            v[u] = __builtin_nontemporal_load((const i32x4 *)(keys + base + ((uint64_t)u * kThreads + tid) * 4));
+        }
+    };
+    // The first keys are requested before the guard's uncached read of the preempt word, so
+    // that the two memory round trips overlap (reading keys has no side effect).
+    i32x4 a[kUnits], b[kUnits];
+    if (begin < full_end) load_iter(a, begin);
 
     if (kGuard) {
         if (!guard.Enter()) return; // Enter() contains the barrier that also publishes the cleared counters
@@ -188,13 +240,10 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
         __syncthreads();
     }
 
-    const uint64_t begin = (uint64_t)blockIdx.x * chunk;
-    const uint64_t end = begin + chunk < n ? begin + chunk : n;
-    const bool vec_ok = (((uintptr_t)keys) & 15) == 0; // chunk starts are multiples of 4 keys
-
     uint32_t hot[kHotBins];
 #pragma unroll
     for (uint32_t b = 0; b < kHotBins; ++b) hot[b] = 0;
+    uint32_t added = 0; // merge layout: keys this wave added to the packed counters
 
     // Lists the tail keys among k[0, count) one key vector at a time: one reservation for
     // the wave, each key placed by its rank among the wave's tail lanes of that vector.
@@ -230,9 +279,15 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
         for (uint32_t j = 0; j < kN; ++j) {
 #pragma unroll
             for (uint32_t b = 0; b < kHotBins; ++b) AddPopcount(hot[b], __ballot(k[j] == b));
-            if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j]], 1u);
+            if (kMerge) {
+                const bool counted = k[j] - kHotBins < main_range;
+                AddPopcount(added, __ballot(counted));
+                if (counted) LdsAdd(&sh.bins[k[j] & (kLdsBins - 1)], 1u + (k[j] >> 15) * 65535u);
+            } else {
+                if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j]], 1u);
+            }
         }
-        if (tail_range != 0) {
+        if (!kMerge && tail_range != 0) {
             // Tail keys are rare for skewed inputs, and VALU issue is what bounds this loop:
             // each thread first gathers its own tail keys (up to four 16-bit values in two
             // registers, newest in the low half of `lo`), then the wave places them with at
@@ -280,21 +335,11 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     using Units = std::integral_constant<uint32_t, kUnits>;
     using OneUnit = std::integral_constant<uint32_t, 1>;
 
-    auto load_iter = [&](i32x4 *v, uint64_t base) {
-#pragma unroll
-        for (uint32_t u = 0; u < kUnits; ++u) {
-            v[u] = __builtin_nontemporal_load((const i32x4 *)(keys + base + ((uint64_t)u * kThreads + tid) * 4));
-        }
-    };
-
     // Full iterations: plain 128-bit loads, two register sets so that the next
     // iteration's keys are in flight while this one's are counted.
     uint64_t base = begin;
     bool quit = false;
-    if (vec_ok) {
-        const uint64_t full_end = begin + (end - begin) / kIterKeys * kIterKeys;
-        i32x4 a[kUnits], b[kUnits];
-        if (base < full_end) load_iter(a, base);
+    {
         while (base < full_end) {
             const bool has_b = base + kIterKeys < full_end;
             if (has_b) load_iter(b, base + kIterKeys);
@@ -328,61 +373,220 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
         process(&v, OneUnit {});
     }
 
-    // Ballot counters are per wave: lane 0 of each wave folds them into the LDS counters.
+    // Ballot counters are per wave: lane 0 of each wave folds them into the group's.
     if (lane == 0) {
 #pragma unroll
         for (uint32_t b = 0; b < kHotBins; ++b) {
-            if (hot[b] != 0 && b < lds_used) LdsAdd(&sh.bins[b], hot[b]);
+            if (hot[b] == 0 || b >= lds_used) continue;
+            if (kMerge) LdsAdd(&sh.hot[b], hot[b]);
+            else        LdsAdd(&sh.bins[b], hot[b]);
         }
     }
+    if (kMerge && lane == 0) LdsAdd(&sh.added, added);
     __syncthreads();
 
     if (kGuard) {
-        // Last point without side effects: all waves agree on writing out or abandoning.
-        if (tid == 0) sh.guard_word = (sh.bailed == 0 && guard.WaveStillCurrent()) ? 1u : 0u;
-        __syncthreads();
-        if (sh.guard_word == 0) return;
+        // Last point without side effects: the group abandons if any of its waves saw a
+        // deactivation (the barrier above published their verdicts). The preempt word is
+        // not read again here: that round trip would sit exposed in front of every
+        // write-out, and a group that writes out just after a deactivation is no different
+        // from one that was a little further along.
+        if (sh.bailed != 0) return;
     }
 
     const uint32_t rot = (blockIdx.x * 37u) & (kSegs - 1);
-    SweepOut(sh, bins, lds_used, rot);
-
-    if (tail_range != 0) {
-        const uint32_t listed = sh.tail_count;
+    if (kMerge) {
+        uint32_t *part = partials + (size_t)blockIdx.x * kPartialWords;
+        uint32_t halves = 0;
+        for (uint32_t i = tid * 4; i < kLdsBins; i += kThreads * 4) {
+            const u32x4 w = *(const u32x4 *)&sh.bins[i];
+            *(u32x4 *)&part[i] = w;
+            halves += (w.x & 0xFFFFu) + (w.x >> 16) + (w.y & 0xFFFFu) + (w.y >> 16)
+                    + (w.z & 0xFFFFu) + (w.z >> 16) + (w.w & 0xFFFFu) + (w.w >> 16);
+        }
+        if (tid < 64) part[kLdsBins + tid] = tid < kHotBins ? sh.hot[tid] : 0u;
+        LdsAdd(&sh.sum, halves);
         __syncthreads();
-        ClearBins(sh);
-        __syncthreads();
-        if (listed <= kTailCap) {
-            for (uint32_t i = tid; i < listed; i += kThreads) LdsAdd(&sh.bins[sh.tail[i] - kLdsBins], 1u);
-        } else {
-            // The list overflowed: count the chunk's tail keys from memory instead.
-            for (uint64_t idx = begin + tid; idx < end; idx += kThreads) {
-                const uint32_t key = (uint32_t)keys[idx];
-                if (key - kLdsBins < tail_range) LdsAdd(&sh.bins[key - kLdsBins], 1u);
+        if (__builtin_amdgcn_readfirstlane(sh.sum) != __builtin_amdgcn_readfirstlane(sh.added)) {
+            // A 16-bit half overflowed: this group's partial counts nothing, and the chunk
+            // is counted again with 32-bit counters, one half of the bins at a time.
+            __syncthreads();
+            for (uint32_t i = tid * 4; i < kLdsBins; i += kThreads * 4) *(u32x4 *)&part[i] = u32x4 { 0, 0, 0, 0 };
+            if (tid < 64) part[kLdsBins + tid] = 0u;
+            for (uint32_t first = 0; first < n_bins; first += kLdsBins) {
+                const uint32_t count = n_bins - first < kLdsBins ? n_bins - first : kLdsBins;
+                ClearBins(sh);
+                __syncthreads();
+                for (uint64_t idx = begin + tid; idx < end; idx += kThreads) {
+                    const uint32_t key = (uint32_t)keys[idx];
+                    if (key - first < count) LdsAdd(&sh.bins[key - first], 1u);
+                }
+                __syncthreads();
+                SweepOut(sh, bins + first, count, rot);
+                __syncthreads();
             }
         }
-        __syncthreads();
-        SweepOut(sh, bins + kLdsBins, tail_range, rot);
+    } else {
+        SweepOut(sh, bins, lds_used, rot);
+
+        if (tail_range != 0) {
+            const uint32_t listed = sh.tail_count;
+            __syncthreads();
+            ClearBins(sh);
+            __syncthreads();
+            if (listed <= kTailCap) {
+                for (uint32_t i = tid; i < listed; i += kThreads) LdsAdd(&sh.bins[sh.tail[i] - kLdsBins], 1u);
+            } else {
+                // The list overflowed: count the chunk's tail keys from memory instead.
+                for (uint64_t idx = begin + tid; idx < end; idx += kThreads) {
+                    const uint32_t key = (uint32_t)keys[idx];
+                    if (key - kLdsBins < tail_range) LdsAdd(&sh.bins[key - kLdsBins], 1u);
+                }
+            }
+            __syncthreads();
+            SweepOut(sh, bins + kLdsBins, tail_range, rot);
+        }
     }
 
     if (kGuard) guard.Commit();
 }
 
+/// Sums the packed partial histograms of the counting groups and adds the totals to
+/// bins. Group j owns packed words [j * kMergeWords, (j + 1) * kMergeWords): thread
+/// (row, col) reads four of them from partials row, row + 32, ...; its progress byte is
+/// first_wg + j.
+template <bool kGuard>
+__global__ __launch_bounds__(kThreads)
+void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part, uint32_t *__restrict__ bins,
+                          uint32_t n_bins, uint32_t first_wg, XGuardArgs g)
+{
+    constexpr uint32_t kCols = kMergeWords / 4, kRows = kThreads / kCols; // 32 x 32
+    __shared__ uint32_t red[kRows][8][kCols];
+    __shared__ uint32_t total[2][kMergeWords];
+    __shared__ uint32_t hot_total[kHotBins];
+    __shared__ uint32_t guard_word;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t col = tid % kCols, row = tid / kCols;
+    const uint32_t word0 = blockIdx.x * kMergeWords + col * 4;
+    auto load_words = [&](uint32_t p) {
+        return p < n_part ? *(const u32x4 *)(partials + (size_t)p * kPartialWords + word0) : u32x4 { 0, 0, 0, 0 };
+    };
+    uint32_t acc[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+    auto add_words = [&](const u32x4 &w) {
+        acc[0] += w.x & 0xFFFFu; acc[1] += w.y & 0xFFFFu; acc[2] += w.z & 0xFFFFu; acc[3] += w.w & 0xFFFFu;
+        acc[4] += w.x >> 16;     acc[5] += w.y >> 16;     acc[6] += w.z >> 16;     acc[7] += w.w >> 16;
+    };
+    // The first eight rows are requested before the guard's uncached read of the preempt
+    // word: the kernel is short, and the round trips overlap. Reading has no side effect
+    // (after a flushed counting launch the words are stale, and nothing is done with them).
+    u32x4 first[8];
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) first[i] = load_words(row + i * kRows);
+
+    if (kGuard) {
+        // A flushed counting launch leaves partials missing; then this launch is flushed
+        // too (the preempt word only ever counts up), but make sure: every counting group
+        // must have committed. Their progress bytes are requested ahead of the guard too.
+        uint8_t tag[kMaxPartials / kThreads];
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) {
+            const uint32_t p = tid + i * kThreads;
+            tag[i] = g.done != nullptr && p < n_part ? __builtin_nontemporal_load(&g.done[p]) : (uint8_t)g.gen;
+        }
+        XGuardBlock guard(g, first_wg + blockIdx.x, &guard_word);
+        if (!guard.Enter()) return;
+        int all = 1;
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) all &= tag[i] == (uint8_t)g.gen;
+        if (!__syncthreads_and(all)) return;
+    }
+    if (tid < kHotBins) hot_total[tid] = 0;
+
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) add_words(first[i]);
+#pragma unroll 8
+    for (uint32_t p = row + 8 * kRows; p < n_part; p += kRows) add_words(load_words(p));
+#pragma unroll
+    for (uint32_t v = 0; v < 8; ++v) red[row][v][col] = acc[v];
+    __syncthreads();
+    if (blockIdx.x == 0) {
+        // the ballot bins' counts ride behind the packed words of every partial
+        for (uint32_t p = tid; p < n_part * kHotBins; p += kThreads) {
+            const uint32_t v = partials[(size_t)(p / kHotBins) * kPartialWords + kLdsBins + p % kHotBins];
+            if (v != 0) LdsAdd(&hot_total[p % kHotBins], v);
+        }
+    }
+    if (tid < 8 * kCols) {
+        const uint32_t v = tid / kCols, c = tid % kCols;
+        uint32_t t = 0;
+#pragma unroll
+        for (uint32_t r = 0; r < kRows; ++r) t += red[r][v][c];
+        total[v >> 2][c * 4 + (v & 3)] = t;
+    }
+    __syncthreads();
+
+    const bool pair_ok = (((uintptr_t)bins) & 7) == 0;
+    if (tid < kMergeWords) {
+        const uint32_t half = tid / (kMergeWords / 2), q = tid % (kMergeWords / 2);
+        const uint32_t bin = half * kLdsBins + blockIdx.x * kMergeWords + q * 2;
+        uint32_t lo = total[half][q * 2], hi = total[half][q * 2 + 1];
+        if (bin < kHotBins) lo += hot_total[bin];
+        if (bin + 1 < kHotBins) hi += hot_total[bin + 1];
+        if ((lo | hi) != 0) {
+            if (pair_ok && bin + 1 < n_bins) {
+                PairFix(bins + bin, PairAdd(bins + bin, lo, hi), lo);
+            } else {
+                if (lo != 0 && bin < n_bins) GlobalAdd(bins + bin, lo);
+                if (hi != 0 && bin + 1 < n_bins) GlobalAdd(bins + bin + 1, hi);
+            }
+        }
+    }
+    if (kGuard) {
+        XGuardBlock guard(g, first_wg + blockIdx.x, &guard_word);
+        guard.Commit();
+    }
+}
+
 class HipHistogramCommand final : public HipGuardedCommand
 {
 public:
+    /// n_count_wg counting groups; with `merge`, kMergeGroups merge groups follow them in
+    /// the progress map.
     HipHistogramCommand(const void *keys, size_t n, void *bins, uint32_t n_bins, uint32_t chunk,
-                        uint32_t n_wg, int guard_mode)
-        : HipGuardedCommand(n_wg, guard_mode)
-        , keys_((const int32_t *)keys), n_(n), bins_((uint32_t *)bins), n_bins_(n_bins), chunk_(chunk) {}
+                        uint32_t n_count_wg, bool merge, int guard_mode)
+        : HipGuardedCommand(n_count_wg + (merge ? kMergeGroups : 0), guard_mode)
+        , keys_((const int32_t *)keys), n_(n), bins_((uint32_t *)bins), n_bins_(n_bins), chunk_(chunk)
+        , n_count_wg_(n_count_wg), merge_(merge) {}
 
 protected:
+    virtual hipError_t PrepareLaunch(HipQueue &q) override
+    {
+        // A replay must find the partials of the flushed launch: keep the first buffer.
+        if (!merge_ || n_ == 0 || partials_ != nullptr) return hipSuccess;
+        partials_ = (uint32_t *)q.Scratch((size_t)n_count_wg_ * kPartialWords * sizeof(uint32_t));
+        // No scratch: the one-kernel layout works on the same chunks (decided before the
+        // first launch, so every replay takes the same path).
+        if (partials_ == nullptr) merge_ = false;
+        return hipSuccess;
+    }
+
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
     {
         if (n_ == 0) return hipSuccess;
-        const dim3 grid(n_wg_), block(kThreads);
-        if (guarded) hipLaunchKernelGGL(HistogramKernel<true>, grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, g);
-        else         hipLaunchKernelGGL(HistogramKernel<false>, grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, g);
+        const dim3 grid(n_count_wg_), block(kThreads);
+        if (!merge_) {
+            if (guarded) hipLaunchKernelGGL((HistogramKernel<true, false>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
+            else         hipLaunchKernelGGL((HistogramKernel<false, false>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
+            return hipGetLastError();
+        }
+        if (guarded) hipLaunchKernelGGL((HistogramKernel<true, true>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
+        else         hipLaunchKernelGGL((HistogramKernel<false, true>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return err;
+        const dim3 merge_grid(kMergeGroups);
+        if (guarded) hipLaunchKernelGGL(HistogramMergeKernel<true>, merge_grid, block, 0, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
+        else         hipLaunchKernelGGL(HistogramMergeKernel<false>, merge_grid, block, 0, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
         return hipGetLastError();
     }
 
@@ -392,7 +596,18 @@ private:
     uint32_t *bins_;
     const uint32_t n_bins_;
     const uint32_t chunk_;
+    const uint32_t n_count_wg_;
+    bool merge_;
+    uint32_t *partials_ = nullptr;
 };
+
+/// Keys from which the two-kernel layout is used (XSCHED_HIP_HIST_MERGE_MIN_KEYS).
+inline uint64_t MergeMinKeys()
+{
+    const char *env = getenv("XSCHED_HIP_HIST_MERGE_MIN_KEYS");
+    if (env == nullptr || *env == 0) return kMergeMinKeys;
+    return strtoull(env, nullptr, 0);
+}
 
 } // namespace hist
 
@@ -407,10 +622,19 @@ EXPORT_C_FUNC XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void
         return kXSchedErrorInvalidValue;
     }
     if (n_bins == 0 || n_bins > 65536) return kXSchedErrorInvalidValue;
-    const uint32_t chunk = hist::ChunkFor(n);
-    const uint64_t n_wg = n == 0 ? 1 : (n + chunk - 1) / chunk;
+    bool merge = n != 0 && n >= hist::MergeMinKeys();
+    const char *floor_env = getenv("XSCHED_HIP_HIST_MIN_CHUNK");
+    const uint64_t floor = floor_env && *floor_env ? strtoull(floor_env, nullptr, 0)
+                                                   : (merge ? hist::kMergeMinChunk : hist::kMinChunk);
+    uint32_t chunk = hist::ChunkFor(n, floor);
+    uint64_t n_wg = n == 0 ? 1 : (n + chunk - 1) / chunk;
+    if (merge && n_wg > hist::kMaxPartials) {
+        merge = false;
+        chunk = hist::ChunkFor(n);
+        n_wg = (n + chunk - 1) / chunk;
+    }
     if (n_wg > GuardState::kMaxWorkGroups) return kXSchedErrorInvalidValue;
     *cmd = HwCommandManager::Add(std::make_shared<hist::HipHistogramCommand>(
-        keys, n, bins, n_bins, chunk, (uint32_t)n_wg, guard));
+        keys, n, bins, n_bins, chunk, (uint32_t)n_wg, merge, guard));
     return kXSchedSuccess;
 }
