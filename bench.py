@@ -262,9 +262,10 @@ def config4(H, a):
     line["bg"] = {"alone_GBs_4_queues_side_by_side": 4 * hist_bytes(bg_n) / head["bg_alone_ms"] / 1e6,
                   "contended_GBs": hist_bytes(bg_n) * head["bg_cont_cmds"] / head["bg_cont_elapsed"] / 1e9}
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "HistogramKernel",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "HistogramKernel + HistogramMergeKernel",
                         "algorithmic_bytes_per_launch": hist_bytes(bg_n), "avg_launch_ms": per_launch_ms,
-                        "note": "one queue streaming the guarded kernel back to back"}
+                        "note": "one queue streaming guarded histogram commands back to back; a command is the "
+                                "counting kernel followed by the merge kernel, avg_launch_ms covers both"}
     if not a.quick:
         ms_plain = bg_ms_per_launch(H, H.HIST, bg_n, 1, 0, 20, 4)
         line["guard"] = {"plain_GBs": hist_bytes(bg_n) / ms_plain / 1e6, "level2_GBs": achieved,
