@@ -42,7 +42,13 @@
 // c in [0, flag_mask]. Uncached reads of ONE address are served one after the other by
 // a single memory channel (about 27 ns each on MI355X), which would cap a kernel at
 // some 37 M work-groups per second; work-group w reads copy (w & flag_mask), so the
-// reads spread over many channels. The host rewrites all copies on a deactivation.
+// reads spread over many channels. The host rewrites all copies on a deactivation, one
+// after the other: for the microseconds that takes, work-groups that read different
+// copies disagree. Each work-group decides for itself, so a single kernel is safe; a
+// kernel that needs ALL work-groups of an earlier launch must check their progress
+// bytes, and a command that reads what an earlier flushable command of its queue wrote
+// must map the data to work-groups (hence to copies) the same way, or be kept apart
+// from it by the caller.
 #define kXGuardFlagStrideWords 64u /* 256 bytes between copies */
 
 struct XGuardArgs
@@ -81,6 +87,24 @@ __device__ __forceinline__ uint32_t xguard_read_flag(const uint32_t *flag)
         __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
 #endif
     return v;
+}
+
+// The same read in two halves, for a loop that has other work to do while the word is
+// on its way: Begin() issues the load, End() hands out the value. This one is a VECTOR
+// load (every lane reads the same word, one memory request): vector loads return in
+// order and are counted apart from LDS operations, so the wait the compiler places in
+// front of End()'s use covers this load and older ones only. The scalar load above
+// shares its counter with LDS operations and returns out of order, so waiting for it
+// means waiting for every LDS atomic the wave has issued - which stalls a loop that
+// lives on having many of them in flight.
+__device__ __forceinline__ uint32_t xguard_read_flag_begin(const uint32_t *flag)
+{
+    return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__device__ __forceinline__ uint32_t xguard_read_flag_end(uint32_t v)
+{
+    return __builtin_amdgcn_readfirstlane(v);
 }
 
 __device__ __forceinline__ bool xguard_committed(const XGuardArgs &g, uint32_t wg)
@@ -161,6 +185,18 @@ public:
     __device__ __forceinline__ bool WaveStillCurrent() const
     {
         return xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+    }
+
+    /// WaveStillCurrent() split in two so that the read of the preempt word overlaps the
+    /// work between the calls: `pending = WavePollBegin(); ...; if (!WavePollEnd(pending))`.
+    __device__ __forceinline__ uint32_t WavePollBegin() const
+    {
+        return xguard_read_flag_begin(xguard_flag_copy(g_, wg_));
+    }
+
+    __device__ __forceinline__ bool WavePollEnd(uint32_t pending) const
+    {
+        return xguard_read_flag_end(pending) == g_.epoch;
     }
 
     /// Call after the last store of the work-group (all waves; one barrier inside).

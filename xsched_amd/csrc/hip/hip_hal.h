@@ -91,6 +91,30 @@ private:
     uint64_t in_use_ = 0;
 };
 
+/// Device buffers that commands of one queue borrow for data they pass from one of their
+/// kernels to the next (or from a flushed launch to its replay). A command takes a buffer
+/// at its first launch and gives it back when it is destroyed, i.e. after its last launch
+/// has left the device; buffers are recycled, never freed before the pool is. Commands in
+/// flight at the same time must not share one: the copies of the preempt word are written
+/// one after the other, so a work-group of a later command can still pass its entry
+/// check while an earlier command has already been flushed and needs its data for the replay.
+class ScratchPool
+{
+public:
+    explicit ScratchPool(int device): device_(device) {}
+    ~ScratchPool();
+    /// A buffer of at least `bytes`, or nullptr when the device has no memory for one.
+    void *Acquire(size_t bytes);
+    void Release(void *ptr);
+    size_t Buffers();
+
+private:
+    struct Buffer { void *ptr; size_t bytes; bool busy; };
+    const int device_;
+    std::mutex mtx_;
+    std::vector<Buffer> buffers_;
+};
+
 class HipQueue;
 
 class HipCommand : public preempt::HwCommand
@@ -177,12 +201,7 @@ public:
     hipStream_t Stream() const { return stream_; }
     XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }
     const std::shared_ptr<GuardState> &Guard() const { return guard_; }
-    /// Device memory of at least `bytes` that belongs to this queue until it is destroyed,
-    /// for kernels of its commands that pass data from one launch to the next. The
-    /// commands of a queue run in order, so they can share it; its contents survive a
-    /// deactivation. Grows by allocating anew (earlier buffers stay valid for launches
-    /// that already carry their address). Returns nullptr when the allocation fails.
-    void *Scratch(size_t bytes);
+    const std::shared_ptr<ScratchPool> &Scratch() const { return scratch_; }
 
     // statistics (see HipQueueGetStats)
     std::atomic<uint64_t> n_launch { 0 }, n_replay { 0 }, n_deactivate { 0 }, n_reactivate { 0 };
@@ -195,8 +214,7 @@ private:
     std::atomic<XPreemptLevel> level_ { kPreemptLevelUnknown };
     std::shared_ptr<GuardState> guard_;
     hipStream_t op_stream_ = nullptr; // flag writes when the word lives in device memory
-    std::mutex scratch_mtx_;
-    std::vector<std::pair<void *, size_t>> scratch_; // last one is current
+    std::shared_ptr<ScratchPool> scratch_;
 };
 
 /// Microseconds a marker wait polls before it blocks in the driver.

@@ -291,6 +291,7 @@ HipQueue::HipQueue(hipStream_t stream): stream_(stream)
     HIP_ASSERT(hipGetDeviceProperties(&prop, device_));
     xdevice_ = MakeDevice(kDeviceTypeGPU, MakePciId(prop.pciDomainID, prop.pciBusID, prop.pciDeviceID, 0));
     guard_ = std::make_shared<GuardState>(device_);
+    scratch_ = std::make_shared<ScratchPool>(device_);
     HIP_ASSERT(hipStreamCreateWithFlags(&op_stream_, hipStreamNonBlocking)); // default priority
     // Nothing of the application may still be running on the stream (hip_queue.cpp:35-36).
     HIP_ASSERT(hipStreamSynchronize(stream_));
@@ -299,7 +300,6 @@ HipQueue::HipQueue(hipStream_t stream): stream_(stream)
 HipQueue::~HipQueue()
 {
     if (op_stream_) (void)hipStreamDestroy(op_stream_);
-    for (auto &buf : scratch_) (void)hipFree(buf.first);
 }
 
 void HipQueue::OnXQueueCreate() { HIP_ASSERT(hipSetDevice(device_)); }
@@ -335,15 +335,38 @@ private:
 
 } // namespace
 
-void *HipQueue::Scratch(size_t bytes)
+ScratchPool::~ScratchPool()
 {
-    std::lock_guard<std::mutex> lock(scratch_mtx_);
-    if (!scratch_.empty() && scratch_.back().second >= bytes) return scratch_.back().first;
+    for (auto &buf : buffers_) (void)hipFree(buf.ptr);
+}
+
+void *ScratchPool::Acquire(size_t bytes)
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    Buffer *best = nullptr;
+    for (auto &buf : buffers_) {
+        if (!buf.busy && buf.bytes >= bytes && (best == nullptr || buf.bytes < best->bytes)) best = &buf;
+    }
+    if (best != nullptr) { best->busy = true; return best->ptr; }
     DeviceScope scope(device_);
     void *ptr = nullptr;
     if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    scratch_.emplace_back(ptr, bytes);
+    buffers_.push_back(Buffer { ptr, bytes, true });
     return ptr;
+}
+
+void ScratchPool::Release(void *ptr)
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    for (auto &buf : buffers_) {
+        if (buf.ptr == ptr) { buf.busy = false; return; }
+    }
+}
+
+size_t ScratchPool::Buffers()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    return buffers_.size();
 }
 
 void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)

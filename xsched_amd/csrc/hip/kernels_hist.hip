@@ -1,11 +1,12 @@
 // Guarded integer histogram for gfx950: bins[keys[i]] += 1, keys int32 in
 // [0, n_bins), n_bins <= 65536, bins uint32.
 //
-// The keys are read once (4 bytes per key). What bounds the kernel on MI355X besides
-// that read is the LDS atomic unit (a 64-lane ds_add on random addresses retires in
-// ~38 cycles per CU) and the merge of the per-group counts into the one result array:
-// device-wide atomic adds retire at ~90-110 G/s however they are arranged, and 256
-// groups times 65536 bins is a lot of them.
+// The keys are read once (4 bytes per key). Two things used to cost more than that read
+// on MI355X: the LDS atomics (a 64-lane ds_add on random addresses retires in ~38
+// cycles per CU; with 16 waves per CU they hide under the loads) and the merge of the
+// per-group counts into the one result array (device-wide atomic adds retire at
+// ~90-110 G/s however they are arranged, and 256 groups times 65536 bins is a lot of
+// them; hence the second kernel below).
 //
 // One work-group of 1024 threads per compute unit owns a contiguous chunk of keys
 // (sized so that a launch has about one work-group per CU) and keeps everything it
@@ -14,16 +15,19 @@
 // all keys and would otherwise serialise the LDS atomics of a wave on one address.
 // The other keys go to LDS counters, in one of two layouts:
 //
-// Two kernels (kMerge; the layout in use up to 2^28 keys). 32768 LDS words hold all 65536 bins as 16-bit
-// halves: word w counts bin w in its low half and bin w + 32768 in its high half (a
-// hot low bin shares its word with a cold high one), one ds_add of 1 or 65536 per key.
+// Two kernels (kMerge; the layout in use up to 2^28 keys). 32768 LDS words hold all
+// 65536 bins as 16-bit halves: word w counts bin w in its low half and bin w + 32768 in its high half (a
+// hot low bin shares its word with a cold high one), one ds_add of 1 or 65536 per key
+// (without a branch: one vote per iteration tells whether every key of the wave is
+// below n_bins, and lanes that hold a ballot key add to a dummy word of their own).
 // The group then stores its words (128 KiB, plain coalesced stores) as one partial
-// histogram into a scratch buffer of the queue, and a second kernel sums the partials
+// histogram into a scratch buffer, and a second kernel sums the partials
 // (each of its groups reads a 512-byte column of every partial) and adds the totals to
 // the result with one 64-bit atomic per pair of bins. A half overflows only when one
 // bin outside the ballot bins takes 65536 keys of a chunk (at least a quarter of it).
 // Every overflow lowers the sum of all halves by at least 65534 and nothing raises it,
-// so "sum of halves == keys added" proves there was none; a group that fails the
+// so "sum of halves == keys that must be in the words" (all keys of the chunk minus the
+// ballot keys and the invalid ones) proves there was none; a group that fails the
 // test stores an all-zero partial and recounts its chunk the slow way (32-bit
 // counters, two passes over its keys, atomic sweep into the result).
 //
@@ -40,13 +44,15 @@
 // keys instead.
 //
 // Guard: entry check, and because a group has no side effects before its write-out,
-// every wave re-reads the preempt word every second iteration and the group abandons
+// every wave re-reads the preempt word every 32768 keys of the group and the group abandons
 // itself (its progress byte stays untagged, a replay redoes the chunk). The write-out
 // runs to completion and commits. The groups of the merge kernel have progress bytes
 // of their own behind those of the counting groups, and run only when every counting
-// group has committed; the scratch buffer belongs to the queue, whose commands run in
-// order, so the partials of a flushed launch are still there for the replay. Integer
-// adds commute, so the result does not depend on the order in which work-groups (or
+// group has committed; the scratch buffer is the command's own from its first launch
+// until it is destroyed, so the partials of a flushed launch are still there for the
+// replay (a later command of the queue must not write into them: its groups may pass
+// their entry check on a copy of the preempt word that has not been rewritten yet while
+// this command is already flushed). Integer adds commute, so the result does not depend on the order in which work-groups (or
 // replays) run.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
@@ -68,9 +74,17 @@ constexpr uint32_t kHotBins = XSCHED_HIST_HOT_BINS;
 constexpr uint32_t kLdsBins = 1u << 15;       // 128 KiB of counters
 constexpr uint32_t kTailCap = 14336;          // 16-bit entries, 28 KiB
 #ifndef XSCHED_HIST_UNITS
-#define XSCHED_HIST_UNITS 4
+#define XSCHED_HIST_UNITS 2
 #endif
 constexpr uint32_t kUnits = XSCHED_HIST_UNITS;  // 128-bit loads per thread and iteration
+#ifndef XSCHED_HIST_DEPTH
+#define XSCHED_HIST_DEPTH 2
+#endif
+constexpr uint32_t kDepth = XSCHED_HIST_DEPTH;  // iterations of keys in flight or being counted
+#ifndef XSCHED_HIST_POLL_TURNS
+#define XSCHED_HIST_POLL_TURNS 2
+#endif
+constexpr uint32_t kPollTurns = XSCHED_HIST_POLL_TURNS; // turns of the ring per look at the preempt word
 constexpr uint32_t kUnitKeys = kThreads * 4;
 constexpr uint32_t kIterKeys = kUnitKeys * kUnits;
 constexpr uint32_t kMinChunk = kUnitKeys;
@@ -109,8 +123,9 @@ struct Shared
     uint32_t bailed;
     uint32_t guard_word;
     uint32_t hot[kHotBins]; // merge layout: ballot counts of the whole group
-    uint32_t added;         // merge layout: keys added to the packed counters
+    uint32_t invalid;       // merge layout: keys outside [0, n_bins), absent ones included
     uint32_t sum;           // merge layout: sum of all 16-bit halves
+    uint32_t dummy[64];     // merge layout: where the lanes that hold a ballot key add
 };
 
 __device__ __forceinline__ void LdsAdd(uint32_t *p, uint32_t v)
@@ -215,7 +230,7 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     XGuardBlock guard(g, blockIdx.x, &sh.guard_word);
 
     ClearBins(sh);
-    if (tid == 0) { sh.tail_count = 0; sh.bailed = 0; sh.added = 0; sh.sum = 0; }
+    if (tid == 0) { sh.tail_count = 0; sh.bailed = 0; sh.invalid = 0; sh.sum = 0; }
     if (tid < kHotBins) sh.hot[tid] = 0;
 
     const uint64_t begin = (uint64_t)blockIdx.x * chunk;
@@ -227,12 +242,28 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 #pragma unroll
         for (uint32_t u = 0; u < kUnits; ++u) {
             v[u] = __builtin_nontemporal_load((const i32x4 *)(keys + base + ((uint64_t)u * kThreads + tid) * 4));
+            if (u + 1 < kUnits) asm volatile("" ::: "memory");
         }
     };
-    // The first keys are requested before the guard's uncached read of the preempt word, so
-    // that the two memory round trips overlap (reading keys has no side effect).
-    i32x4 a[kUnits], b[kUnits];
-    if (begin < full_end) load_iter(a, begin);
+    // A ring of kDepth register sets: the set just counted is refilled with the keys of
+    // kDepth iterations ahead. The first sets are requested before the guard's uncached
+    // read of the preempt word, so that the memory round trips overlap (reading keys has
+    // no side effect).
+    constexpr uint64_t kTurnKeys = (uint64_t)kDepth * kIterKeys;
+    constexpr uint64_t kLoopKeys = kTurnKeys * kPollTurns; // one trip of the main loop
+    const uint64_t turns_end = begin + (full_end - begin) / kLoopKeys * kLoopKeys;
+    i32x4 ring[kDepth][kUnits];
+    if (begin < turns_end) {
+        // Every set is loaded, no branch per set, and in the order in which the loop
+        // refills them (the empty statements keep the scheduler from permuting the loads:
+        // the loop's waits count on that order). A chunk shorter than one trip of the loop
+        // does not use it at all, so that these registers are written on this path only.
+#pragma unroll
+        for (uint32_t d = 0; d < kDepth; ++d) {
+            load_iter(ring[d], begin + (uint64_t)d * kIterKeys);
+            asm volatile("" ::: "memory");
+        }
+    }
 
     if (kGuard) {
         if (!guard.Enter()) return; // Enter() contains the barrier that also publishes the cleared counters
@@ -243,7 +274,7 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     uint32_t hot[kHotBins];
 #pragma unroll
     for (uint32_t b = 0; b < kHotBins; ++b) hot[b] = 0;
-    uint32_t added = 0; // merge layout: keys this wave added to the packed counters
+    uint32_t invalid = 0; // merge layout: keys of this thread outside [0, n_bins), absent ones included
 
     // Lists the tail keys among k[0, count) one key vector at a time: one reservation for
     // the wave, each key placed by its rank among the wave's tail lanes of that vector.
@@ -275,15 +306,37 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             k[u * 4 + 0] = (uint32_t)v[u].x; k[u * 4 + 1] = (uint32_t)v[u].y;
             k[u * 4 + 2] = (uint32_t)v[u].z; k[u * 4 + 3] = (uint32_t)v[u].w;
         }
+        if (kMerge) {
 #pragma unroll
-        for (uint32_t j = 0; j < kN; ++j) {
+            for (uint32_t j = 0; j < kN; ++j) {
 #pragma unroll
-            for (uint32_t b = 0; b < kHotBins; ++b) AddPopcount(hot[b], __ballot(k[j] == b));
-            if (kMerge) {
-                const bool counted = k[j] - kHotBins < main_range;
-                AddPopcount(added, __ballot(counted));
-                if (counted) LdsAdd(&sh.bins[k[j] & (kLdsBins - 1)], 1u + (k[j] >> 15) * 65535u);
+                for (uint32_t b = 0; b < kHotBins; ++b) AddPopcount(hot[b], __ballot(k[j] == b));
+            }
+            // Are all keys of the wave below n_bins (the usual case)? One max per key pair
+            // and one vote per iteration decide it; then every key is either a ballot key
+            // or counted, nothing has to be tallied per key, and the LDS add needs no
+            // branch: ballot keys add to a lane-private dummy word instead.
+            uint32_t largest = k[0];
+#pragma unroll
+            for (uint32_t j = 1; j < kN; ++j) largest = largest > k[j] ? largest : k[j];
+            if (__ballot(largest >= n_bins) == 0) {
+#pragma unroll
+                for (uint32_t j = 0; j < kN; ++j) {
+                    uint32_t *word = k[j] >= kHotBins ? &sh.bins[k[j] & (kLdsBins - 1)] : &sh.dummy[lane];
+                    LdsAdd(word, 1u + (k[j] >> 15) * 65535u);
+                }
             } else {
+#pragma unroll
+                for (uint32_t j = 0; j < kN; ++j) {
+                    if (k[j] >= n_bins) invalid += 1;
+                    if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j] & (kLdsBins - 1)], 1u + (k[j] >> 15) * 65535u);
+                }
+            }
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < kN; ++j) {
+#pragma unroll
+                for (uint32_t b = 0; b < kHotBins; ++b) AddPopcount(hot[b], __ballot(k[j] == b));
                 if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j]], 1u);
             }
         }
@@ -335,43 +388,64 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     using Units = std::integral_constant<uint32_t, kUnits>;
     using OneUnit = std::integral_constant<uint32_t, 1>;
 
-    // Full iterations: plain 128-bit loads, two register sets so that the next
-    // iteration's keys are in flight while this one's are counted.
-    uint64_t base = begin;
-    bool quit = false;
-    {
-        while (base < full_end) {
-            const bool has_b = base + kIterKeys < full_end;
-            if (has_b) load_iter(b, base + kIterKeys);
-            process(a, Units {});
-            base += kIterKeys;
-            if (!has_b) break;
-            const bool has_a = base + kIterKeys < full_end;
-            if (has_a) load_iter(a, base + kIterKeys);
-            process(b, Units {});
-            base += kIterKeys;
-            if (kGuard && !guard.WaveStillCurrent()) {
-                if (lane == 0) sh.bailed = 1;
-                quit = true;
-                break;
+    // Counts the chunk; false when the wave saw a deactivation and gave up.
+    //
+    // Full iterations go through the ring. Whole turns of it run without a branch around
+    // their loads (a refill that would start beyond the last full iteration re-reads that
+    // one instead, unused), so the compiler can count exactly how many loads may still be
+    // in flight where it needs one of them. The preempt word is requested at the start of
+    // a trip of the loop (kPollTurns turns) and looked at at its end: by then the refills
+    // issued behind it are the only loads it does not wait for.
+    auto count_chunk = [&]() -> bool {
+        uint64_t base = begin;
+        if (base < turns_end) {
+            do {
+                const uint32_t polled = kGuard ? guard.WavePollBegin() : 0u;
+#pragma unroll
+                for (uint32_t t = 0; t < kPollTurns; ++t) {
+#pragma unroll
+                    for (uint32_t d = 0; d < kDepth; ++d) {
+                        process(ring[d], Units {});
+                        const uint64_t next = base + (uint64_t)d * kIterKeys + kTurnKeys;
+                        load_iter(ring[d], next < full_end ? next : full_end - kIterKeys);
+                    }
+                    base += kTurnKeys;
+                }
+                if (kGuard && !guard.WavePollEnd(polled)) return false;
+            } while (base < turns_end);
+            // fewer than kDepth full iterations are left, and their keys are in the ring already
+#pragma unroll
+            for (uint32_t d = 0; d < kDepth; ++d) {
+                if (base < full_end) {
+                    process(ring[d], Units {});
+                    base += kIterKeys;
+                }
             }
         }
-    }
-    // Ragged remainder (and unaligned key arrays): one unit at a time, absent keys read
-    // as the sentinel.
-    for (; !quit && base < end; base += kUnitKeys) {
-        const uint64_t idx = base + (uint64_t)tid * 4;
-        i32x4 v = { -1, -1, -1, -1 };
-        if (vec_ok && idx + 3 < end) {
-            v = __builtin_nontemporal_load((const i32x4 *)(keys + idx));
-        } else {
-            if (idx + 0 < end) v.x = keys[idx + 0];
-            if (idx + 1 < end) v.y = keys[idx + 1];
-            if (idx + 2 < end) v.z = keys[idx + 2];
-            if (idx + 3 < end) v.w = keys[idx + 3];
+        // what a chunk has beyond whole trips of the loop and the ring: one iteration at a time
+        for (; base < full_end; base += kIterKeys) {
+            i32x4 v[kUnits];
+            load_iter(v, base);
+            process(v, Units {});
         }
-        process(&v, OneUnit {});
-    }
+        // Ragged remainder (and unaligned key arrays): one unit at a time, absent keys read
+        // as the sentinel.
+        for (; base < end; base += kUnitKeys) {
+            const uint64_t idx = base + (uint64_t)tid * 4;
+            i32x4 v = { -1, -1, -1, -1 };
+            if (vec_ok && idx + 3 < end) {
+                v = __builtin_nontemporal_load((const i32x4 *)(keys + idx));
+            } else {
+                if (idx + 0 < end) v.x = keys[idx + 0];
+                if (idx + 1 < end) v.y = keys[idx + 1];
+                if (idx + 2 < end) v.z = keys[idx + 2];
+                if (idx + 3 < end) v.w = keys[idx + 3];
+            }
+            process(&v, OneUnit {});
+        }
+        return true;
+    };
+    if (!count_chunk() && lane == 0) sh.bailed = 1;
 
     // Ballot counters are per wave: lane 0 of each wave folds them into the group's.
     if (lane == 0) {
@@ -382,7 +456,7 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             else        LdsAdd(&sh.bins[b], hot[b]);
         }
     }
-    if (kMerge && lane == 0) LdsAdd(&sh.added, added);
+    if (kMerge && invalid != 0) LdsAdd(&sh.invalid, invalid);
     __syncthreads();
 
     if (kGuard) {
@@ -407,7 +481,13 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
         if (tid < 64) part[kLdsBins + tid] = tid < kHotBins ? sh.hot[tid] : 0u;
         LdsAdd(&sh.sum, halves);
         __syncthreads();
-        if (__builtin_amdgcn_readfirstlane(sh.sum) != __builtin_amdgcn_readfirstlane(sh.added)) {
+        // every key slot the group went through (absent keys of the ragged end included) is
+        // a ballot key, an invalid one, or in the words
+        uint32_t expected = (uint32_t)(full_end - begin)
+                          + (uint32_t)((end - full_end + kUnitKeys - 1) / kUnitKeys) * kUnitKeys - sh.invalid;
+#pragma unroll
+        for (uint32_t b = 0; b < kHotBins; ++b) expected -= sh.hot[b];
+        if (__builtin_amdgcn_readfirstlane(sh.sum) != __builtin_amdgcn_readfirstlane(expected)) {
             // A 16-bit half overflowed: this group's partial counts nothing, and the chunk
             // is counted again with 32-bit counters, one half of the bins at a time.
             __syncthreads();
@@ -558,13 +638,16 @@ public:
         : HipGuardedCommand(n_count_wg + (merge ? kMergeGroups : 0), guard_mode)
         , keys_((const int32_t *)keys), n_(n), bins_((uint32_t *)bins), n_bins_(n_bins), chunk_(chunk)
         , n_count_wg_(n_count_wg), merge_(merge) {}
+    virtual ~HipHistogramCommand() { if (partials_ != nullptr) pool_->Release(partials_); }
 
 protected:
     virtual hipError_t PrepareLaunch(HipQueue &q) override
     {
-        // A replay must find the partials of the flushed launch: keep the first buffer.
+        // A replay must find the partials of the flushed launch: the buffer taken at the
+        // first launch is kept until the command is destroyed.
         if (!merge_ || n_ == 0 || partials_ != nullptr) return hipSuccess;
-        partials_ = (uint32_t *)q.Scratch((size_t)n_count_wg_ * kPartialWords * sizeof(uint32_t));
+        pool_ = q.Scratch();
+        partials_ = (uint32_t *)pool_->Acquire((size_t)n_count_wg_ * kPartialWords * sizeof(uint32_t));
         // No scratch: the one-kernel layout works on the same chunks (decided before the
         // first launch, so every replay takes the same path).
         if (partials_ == nullptr) merge_ = false;
@@ -598,6 +681,7 @@ private:
     const uint32_t chunk_;
     const uint32_t n_count_wg_;
     bool merge_;
+    std::shared_ptr<ScratchPool> pool_;
     uint32_t *partials_ = nullptr;
 };
 
