@@ -110,6 +110,7 @@ public:
 
 private:
     struct Buffer { void *ptr; size_t bytes; bool busy; };
+    static constexpr int kInitialBuffers = 3;
     const int device_;
     std::mutex mtx_;
     std::vector<Buffer> buffers_;

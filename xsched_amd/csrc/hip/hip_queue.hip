@@ -348,11 +348,19 @@ void *ScratchPool::Acquire(size_t bytes)
         if (!buf.busy && buf.bytes >= bytes && (best == nullptr || buf.bytes < best->bytes)) best = &buf;
     }
     if (best != nullptr) { best->busy = true; return best->ptr; }
+    // Nothing free: allocate for this command and, the first time, for the ones that will
+    // be in flight with it, so that a queue in steady state allocates nothing while its
+    // kernels run.
     DeviceScope scope(device_);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    buffers_.push_back(Buffer { ptr, bytes, true });
-    return ptr;
+    void *first = nullptr;
+    const int count = buffers_.empty() ? kInitialBuffers : 1;
+    for (int i = 0; i < count; ++i) {
+        void *ptr = nullptr;
+        if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
+        buffers_.push_back(Buffer { ptr, bytes, first == nullptr });
+        if (first == nullptr) first = ptr;
+    }
+    return first;
 }
 
 void ScratchPool::Release(void *ptr)
