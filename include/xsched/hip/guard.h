@@ -31,8 +31,8 @@
 // counter, so nothing has to be cleared or read back on resume; one byte per
 // work-group instead of two words.
 //
-// Cost: one uncached scalar load per work-group (hidden by the other resident
-// waves), one compare, and one byte store per work-group.
+// Cost: one uncached and one cached scalar load per work-group (hidden by the other
+// resident waves), two compares, and one byte store per work-group.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -44,11 +44,16 @@
 // some 37 M work-groups per second; work-group w reads copy (w & flag_mask), so the
 // reads spread over many channels. The host rewrites all copies on a deactivation, one
 // after the other: for the microseconds that takes, work-groups that read different
-// copies disagree. Each work-group decides for itself, so a single kernel is safe; a
-// kernel that needs ALL work-groups of an earlier launch must check their progress
-// bytes, and a command that reads what an earlier flushable command of its queue wrote
-// must map the data to work-groups (hence to copies) the same way, or be kept apart
-// from it by the caller.
+// copies disagree. Within one launch that is harmless, each work-group decides for
+// itself. Across launches it would let a work-group of a LATER launch run (its copy still
+// old) although a work-group of an EARLIER launch has been flushed (its copy already
+// new), and read what the flushed one has not written yet. The queue's `flushed` word
+// closes that: a work-group that finds its copy changed stores the epoch of its launch
+// there before it leaves, and every work-group also refuses to run when it finds its own
+// epoch in that word. The word lives in ordinary cached memory: what a launch stored is
+// visible to every later launch of the stream (kernel boundary), which is all that is
+// needed, and reading it costs a cache hit. A kernel that needs ALL work-groups of an
+// earlier launch (not just "none flushed") still has to check their progress bytes.
 #define kXGuardFlagStrideWords 64u /* 256 bytes between copies */
 
 struct XGuardArgs
@@ -59,6 +64,7 @@ struct XGuardArgs
     uint32_t        resume;    // nonzero: skip work-groups that have already committed
     uint32_t        flag_mask; // number of copies of the preempt word minus one (2^k - 1)
     uint32_t        gen;       // generation tag of this command in its progress map (1..255)
+    uint32_t       *flushed;   // the queue's "a work-group of this epoch was flushed" word; may be null
 };
 
 __device__ __forceinline__ const uint32_t *xguard_flag_copy(const XGuardArgs &g, uint32_t wg)
@@ -121,6 +127,19 @@ __device__ __forceinline__ void xguard_commit(const XGuardArgs &g, uint32_t wg)
     g.done[wg] = (uint8_t)g.gen;
 }
 
+/// Called by ONE lane of a work-group that leaves because its copy of the preempt word
+/// has changed (at entry or at a later look): later launches of this epoch must not run.
+__device__ __forceinline__ void xguard_note_flush(const XGuardArgs &g)
+{
+    if (g.flushed) *g.flushed = g.epoch;
+}
+
+/// True when an earlier launch of this epoch has been flushed (wave-uniform).
+__device__ __forceinline__ bool xguard_epoch_flushed(const XGuardArgs &g)
+{
+    return g.flushed != nullptr && __builtin_amdgcn_readfirstlane(*g.flushed) == g.epoch;
+}
+
 /// Guard of a work-group that is ONE wavefront (blockDim == 64): the decision is
 /// wave-uniform by construction, no LDS or barrier is needed.
 class XGuardWave
@@ -131,7 +150,12 @@ public:
     /// False: this work-group must not run (flushed, or finished by an earlier launch).
     __device__ __forceinline__ bool Enter() const
     {
-        if (xguard_read_flag(xguard_flag_copy(g_, wg_)) != g_.epoch) return false;
+        const bool earlier_flushed = xguard_epoch_flushed(g_);
+        if (xguard_read_flag(xguard_flag_copy(g_, wg_)) != g_.epoch) {
+            if ((threadIdx.x & 63) == 0) xguard_note_flush(g_);
+            return false;
+        }
+        if (earlier_flushed) return false;
         if (g_.resume && g_.done && xguard_committed(g_, wg_)) return false;
         return true;
     }
@@ -158,7 +182,10 @@ public:
     __device__ __forceinline__ bool Enter() const
     {
         if (threadIdx.x < 64) {
+            const bool earlier_flushed = xguard_epoch_flushed(g_);
             bool go = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+            if (!go && threadIdx.x == 0) xguard_note_flush(g_);
+            if (earlier_flushed) go = false;
             if (go && g_.resume && g_.done && xguard_committed(g_, wg_)) go = false;
             if (threadIdx.x == 0) *lds_ = go ? 1u : 0u;
         }
@@ -173,7 +200,11 @@ public:
     __device__ __forceinline__ bool StillCurrent() const
     {
         __syncthreads();
-        if (threadIdx.x == 0) *lds_ = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch ? 1u : 0u;
+        if (threadIdx.x == 0) {
+            const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+            if (!current) xguard_note_flush(g_);
+            *lds_ = current ? 1u : 0u;
+        }
         __syncthreads();
         return *lds_ != 0;
     }
@@ -184,7 +215,9 @@ public:
     /// has in front of its write-out.
     __device__ __forceinline__ bool WaveStillCurrent() const
     {
-        return xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+        const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
+        if (!current && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
+        return current;
     }
 
     /// WaveStillCurrent() split in two so that the read of the preempt word overlaps the
@@ -196,7 +229,9 @@ public:
 
     __device__ __forceinline__ bool WavePollEnd(uint32_t pending) const
     {
-        return xguard_read_flag_end(pending) == g_.epoch;
+        const bool current = xguard_read_flag_end(pending) == g_.epoch;
+        if (!current && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
+        return current;
     }
 
     /// Call after the last store of the work-group (all waves; one barrier inside).

@@ -37,6 +37,12 @@ XResult HipQueueCreate(HwQueueHandle *hwq, void *stream);
  * block in the driver, [6] progress-map slots in use, [7] current preempt epoch. */
 XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
 
+/* For tests of the guard protocol: stores the queue's current preempt epoch into its
+ * "flushed" word, as a work-group does that leaves because a deactivation reached it.
+ * Guarded launches of that epoch then do nothing (they wait for a replay, which only a
+ * deactivation / reactivation of the queue brings). No counterpart in the reference. */
+XResult HipQueueMarkEpochFlushed(HwQueueHandle hwq);
+
 /* ---- guarded victim kernels: flushable at level 2 ---------------------------
  * `guard`: 0 = plain kernel (never flushable, property None),
  *          1 = guarded kernel, property Deactivatable: at level 2 it carries the

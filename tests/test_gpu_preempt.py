@@ -238,3 +238,69 @@ def test_cross_queue_wait_on_recorded_event_follows_replays(xs, gpu):
     assert st[2] > 0, "queue A was never deactivated: the test did not exercise level 2"
     assert np.array_equal(got_a.view(np.uint32), want_a.view(np.uint32))
     assert np.array_equal(got_b.view(np.uint32), want_b.view(np.uint32)), "B ran before A had finished"
+
+
+@pytest.mark.parametrize("kind", ["axpy", "axpy few waves", "histogram", "gemm"])
+def test_launches_of_a_flushed_epoch_do_not_run(xs, gpu, kind):
+    """The copies of the preempt word are rewritten one after the other, so a work-group of
+    a later launch may still read an old copy when an earlier launch has already been
+    flushed. What keeps it from running ahead is the queue's "flushed" word: a flushed
+    work-group leaves the epoch of its launch there, and no work-group runs under an epoch
+    it finds there. The race itself cannot be staged; the test writes the word the way a
+    flushed work-group does and checks both halves of the rule: commands of that epoch
+    leave memory untouched, commands launched after a deactivation / reactivation (a new
+    epoch) run."""
+    torch = gpu
+    print(f"case flushed-epoch {kind}", flush=True)
+    q = Queue(xs, torch, level=2, threshold=4, batch=2)
+    p = xs.preempt()
+    if kind.startswith("axpy"):
+        n = (1 << 20) + 3
+        x_h = oracle.fill_uniform(3, 0, 0, n)
+        y_h = oracle.fill_uniform(3, 1, 0, n)
+        x, y = torch.from_numpy(x_h).cuda(), torch.from_numpy(y_h).cuda()
+        make = lambda: axpy_cmd(xs, 0.5, x, y, n, 3 if "few" in kind else 1)
+        read = lambda: y.cpu().numpy().view(np.uint32)
+        before = y_h.view(np.uint32)
+        after = oracle.axpy(0.5, x_h, y_h, 1).view(np.uint32)
+    elif kind == "histogram":
+        n, n_bins = (1 << 20) + 5, 65536
+        keys_h = oracle.fill_zipf(4, 1, 0, n, oracle.zipf_table(n_bins), n_bins)
+        keys = torch.from_numpy(keys_h).cuda()
+        bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+        make = lambda: hist_cmd(xs, keys, n, bins, n_bins, 1)
+        read = lambda: bins.cpu().numpy().view(np.uint32)
+        before = np.zeros(n_bins, np.uint32)
+        after = oracle.histogram(keys_h, n_bins)
+    else:
+        M = N = K = 512
+        a_h = oracle.fill_normal_bf16(5, 0, 0, M * K)
+        b_h = oracle.fill_normal_bf16(5, 1, 0, K * N)
+        a = torch.from_numpy(a_h.view(np.int16).reshape(M, K)).cuda()
+        b = torch.from_numpy(b_h.view(np.int16).reshape(K, N)).cuda()
+        c = torch.zeros(M, N, dtype=torch.int16, device="cuda")
+        make = lambda: gemm_cmd(xs, a, b, c, M, N, K, 1)
+        read = lambda: c.cpu().numpy().view(np.uint16).ravel()
+        before = np.zeros(M * N, np.uint16)
+        # what an undisturbed queue computes (bit-identical run to run: fixed summation order)
+        c2 = torch.zeros(M, N, dtype=torch.int16, device="cuda")
+        q2 = Queue(xs, torch, level=2)
+        q2.submit(gemm_cmd(xs, a, b, c2, M, N, K, 1))
+        q2.wait()
+        q2.close()
+        after = c2.cpu().numpy().view(np.uint16).ravel()
+        assert after.any()
+
+    xs.check(xs.halhip().HipQueueMarkEpochFlushed(q.hwq))
+    q.submit(make())
+    q.submit(make())
+    q.wait()
+    untouched = read().copy()
+    xs.check(p.XQueueSuspend(q.xq, 0))
+    xs.check(p.XQueueResume(q.xq, 0))
+    q.submit(make())
+    q.wait()
+    ran = read().copy()
+    q.close()
+    assert np.array_equal(untouched, before), "a launch of a flushed epoch wrote something"
+    assert np.array_equal(ran, after), "a launch of the next epoch did not run exactly once"

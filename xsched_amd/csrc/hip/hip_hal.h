@@ -59,6 +59,8 @@ public:
     /// Device-visible address of copy 0 of the preempt word, and copies - 1.
     const uint32_t *FlagDevPtr() const { return flag_dev_; }
     uint32_t FlagMask() const { return copies_ - 1; }
+    /// The word in which flushed work-groups leave the epoch of their launch (cached device memory).
+    uint32_t *FlushedDevPtr() const { return flushed_dev_; }
     uint32_t Epoch() const { return epoch_.load(std::memory_order_acquire); }
 
     /// Bump the preempt word; visible to running kernels within a memory round trip.
@@ -80,6 +82,7 @@ private:
     uint32_t copies_ = 1;            // power of two
     uint32_t *flag_host_ = nullptr;  // pinned image of all copies (the word itself when on host)
     uint32_t *flag_dev_ = nullptr;   // GPU address of copy 0
+    uint32_t *flushed_dev_ = nullptr; // written by flushed work-groups, read by later launches
     std::atomic<uint32_t> epoch_ { 0 };
 
     bool write_through_bar_ = false; // CPU stores straight into device memory

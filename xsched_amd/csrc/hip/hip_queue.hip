@@ -102,11 +102,16 @@ GuardState::GuardState(int device): device_(device)
     copies_ = 1;
     while ((int64_t)copies_ * 2 <= copies && copies_ < 4096) copies_ *= 2;
 
+    // no launch ever carries epoch 0xFFFFFFFF
+    HIP_ASSERT(hipMalloc((void **)&flushed_dev_, 256));
+    HIP_ASSERT(hipMemset(flushed_dev_, 0xFF, 256));
+
     const size_t bytes = (size_t)copies_ * kXGuardFlagStrideWords * sizeof(uint32_t);
     HIP_ASSERT(hipHostMalloc((void **)&flag_host_, bytes, hipHostMallocMapped | hipHostMallocCoherent));
     memset(flag_host_, 0, bytes);
     if (flag_on_host_) {
         HIP_ASSERT(hipHostGetDevicePointer((void **)&flag_dev_, flag_host_, 0));
+        HIP_ASSERT(hipDeviceSynchronize());
         return;
     }
     HIP_ASSERT(hipExtMallocWithFlags((void **)&flag_dev_, bytes, hipDeviceMallocFinegrained));
@@ -128,6 +133,7 @@ GuardState::~GuardState()
     // any more (each guarded command keeps a reference while it owns a slot).
     for (uint8_t *a : arenas_) (void)hipFree(a);
     if (!flag_on_host_ && flag_dev_) (void)hipFree(flag_dev_);
+    if (flushed_dev_) (void)hipFree(flushed_dev_);
     if (flag_host_) (void)hipHostFree(flag_host_);
 }
 
@@ -263,6 +269,7 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
     g.epoch = q.Guard()->Epoch();
     g.resume = replay ? 1u : 0u;
     g.flag_mask = q.Guard()->FlagMask();
+    g.flushed = q.Guard()->FlushedDevPtr();
 
     if (guarded && level2) {
         if (slot_.done == nullptr) {
@@ -457,6 +464,17 @@ EXPORT_C_FUNC XResult HipQueueCreate(HwQueueHandle *hwq, void *stream)
     XResult res = HwQueueManager::Add(h, [&]() { return std::make_shared<HipQueue>((hipStream_t)stream); });
     if (res == kXSchedSuccess) *hwq = h;
     return res;
+}
+
+EXPORT_C_FUNC XResult HipQueueMarkEpochFlushed(HwQueueHandle hwq)
+{
+    auto q = std::dynamic_pointer_cast<HipQueue>(HwQueueManager::Get(hwq));
+    if (q == nullptr) return kXSchedErrorNotFound;
+    const uint32_t epoch = q->Guard()->Epoch();
+    // behind whatever the stream still holds, as a flushed work-group's store would be
+    hipError_t err = hipMemcpyAsync(q->Guard()->FlushedDevPtr(), &epoch, sizeof(epoch), hipMemcpyHostToDevice, q->Stream());
+    if (err == hipSuccess) err = hipStreamSynchronize(q->Stream());
+    return err == hipSuccess ? kXSchedSuccess : kXSchedErrorUnknown;
 }
 
 EXPORT_C_FUNC XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out)

@@ -110,6 +110,8 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
     constexpr uint32_t kStepVecs = kLanes * kVecPerStep;
     const uint32_t lane = threadIdx.x;
     const uint32_t *flag = xguard_flag_copy(g, blockIdx.x);
+    // an earlier launch of this epoch was flushed: this one must not run ahead of its replay
+    if (xguard_epoch_flushed(g)) return;
 
     for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
         const uint64_t chunk_base = (uint64_t)c * steps * kStepVecs;
@@ -125,7 +127,10 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
         }
         // The scalar read of the preempt word waits for itself only: the vector loads
         // above stay in flight across it. A flushed wave drops what it has loaded.
-        if (xguard_read_flag(flag) != g.epoch) return;
+        if (xguard_read_flag(flag) != g.epoch) {
+            if (lane == 0) xguard_note_flush(g);
+            return;
+        }
         if (g.resume && g.done && xguard_committed(g, c)) continue;
 
         if (full) {

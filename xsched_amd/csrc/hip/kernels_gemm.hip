@@ -217,7 +217,9 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         load_b_frags(cur, 3, fb);
 
         if (kGuard && (t % kPollSteps) == kPollSteps - 1 && tid == 0) {
-            guard_word = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch ? 1u : 0u;
+            const bool current = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch;
+            if (!current) xguard_note_flush(g);
+            guard_word = current ? 1u : 0u;
         }
         __syncthreads(); // buffer cur^1 is complete, buffer cur is free to be overwritten
         if (kGuard && (t % kPollSteps) == kPollSteps - 1) {
