@@ -137,7 +137,7 @@ __device__ __forceinline__ void xguard_note_flush(const XGuardArgs &g)
 /// True when an earlier launch of this epoch has been flushed (wave-uniform).
 __device__ __forceinline__ bool xguard_epoch_flushed(const XGuardArgs &g)
 {
-    return g.flushed != nullptr && __builtin_amdgcn_readfirstlane(*g.flushed) == g.epoch;
+    return g.flushed != nullptr && (uint32_t)__builtin_amdgcn_readfirstlane((int)*g.flushed) == g.epoch;
 }
 
 /// Guard of a work-group that is ONE wavefront (blockDim == 64): the decision is
