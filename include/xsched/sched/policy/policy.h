@@ -44,7 +44,11 @@ private:
     AddTimerFunc add_timer_func_ = nullptr;
 };
 
-/// Fatal for a type this build does not carry.
+/// Whether CreatePolicy() has a class for the type (every named type except the strict
+/// process partition, which the reference declares but never implemented either).
+bool PolicyAvailable(XPolicyType type);
+
+/// Fatal for a type without a class.
 std::unique_ptr<Policy> CreatePolicy(XPolicyType type);
 
 } // namespace xsched::sched

@@ -138,6 +138,9 @@ DRV_EXPORT size_t DRV(bytes_hint_kdeadline)(uint64_t k, void *out, size_t cap)
 DRV_EXPORT size_t DRV(bytes_hint_laxity)(uint64_t xq, int64_t lax, int lp, int cp, void *out, size_t cap)
 { LaxityHint h(xq, lax, lp, cp); return CopyOut(h.Data(), h.Size(), out, cap); }
 
+DRV_EXPORT size_t DRV(bytes_hint_window_active)(int pid, uint64_t display, void *out, size_t cap)
+{ WindowActiveHint h((PID)pid, display); return CopyOut(h.Data(), h.Size(), out, cap); }
+
 DRV_EXPORT size_t DRV(bytes_event_hint_priority)(uint64_t xq, int prio, void *out, size_t cap)
 { HintEvent e(std::make_shared<PriorityHint>(xq, prio)); return CopyOut(e.Data(), e.Size(), out, cap); }
 

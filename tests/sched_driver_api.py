@@ -19,6 +19,7 @@ FIELDS = {
     "hint_deadline": [(0, 4), (8, 8), (16, 8)],
     "hint_kdeadline": [(0, 4), (8, 8)],
     "hint_laxity": [(0, 4), (8, 8), (16, 8), (24, 4), (28, 4)],
+    "hint_window_active": [(0, 4), (4, 4), (8, 8)],
     "event_hint_priority": [(0, 8), (8, 8), (16, 4), (24, 8), (32, 4)],
     "event_process_create": [(0, 264)],
     "event_process_destroy": [(0, 8)],
@@ -124,6 +125,7 @@ RECORD_ARGS = {
     "hint_deadline": [c_uint64, c_int64],
     "hint_kdeadline": [c_uint64],
     "hint_laxity": [c_uint64, c_int64, c_int, c_int],
+    "hint_window_active": [c_int, c_uint64],
     "event_hint_priority": [c_uint64, c_int],
     "event_process_create": [c_char_p],
     "event_process_destroy": [c_int],

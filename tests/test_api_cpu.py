@@ -323,3 +323,93 @@ def test_laxity_policy_promotes_after_the_laxity(xs):
     for xq, hw in ((xq_a, hw_a), (xq_b, hw_b)):
         xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hw))
     xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+
+
+def test_every_policy_with_a_class_can_be_selected(xs):
+    """The reference names eleven policies and implements ten (the strict process
+    partition has an enum value and a name only); so does this build."""
+    p = xs.preempt()
+    for policy in (1, 2, 3, 4, 5, 7, 8, 9, 10, 11):
+        assert p.XHintSetScheduler(xs.kSchedulerLocal, policy) == xs.kXSchedSuccess, policy
+    for policy in (0, 6, 12, -1):
+        assert p.XHintSetScheduler(xs.kSchedulerLocal, policy) == xs.kXSchedErrorInvalidValue, policy
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+
+
+def test_kedf_runs_the_earliest_deadline_first(xs):
+    """KEDF with k = 1 through the C API: of two queues with work, the one whose deadline
+    (ready time + XHintDeadline) comes first runs; the other's backlog moves only when the
+    first is idle. With XHintKDeadline(2) both run."""
+    p, h = xs.preempt(), xs.halhost()
+    xs.check(p.XHintSetScheduler(xs.kSchedulerLocal, 7))
+    hw_a, hw_b = xs.host_queue_create(), xs.host_queue_create()
+    xq_a, xq_b = xs.xqueue_create(hw_a), xs.xqueue_create(hw_b)
+    xs.check(p.XHintDeadline(xq_a, 1_000))            # 1 ms after it becomes ready
+    xs.check(p.XHintDeadline(xq_b, 10_000_000))       # 10 s
+    gate = threading.Event()
+
+    @xs.HostKernelFn
+    def slow(arg, wg, n_wg):
+        gate.wait(5)
+
+    @xs.HostKernelFn
+    def quick(arg, wg, n_wg):
+        pass
+
+    cmd = c_uint64()
+    xs.check(h.HostKernelCommandCreate(byref(cmd), slow, None, 1, 0))
+    xs.check(p.XQueueSubmit(xq_a, cmd.value))
+    time.sleep(0.05)
+    for _ in range(4):
+        xs.check(h.HostKernelCommandCreate(byref(cmd), quick, None, 1, 0))
+        xs.check(p.XQueueSubmit(xq_b, cmd.value))
+    time.sleep(0.1)
+    held, _, _ = host_stats(xs, hw_b)
+    xs.check(p.XHintKDeadline(2))
+    time.sleep(0.1)
+    released, _, _ = host_stats(xs, hw_b)
+    gate.set()
+    xs.check(p.XQueueWaitAll(xq_a)); xs.check(p.XQueueWaitAll(xq_b))
+    assert held == 0, "the later deadline ran while the earlier one had work"
+    assert released == 4
+    for xq, hw in ((xq_a, hw_a), (xq_b, hw_b)):
+        xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hw))
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+
+
+def test_utilization_partition_takes_turns(xs):
+    """UP through the C API: two queues with equal shares of a 40 ms timeslice, both with a
+    long backlog of 2 ms commands. At any time only one of them runs; over 400 ms both make
+    progress and neither gets more than about three quarters of the work done."""
+    p, h = xs.preempt(), xs.halhost()
+    xs.check(p.XHintSetScheduler(xs.kSchedulerLocal, 4))
+    hw_a, hw_b = xs.host_queue_create(), xs.host_queue_create()
+    xq_a, xq_b = xs.xqueue_create(hw_a), xs.xqueue_create(hw_b)
+    for xq in (xq_a, xq_b):
+        xs.check(p.XQueueSetLaunchConfig(xq, 2, 1))
+        xs.check(p.XHintUtilization(xq, 50))
+    xs.check(p.XHintTimeslice(40_000))
+
+    @xs.HostKernelFn
+    def work(arg, wg, n_wg):
+        time.sleep(0.002)
+
+    cmd = c_uint64()
+    for _ in range(400):
+        for xq in (xq_a, xq_b):
+            xs.check(h.HostKernelCommandCreate(byref(cmd), work, None, 1, 0))
+            xs.check(p.XQueueSubmit(xq, cmd.value))
+    time.sleep(0.4)
+    done_a, _, _ = host_stats(xs, hw_a)
+    done_b, _, _ = host_stats(xs, hw_b)
+    # drop what is left instead of waiting another second for it
+    for xq in (xq_a, xq_b):
+        xs.check(p.XQueueSuspend(xq, 0)); xs.check(p.XQueueResume(xq, 1))
+        xs.check(p.XQueueWaitAll(xq))
+    total = done_a + done_b
+    print("UP: a %d b %d" % (done_a, done_b))
+    assert total > 60
+    assert 0.25 < done_a / total < 0.75
+    for xq, hw in ((xq_a, hw_a), (xq_b, hw_b)):
+        xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hw))
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))

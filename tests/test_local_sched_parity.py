@@ -1,5 +1,6 @@
 """The LocalScheduler of this repository (event queue, worker, Status mirror, operation
-ids, policy switch, timers) against
+ids, policy switch, timers) and through it every policy (HPF, LAX, HHPF, CHPF, UP, PUP,
+KEDF, AWF, CFS, MLFQ) against
 (a) golden vectors recorded from the reference's own LocalScheduler
     (tests/golden/local_sched_vectors.json, written by
     tests/golden/make_local_sched_vectors.py from oracle/_ref/libsched_ref.so), and
@@ -60,8 +61,8 @@ def test_fixture_covers_the_current_scripts(golden):
 
 def test_fixture_is_not_trivial(golden):
     ops = [op for entry in golden.values() for rnd in entry["operations"] for op in rnd]
-    assert len(ops) > 1000
-    assert sum(1 for op in ops if op[3]) > 200        # rounds with something suspended
+    assert len(ops) > 2500
+    assert sum(1 for op in ops if op[3]) > 900        # rounds with something suspended
     assert sum(1 for op in ops if op[0] == 0) > 10    # operations for a process never announced
     assert max(op[0] for op in ops) > 30
 
@@ -74,9 +75,29 @@ def test_operations_match_golden(probe, golden, name):
 
 def test_operations_against_live_reference(probe, ref):
     for seed in range(200, 206):
-        for policy in (scripts.HPF, scripts.LAX):
+        for policy in (scripts.HPF, scripts.LAX) + tuple(scripts.RANDOM_POLICIES.values()):
             script = scripts.random_script(seed, policy)
             assert scripts.play(probe, script) == scripts.play(ref, script), (seed, policy)
+
+
+def test_wall_clock_policies_against_live_reference(probe, ref):
+    """The time-sliced policies (queue and process shares with slices that end, fair share,
+    feedback levels) on scripts whose pauses keep every comparison far from its threshold."""
+    for name, script in scripts.more_policy_scripts().items():
+        assert scripts.play(probe, script) == scripts.play(ref, script), name
+
+
+def test_process_priority_policy_with_real_processes(probe, ref, monkeypatch):
+    """CHPF reads /proc/<pid>/sched: this process and pid 1 run at a normal Linux priority
+    (120, which the policy counts as -120), a pid that does not exist counts as 0 and wins."""
+    monkeypatch.setattr(scripts, "PIDS", (os.getpid(), 1, 4190003))
+    seen_suspended = 0
+    for seed in range(400, 404):
+        script = scripts.random_script(seed, scripts.CHPF)
+        mine = scripts.play(probe, script)
+        assert mine == scripts.play(ref, script), seed
+        seen_suspended += sum(1 for rnd in mine for op in rnd if op[3])
+    assert seen_suspended > 20
 
 
 def timed_laxity_states(drv):

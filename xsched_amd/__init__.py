@@ -26,6 +26,10 @@ kQueueSuspendFlagWaitAll, kQueueSuspendFlagWaitIdle = 2, 4
 kQueueResumeFlagNone, kQueueResumeFlagDropCommands = 0, 1
 kSchedulerUnknown, kSchedulerAppManaged, kSchedulerLocal, kSchedulerGlobal = 0, 1, 2, 3
 kPolicyUnknown, kPolicyHighestPriorityFirst, kPolicyLaxity = 0, 1, 8
+kPolicyHeterogeneousHighestPriorityFirst, kPolicyCPUHighestPriorityFirst = 2, 3
+kPolicyUtilizationPartition, kPolicyProcessUtilizationPartition = 4, 5
+kPolicyKEarliestDeadlineFirst, kPolicyActiveWindowFirst = 7, 9
+kPolicyCompletelyFairScheduler, kPolicyMultiLevelFeedbackQueue = 10, 11
 PRIORITY_NO_EXECUTE, PRIORITY_MIN, PRIORITY_DEFAULT, PRIORITY_MAX = -256, -255, 0, 255
 
 XResult = c_int

@@ -34,7 +34,7 @@ HIPFLAGS = ["--offload-arch=gfx950", "-std=c++20", "-O3", "-fPIC", "-pthread", "
 
 PREEMPT_SRCS = [
     "protocol/log.cpp", "protocol/names.cpp",
-    "sched/protocol.cpp", "sched/policy.cpp", "sched/local.cpp", "sched/global.cpp",
+    "sched/protocol.cpp", "sched/policy.cpp", "sched/policy_extra.cpp", "sched/local.cpp", "sched/global.cpp",
     "sched/channel.cpp",
     "preempt/xcommand.cpp", "preempt/command_buffer.cpp", "preempt/launch_worker.cpp",
     "preempt/async_xqueue.cpp", "preempt/xqueue.cpp", "preempt/agent.cpp",

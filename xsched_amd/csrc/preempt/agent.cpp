@@ -129,7 +129,7 @@ XResult SchedAgent::ReplaceScheduler(XSchedulerType scheduler_type, XPolicyType 
 
     if (current->GetType() == scheduler_type) {
         if (scheduler_type != kSchedulerLocal) return kXSchedSuccess;
-        if (policy_type <= kPolicyUnknown || policy_type >= kPolicyMax) {
+        if (!PolicyAvailable(policy_type)) {
             XWARN("invalid policy type: %d", policy_type);
             return kXSchedErrorInvalidValue;
         }
@@ -140,8 +140,7 @@ XResult SchedAgent::ReplaceScheduler(XSchedulerType scheduler_type, XPolicyType 
     }
 
     // A local scheduler is selected by its policy (see CreateScheduler()).
-    if (scheduler_type == kSchedulerLocal &&
-        (policy_type <= kPolicyUnknown || policy_type >= kPolicyMax)) {
+    if (scheduler_type == kSchedulerLocal && !PolicyAvailable(policy_type)) {
         XWARN("invalid policy type: %d", policy_type);
         return kXSchedErrorInvalidValue;
     }

@@ -157,12 +157,12 @@ void OnSignal(int)
 int main(int argc, char **argv)
 {
     if (argc < 2) {
-        fprintf(stderr, "usage: %s <policy: HPF | LAX> [port, unused]\n", argv[0]);
+        fprintf(stderr, "usage: %s <policy: HPF | HHPF | CHPF | UP | PUP | KEDF | LAX | AWF | CFS | MLFQ> [port, unused]\n", argv[0]);
         return 2;
     }
     const XPolicyType policy = GetPolicyType(argv[1]);
-    if (policy != kPolicyHighestPriorityFirst && policy != kPolicyLaxity) {
-        fprintf(stderr, "xserver: policy '%s' is not available (HPF and LAX are)\n", argv[1]);
+    if (!xsched::sched::PolicyAvailable(policy)) {
+        fprintf(stderr, "xserver: policy '%s' is not available\n", argv[1]);
         return 2;
     }
     signal(SIGINT, OnSignal);
