@@ -118,6 +118,55 @@ DRV_EXPORT int DRV(policy_sched)(void *p, int n, const uint64_t *handles, const 
     return nt;
 }
 
+/// Any hint, from its wire bytes.
+DRV_EXPORT int DRV(policy_recv_hint)(void *p, const void *hint_bytes)
+{
+    auto hint = Hint::CopyConstructor(hint_bytes);
+    if (hint == nullptr) return 0;
+    ((PolicyBox *)p)->policy->RecvHint(hint);
+    return 1;
+}
+
+/// policy_sched with processes: queue i belongs to pids[i] and is listed among that
+/// process's suspended (suspended[i] != 0) or running XQueues.
+DRV_EXPORT int DRV(policy_sched_processes)(void *p, int n, const uint64_t *handles, const uint64_t *devices,
+                                           const uint8_t *ready, const int64_t *ready_time_us, const int *pids,
+                                           const uint8_t *suspended, int8_t *decision, int64_t *timers_us,
+                                           int max_timers)
+{
+    auto *box = (PolicyBox *)p;
+    Status status;
+    for (int i = 0; i < n; ++i) {
+        auto xq = std::make_unique<XQueueStatus>();
+        xq->handle = handles[i];
+        xq->device = devices[i];
+        xq->level = kPreemptLevelBlock;
+        xq->pid = (PID)pids[i];
+        xq->threshold = 16;
+        xq->batch_size = 8;
+        xq->ready = ready[i] != 0;
+        xq->suspended = suspended[i] != 0;
+        xq->ready_time = std::chrono::system_clock::time_point(std::chrono::microseconds(ready_time_us[i]));
+        status.xqueue_status[handles[i]] = std::move(xq);
+        auto &ps = status.process_status[(PID)pids[i]];
+        if (ps == nullptr) {
+            ps = std::make_unique<ProcessStatus>();
+            ps->info.pid = (PID)pids[i];
+        }
+        (suspended[i] != 0 ? ps->suspended_xqueues : ps->running_xqueues).insert(handles[i]);
+    }
+    box->decision.clear();
+    box->timers_us.clear();
+    box->policy->Sched(status);
+    for (int i = 0; i < n; ++i) {
+        auto it = box->decision.find(handles[i]);
+        decision[i] = it == box->decision.end() ? (int8_t)-1 : it->second;
+    }
+    const int nt = (int)box->timers_us.size();
+    for (int i = 0; i < nt && i < max_timers; ++i) timers_us[i] = box->timers_us[i];
+    return nt;
+}
+
 // ---- wire records ----------------------------------------------------------------
 
 DRV_EXPORT size_t DRV(bytes_hint_priority)(uint64_t xq, int prio, void *out, size_t cap)

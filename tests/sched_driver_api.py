@@ -155,6 +155,28 @@ class _Policy:
     def laxity(self, xq, lax, lp, cp):
         self.drv.fn("policy_hint_laxity", None, [c_void_p, c_uint64, c_int64, c_int, c_int])(self.h, xq, lax, lp, cp)
 
+    def hint(self, hint_bytes):
+        assert self.drv.fn("policy_recv_hint", c_int, [c_void_p, c_char_p])(self.h, hint_bytes) == 1
+
+    def sched_processes(self, queues):
+        """queues: list of (handle, device, ready, ready_time_us, pid, suspended) ->
+        (decisions, timers); decisions: 1 suspend, 0 resume, -1 not touched"""
+        n = len(queues)
+        f = self.drv.fn("policy_sched_processes", c_int,
+                        [c_void_p, c_int, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint8),
+                         POINTER(c_int64), POINTER(c_int), POINTER(c_uint8), POINTER(c_int8),
+                         POINTER(c_int64), c_int])
+        h = (c_uint64 * n)(*[q[0] for q in queues])
+        d = (c_uint64 * n)(*[q[1] for q in queues])
+        r = (c_uint8 * n)(*[1 if q[2] else 0 for q in queues])
+        t = (c_int64 * n)(*[q[3] for q in queues])
+        pid = (c_int * n)(*[q[4] for q in queues])
+        sus = (c_uint8 * n)(*[1 if q[5] else 0 for q in queues])
+        dec = (c_int8 * n)()
+        timers = (c_int64 * 16)()
+        nt = f(self.h, n, h, d, r, t, pid, sus, dec, timers, 16)
+        return list(dec), list(timers)[:min(nt, 16)]
+
     def sched(self, queues):
         """queues: list of (handle, device, ready, ready_time_us) -> (decisions, timers)"""
         n = len(queues)

@@ -194,3 +194,108 @@ def test_hpf_closed_form(probe):
         want = [1 if prio[h] < bar.get(dev[h], -255) else 0 for h in handles]
         sc = {"queues": [(h, dev[h], ready[h], 0) for h in handles], "hints": list(raw.items())}
         assert run_hpf(probe, sc)[0] == want
+
+
+# ---- budgets of the time-sliced policies ------------------------------------------
+# The operation-stream tests (test_local_sched_parity.py) see WHO runs; how long a turn
+# lasts shows only in the timer a policy asks for. Closed forms, stated from the
+# reference's up.cpp:136-144 and pup.cpp:36-40, 56-66, 84-92, 144-163:
+#   UP   budget = timeslice * share / sum of shares
+#   PUP  share(p) = timeslice * queued processes * util(p) / sum of utils (100 without a hint)
+#        a turn lasts carried + share(p), where carried = what was left of p's last slice,
+#        plus one share for every time p reached the front while idle, and a carried amount
+#        above one share first loses a tenth of the excess.
+
+UP, PUP, CFS, MLFQ = 4, 5, 10, 11
+GPU0 = 0x100000000
+TOLERANCE_US = 30_000   # the test's own run time enters every "left of the slice"
+
+
+def budget_after(policy, queues, processes=True):
+    before = int(time.time() * 1e6)
+    dec, timers = policy.sched_processes(queues) if processes else policy.sched(queues)
+    assert len(timers) == 1, timers
+    return dec, timers[0] - before
+
+
+def up_budgets(drv):
+    p = drv.policy(UP)
+    p.hint(drv.record("hint_timeslice", 10_000_000))
+    p.hint(drv.record("hint_utilization", 0, 1, 30))
+    p.hint(drv.record("hint_utilization", 0, 3, 70))
+    q = lambda h, ready: (h, GPU0, ready, 0)
+    out = []
+    dec, b = budget_after(p, [q(1, True), q(3, True), q(5, True)], processes=False)
+    out.append((dec, b))
+    p.hint(drv.record("hint_utilization", 0, 5, 50))
+    dec, b = budget_after(p, [q(1, False), q(3, True), q(5, True)], processes=False)
+    out.append((dec, b))
+    dec, b = budget_after(p, [q(1, True), q(3, False), q(5, True)], processes=False)
+    out.append((dec, b))
+    p.close()
+    return out
+
+
+UP_EXPECTED = [([0, 1, 1], 3_000_000), ([1, 0, 1], 4_666_666), ([1, 1, 0], 3_333_333)]
+
+
+def pup_budgets(drv):
+    p = drv.policy(PUP)
+    p.hint(drv.record("hint_timeslice", 1_000_000))
+    p.hint(drv.record("hint_utilization", 11, 0, 40))
+    p.hint(drv.record("hint_utilization", 12, 0, 90))
+    state = {0xA: False, 0xB: False, 0xC: False}          # handle -> suspended, as a scheduler would track it
+    pid = {0xA: 11, 0xB: 12, 0xC: 13}
+    out = []
+    for ready in ([1, 1, 1], [0, 1, 1], [0, 0, 1], [0, 1, 0], [0, 0, 1], [1, 0, 0]):
+        queues = [(h, GPU0, bool(r), 0, pid[h], state[h]) for h, r in zip(sorted(state), ready)]
+        dec, b = budget_after(p, queues)
+        for h, d in zip(sorted(state), dec):
+            if d >= 0:
+                state[h] = d == 1
+        out.append(([h for h in sorted(state) if not state[h]], b))
+    p.close()
+    return out
+
+
+SHARE = {11: 3_000_000 * 40 // 230, 12: 3_000_000 * 90 // 230, 13: 3_000_000 * 100 // 230}
+PUP_EXPECTED = [
+    ([0xA], SHARE[11]),                                   # 11 first in the run queue
+    ([0xB], SHARE[12]),                                   # 11 fell idle with almost a whole share left
+    ([0xC], SHARE[13]),
+    ([0xB], 2 * SHARE[12]),                               # 12's leftover share + a new one (11 topped up on the way)
+    ([0xC], 2 * SHARE[13]),
+    ([0xA], SHARE[11] + int(SHARE[11] + (2 * SHARE[11] - SHARE[11]) * 0.9)),   # 2 shares carried: one decays by a tenth
+]
+
+
+def close_to(got, want):
+    assert len(got) == len(want)
+    for (g_who, g_us), (w_who, w_us) in zip(got, want):
+        assert g_who == w_who, (got, want)
+        assert w_us - TOLERANCE_US <= g_us <= w_us + 5_000, (got, want)
+
+
+def test_up_budgets_closed_form(probe):
+    close_to(up_budgets(probe), UP_EXPECTED)
+
+
+def test_pup_budgets_closed_form(probe):
+    close_to(pup_budgets(probe), PUP_EXPECTED)
+
+
+def test_budgets_against_live_reference(probe, ref):
+    close_to(up_budgets(ref), UP_EXPECTED)
+    close_to(pup_budgets(ref), PUP_EXPECTED)
+
+
+@pytest.mark.parametrize("policy,tick_us", [(CFS, 1000), (MLFQ, 5000)])
+def test_tick_of_the_self_clocked_policies(probe, policy, tick_us):
+    """CFS asks to be run again after its 1 ms slice, MLFQ after its 5 ms tick, whenever a
+    queue is ready (reference cfs.cpp:101-103, mlfq.cpp:160-163); never when none is."""
+    p = probe.policy(policy)
+    _, b = budget_after(p, [(1, GPU0, True, 0), (2, GPU0, False, 0)], processes=False)
+    assert tick_us - 200 <= b <= tick_us + 20_000
+    dec, timers = p.sched([(1, GPU0, False, 0), (2, GPU0, False, 0)])
+    assert timers == []
+    p.close()
