@@ -254,6 +254,46 @@ def test_gemm_exact_on_small_integers(xs, gpu, M, N, K, level, guard):
     assert np.array_equal(got, want)
 
 
+def test_gemm_rounding_to_bf16_is_the_oracles(xs, gpu):
+    """Every C[i][j] here is ONE product a_i * b_j (the other 63 terms of the sum are 0 * 0),
+    so the fp32 accumulator holds it exactly and the stored bf16 shows the rounding alone:
+    ties to even, carries into the exponent, overflow to infinity, denormal results,
+    infinities and NaNs. Bit for bit the oracle's (u + 0x7FFF + lsb) >> 16 with quieted NaNs."""
+    torch = gpu
+    M = N = 256
+    K = 64
+    print("case gemm-rounding", flush=True)
+    rng = np.random.default_rng(7)
+
+    def interesting(count):
+        bits = rng.integers(0, 1 << 16, count).astype(np.uint16)            # any bf16 at all
+        bits[:8] = [0x0000, 0x8000, 0x7F80, 0xFF80, 0x7FC0, 0x7F81, 0x0001, 0x807F]
+        bits[8:16] = [0x3F80, 0x3F81, 0x3FFF, 0x4000, 0x7F7F, 0x0080, 0x3F7F, 0xBF81]
+        bits[16:96] = rng.integers(0x3F80, 0x4080, 80).astype(np.uint16)    # products around 1..4 hit ties often
+        bits[96:128] = rng.integers(0x0001, 0x0100, 32).astype(np.uint16)   # denormal and tiny operands
+        return bits
+
+    a_col, b_row = interesting(M), interesting(N)
+    a_bits = np.zeros((M, K), np.uint16)
+    b_bits = np.zeros((K, N), np.uint16)
+    a_bits[:, 5] = a_col
+    b_bits[5, :] = b_row
+    got = _gemm_case(xs, torch, a_bits.ravel(), b_bits.ravel(), M, N, K, 1, 0).reshape(M, N)
+    want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K).reshape(M, N)
+
+    def is_nan(h):
+        return (h & 0x7FFF) > 0x7F80
+    nan_want = is_nan(want)
+    assert np.array_equal(is_nan(got), nan_want)
+    # which NaN comes out (sign, payload) is the matrix unit's business: it answers every
+    # NaN, passed through or made by inf * 0, with its default NaN, the oracle's fmaf keeps
+    # the operand's. Only that it IS a NaN is compared.
+    same = (got == want) | nan_want
+    bad = np.argwhere(~same)
+    assert bad.size == 0, [(hex(a_col[i]), hex(b_row[j]), hex(got[i, j]), hex(want[i, j])) for i, j in bad[:8]]
+    assert np.count_nonzero(~nan_want) > 60000
+
+
 def test_gemm_normal_inputs_within_tolerance(xs, gpu):
     """Seeded N(0,1)-like inputs: the MFMA's internal summation order is not the
     oracle's, so the comparison is on values. Tolerance: one bf16 unit in the last

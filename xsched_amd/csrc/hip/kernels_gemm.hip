@@ -45,12 +45,17 @@ constexpr int kPollSteps = 8;       // K steps between two looks at the preempt 
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 4;       // tile rows walked together
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+/// Round-to-nearest-even to bf16, NaNs quieted: the conversion instruction of gfx950
+/// (v_cvt_pk_bf16_f32), which gives bit for bit what the integer formula
+/// (u + 0x7FFF + ((u >> 16) & 1)) >> 16, NaN -> (u >> 16) | 0x40 gives (a GPU test compares
+/// the two over products that hit ties, overflow, denormals, infinities and NaNs).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
 {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u); // quiet NaN
-    const uint32_t lsb = (u >> 16) & 1u;
-    return (uint16_t)((u + 0x7FFFu + lsb) >> 16);
+    const bf16x2 pair = __builtin_convertvector(f32x2 { f, 0.f }, bf16x2);
+    return (uint16_t)__builtin_bit_cast(uint32_t, pair);
 }
 
 // Work-group id -> tile coordinates. Ids with equal (id % 8) run on one XCD; each
