@@ -80,7 +80,7 @@ __device__ __forceinline__ void TileOf(uint32_t wg, uint32_t tiles_m, uint32_t t
 
 // Two LDS buffers and ONE barrier per K step: while the MFMAs of step t read buffer
 // t % 2, the registers holding tile t + 1 are written to the other buffer and the global
-// loads of tile t + 2 are issued; the A fragments of the next 16-wide k slice are read from
+// loads of tile t + 2 are issued; the fragments of the next 16-wide k slice are read from
 // LDS before the MFMAs of the current slice are issued.
 template <bool kGuard>
 __global__ __launch_bounds__(kThreads)
@@ -189,37 +189,33 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     //   slice 2: fragment reads of slice 3, global loads of tile t+2
     //   barrier  (the other buffer is complete, this one is no longer read)
     //   slice 3: fragment reads of slice 0 of the NEXT tile from the other buffer
-    // A fragments are double-buffered in registers, the two B fragments are re-read per
-    // slice after the slice's MFMAs have been issued: the register file (256 per wave at two
-    // waves per SIMD) has no room for a second set of both.
-    bf16x8 fa[2][4], fb[2];
-    load_frags(0, 0, fa[0], fb);
+    // Both fragment sets are double-buffered in registers (40 of them): the reads of slice
+    // s + 1 are issued before the MFMAs of slice s.
+    bf16x8 fa[2][4], fb[2][2];
+    load_frags(0, 0, fa[0], fb[0]);
 
     auto mfma_slice = [&](int set) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
     for (int t = 0; t < steps; ++t) {
         const int cur = t & 1;
         const int k_next = (t + 2 < steps ? t + 2 : steps - 1) * kStepK;
 
-        load_a_frags(cur, 1, fa[1]);
+        load_frags(cur, 1, fa[1], fb[1]);
         mfma_slice(0);
-        load_b_frags(cur, 1, fb);
 
-        load_a_frags(cur, 2, fa[0]);
+        load_frags(cur, 2, fa[0], fb[0]);
         store_lds(cur ^ 1);
         mfma_slice(1);
-        load_b_frags(cur, 2, fb);
 
-        load_a_frags(cur, 3, fa[1]);
+        load_frags(cur, 3, fa[1], fb[1]);
         load_global(k_next);
         mfma_slice(0);
-        load_b_frags(cur, 3, fb);
 
         if (kGuard && (t % kPollSteps) == kPollSteps - 1 && tid == 0) {
             const bool current = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch;
@@ -231,9 +227,8 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
             if (guard_word == 0) return; // whole group leaves together; nothing was written
         }
 
-        load_a_frags(cur ^ 1, 0, fa[0]);
+        load_frags(cur ^ 1, 0, fa[0], fb[0]);
         mfma_slice(1);
-        load_b_frags(cur ^ 1, 0, fb);
     }
 
 #pragma unroll
