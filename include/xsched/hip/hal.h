@@ -80,6 +80,11 @@ XResult HipMemcpyCommandCreate(HwCommandHandle *cmd, void *dst, const void *src,
 /* hipMemsetAsync. reference hip_command.h:189 */
 XResult HipMemsetCommandCreate(HwCommandHandle *cmd, void *dst, int value, size_t bytes);
 
+/* hipMemsetD16Async / hipMemsetD32Async: `count` elements of `width_bytes` (2 or 4) bytes,
+ * `dst` aligned to the width. reference hip_command.h:190-192 */
+XResult HipMemsetWideCommandCreate(HwCommandHandle *cmd, void *dst, uint32_t value, size_t count,
+                                   uint32_t width_bytes);
+
 /* hipEventRecord(event) in queue order; property Idempotent, always
  * synchronizable. reference hip_command.h:197-219 */
 XResult HipEventRecordCommandCreate(HwCommandHandle *cmd, void *event);
@@ -105,6 +110,15 @@ XResult HipKernelCommandCreate(HwCommandHandle *cmd, const void *host_func,
                                uint32_t block_x, uint32_t block_y, uint32_t block_z,
                                void **args, const size_t *arg_sizes, size_t n_args,
                                uint32_t shared_mem_bytes);
+
+/* hipModuleLaunchKernel of `function` (a hipFunction_t). `packed_args` holds every argument
+ * at its offset in the kernel argument segment (`bytes` in all) and is copied at creation.
+ * reference hip_command.h:124-186 */
+XResult HipModuleKernelCommandCreate(HwCommandHandle *cmd, void *function,
+                                     uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                                     uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                                     uint32_t shared_mem_bytes,
+                                     const void *packed_args, size_t bytes);
 
 #ifdef __cplusplus
 }

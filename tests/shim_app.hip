@@ -1,0 +1,300 @@
+// A plain HIP program that knows nothing of XSched: the interception shim's test subject.
+// It is built twice from this file, once linked against libshimhip.so (shim_app) and once
+// not (shim_app_plain). Both print one line per check; the lines must be equal, and equal
+// to the values computed on the host below.
+//
+//   shim_app [module.co]          the checks (module checks only if a code object is given)
+//   shim_app --bench N            N launches of a tiny kernel on one stream, us per launch
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <chrono>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#define CHECK(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) { \
+    fprintf(stderr, "%s:%d: %s -> %s\n", __FILE__, __LINE__, #expr, hipGetErrorString(e_)); exit(2); } } while (0)
+
+struct Pair { float a; double b; char c; };          // 24 bytes with padding
+struct Wide { uint32_t v[50]; };                      // 200 bytes by value
+
+__device__ uint32_t g_counter;
+
+__global__ void Saxpy(float a, const float *x, float *y, size_t n)
+{
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i < n) y[i] = a * x[i] + y[i];
+}
+
+__global__ void Mixed(Pair p, short s, unsigned char u, double *out, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = p.a + p.b + p.c + s + u + i;
+}
+
+__global__ void SumWide(Wide w, uint32_t *out)
+{
+    uint32_t sum = 0;
+    for (int i = 0; i < 50; ++i) sum += w.v[i] * (uint32_t)(i + 1);
+    out[threadIdx.x] = sum + threadIdx.x;
+}
+
+__global__ void Bump() { if (threadIdx.x == 0 && blockIdx.x == 0) g_counter += 1; }
+
+__global__ void ReadCounter(uint32_t *out) { out[0] = g_counter; }
+
+__global__ void AddInto(uint32_t *dst, const uint32_t *src, uint32_t k, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] += src[i] + k;
+}
+
+// Long enough that work queued behind it is still pending when the host moves on.
+__global__ void Spin(uint32_t *out, uint32_t iters)
+{
+    uint32_t v = threadIdx.x;
+    for (uint32_t i = 0; i < iters; ++i) v = v * 1664525u + 1013904223u;
+    out[threadIdx.x] = v;
+}
+
+static uint64_t Fnv(const void *data, size_t bytes)
+{
+    const uint8_t *p = (const uint8_t *)data;
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < bytes; ++i) { h ^= p[i]; h *= 1099511628211ull; }
+    return h;
+}
+
+static void Report(const char *what, uint64_t got, uint64_t want)
+{
+    printf("%-28s %016llx %s\n", what, (unsigned long long)got, got == want ? "ok" : "MISMATCH");
+}
+
+static void HostFn(void *data) { *(volatile uint32_t *)data = 77; }
+static void Callback(hipStream_t, hipError_t, void *data) { *(volatile uint32_t *)data += 1; }
+
+static int Bench(int launches)
+{
+    hipStream_t s;
+    CHECK(hipStreamCreate(&s));
+    for (int i = 0; i < 200; ++i) Bump<<<1, 64, 0, s>>>();
+    CHECK(hipStreamSynchronize(s));
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < launches; ++i) Bump<<<1, 64, 0, s>>>();
+    const auto t1 = std::chrono::steady_clock::now();
+    CHECK(hipStreamSynchronize(s));
+    const auto t2 = std::chrono::steady_clock::now();
+    const double submit = std::chrono::duration<double, std::micro>(t1 - t0).count() / launches;
+    const double total = std::chrono::duration<double, std::micro>(t2 - t0).count() / launches;
+    printf("bench launches=%d submit_us_per_launch=%.3f total_us_per_launch=%.3f\n", launches, submit, total);
+    CHECK(hipStreamDestroy(s));
+    return 0;
+}
+
+int main(int argc, char **argv)
+{
+    if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
+    const char *module_path = argc >= 2 ? argv[1] : nullptr;
+
+    constexpr size_t n = 1 << 16;
+    hipStream_t s1, s2, s3;
+    CHECK(hipStreamCreate(&s1));
+    CHECK(hipStreamCreateWithFlags(&s2, hipStreamNonBlocking));
+    CHECK(hipStreamCreateWithPriority(&s3, hipStreamDefault, 0));
+
+    // ---- 1. fills of every width, copies from pinned and pageable memory, a kernel chain ----
+    float *x, *y;
+    CHECK(hipMalloc(&x, n * 4)); CHECK(hipMalloc(&y, n * 4));
+    float *pinned, *pinned_out;
+    CHECK(hipHostMalloc(&pinned, n * 4, hipHostMallocDefault));
+    CHECK(hipHostMalloc(&pinned_out, n * 4, hipHostMallocDefault));
+    std::vector<float> pageable(n), want(n);
+    for (size_t i = 0; i < n; ++i) { pinned[i] = (float)(i % 97) * 0.5f; pageable[i] = (float)(i % 13); }
+    CHECK(hipMemcpyAsync(x, pinned, n * 4, hipMemcpyHostToDevice, s1));
+    CHECK(hipMemcpyAsync(y, pageable.data(), n * 4, hipMemcpyHostToDevice, s1));
+    for (size_t i = 0; i < n; ++i) want[i] = pageable[i];
+    for (int rep = 0; rep < 3; ++rep) {
+        Saxpy<<<(n + 255) / 256, 256, 0, s1>>>(2.0f, x, y, n);
+        for (size_t i = 0; i < n; ++i) want[i] = 2.0f * pinned[i] + want[i];
+    }
+    CHECK(hipMemcpyAsync(pinned_out, y, n * 4, hipMemcpyDeviceToHost, s1));
+    CHECK(hipStreamSynchronize(s1));
+    Report("saxpy chain", Fnv(pinned_out, n * 4), Fnv(want.data(), n * 4));
+
+    uint8_t *fills;
+    CHECK(hipMalloc(&fills, 4096));
+    CHECK(hipMemsetAsync(fills, 0xAB, 1024, s1));
+    CHECK(hipMemsetD8Async((hipDeviceptr_t)(fills + 1024), 0x5C, 1024, s1));
+    CHECK(hipMemsetD16Async((hipDeviceptr_t)(fills + 2048), 0xBEEF, 512, s1));
+    CHECK(hipMemsetD32Async((hipDeviceptr_t)(fills + 3072), (int)0xDEADC0DE, 256, s1));
+    std::vector<uint8_t> fills_host(4096), fills_want(4096);
+    CHECK(hipMemcpyAsync(fills_host.data(), fills, 4096, hipMemcpyDeviceToHost, s1)); // pageable destination
+    memset(fills_want.data(), 0xAB, 1024); memset(fills_want.data() + 1024, 0x5C, 1024);
+    for (int i = 0; i < 512; ++i) { const uint16_t v = 0xBEEF; memcpy(&fills_want[2048 + 2 * i], &v, 2); }
+    for (int i = 0; i < 256; ++i) { const uint32_t v = 0xDEADC0DE; memcpy(&fills_want[3072 + 4 * i], &v, 4); }
+    CHECK(hipStreamSynchronize(s1));
+    Report("fills 8/16/32", Fnv(fills_host.data(), 4096), Fnv(fills_want.data(), 4096));
+
+    // ---- 2. arguments of every shape ----------------------------------------------------------
+    double *mixed_out; uint32_t *wide_out;
+    CHECK(hipMalloc(&mixed_out, 512 * 8)); CHECK(hipMalloc(&wide_out, 64 * 4));
+    {
+        Pair p { 1.5f, -2.25, 7 };
+        Wide w;
+        for (int i = 0; i < 50; ++i) w.v[i] = 1000u + 17u * i;
+        Mixed<<<2, 256, 0, s2>>>(p, (short)-300, (unsigned char)200, mixed_out, 512);
+        SumWide<<<1, 64, 0, s2>>>(w, wide_out);
+        p.a = 0; memset(&w, 0, sizeof w); // the launches must have taken copies
+    }
+    std::vector<double> mixed_host(512), mixed_want(512);
+    std::vector<uint32_t> wide_host(64), wide_want(64);
+    CHECK(hipMemcpyDtoHAsync(mixed_host.data(), (hipDeviceptr_t)mixed_out, 512 * 8, s2));
+    CHECK(hipMemcpyDtoHAsync(wide_host.data(), (hipDeviceptr_t)wide_out, 64 * 4, s2));
+    CHECK(hipStreamSynchronize(s2));
+    for (int i = 0; i < 512; ++i) mixed_want[i] = 1.5f + -2.25 + 7 + -300 + 200 + i;
+    uint32_t wsum = 0;
+    for (int i = 0; i < 50; ++i) wsum += (1000u + 17u * i) * (uint32_t)(i + 1);
+    for (int i = 0; i < 64; ++i) wide_want[i] = wsum + i;
+    Report("struct and small scalars", Fnv(mixed_host.data(), 512 * 8), Fnv(mixed_want.data(), 512 * 8));
+    Report("200-byte struct by value", Fnv(wide_host.data(), 64 * 4), Fnv(wide_want.data(), 64 * 4));
+
+    // ---- 3. a kernel without arguments, in order with its neighbours --------------------------
+    uint32_t *counter_out, counter_host = 0, zero = 0;
+    CHECK(hipMalloc(&counter_out, 4));
+    CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_counter), &zero, 4));
+    for (int i = 0; i < 300; ++i) Bump<<<1, 64, 0, s3>>>();
+    ReadCounter<<<1, 1, 0, s3>>>(counter_out);
+    CHECK(hipMemcpyAsync(&counter_host, counter_out, 4, hipMemcpyDeviceToHost, s3));
+    CHECK(hipStreamSynchronize(s3));
+    Report("300 argument-less launches", counter_host, 300);
+
+    // ---- 4. events across streams -------------------------------------------------------------
+    uint32_t *a, *b, *spin;
+    CHECK(hipMalloc(&a, n * 4)); CHECK(hipMalloc(&b, n * 4)); CHECK(hipMalloc(&spin, 256 * 4));
+    CHECK(hipMemsetD32Async((hipDeviceptr_t)a, 5, n, s1));
+    CHECK(hipMemsetD32Async((hipDeviceptr_t)b, 1, n, s2));
+    CHECK(hipStreamSynchronize(s1)); CHECK(hipStreamSynchronize(s2));
+    hipEvent_t start, produced, stop;
+    CHECK(hipEventCreate(&start)); CHECK(hipEventCreate(&produced)); CHECK(hipEventCreate(&stop));
+    CHECK(hipEventRecord(start, s1));
+    Spin<<<1, 256, 0, s1>>>(spin, 2000000);                   // a few milliseconds
+    AddInto<<<n / 256, 256, 0, s1>>>(a, b, 10, n);            // a = 5 + 1 + 10 = 16
+    CHECK(hipEventRecord(produced, s1));
+    CHECK(hipStreamWaitEvent(s2, produced, 0));
+    AddInto<<<n / 256, 256, 0, s2>>>(b, a, 100, n);           // b = 1 + 16 + 100 = 117, only after s1
+    CHECK(hipEventRecord(stop, s2));
+    const hipError_t early = hipEventQuery(stop);
+    CHECK(hipEventSynchronize(stop));
+    float ms = -1.f;
+    CHECK(hipEventElapsedTime(&ms, start, stop));
+    std::vector<uint32_t> b_host(n);
+    CHECK(hipMemcpy(b_host.data(), b, n * 4, hipMemcpyDeviceToHost));
+    uint64_t bad = 0;
+    for (size_t i = 0; i < n; ++i) bad += b_host[i] != 117;
+    Report("cross-stream event order", bad, 0);
+    Report("event query before/after", (uint64_t)(early == hipErrorNotReady || early == hipSuccess) + 2 * (hipEventQuery(stop) == hipSuccess), 3);
+    Report("elapsed time is positive", ms > 0.5f, 1);
+
+    // ---- 5. null-stream work waits for blocking streams ---------------------------------------
+    CHECK(hipMemsetD32Async((hipDeviceptr_t)a, 0, n, s1));
+    Spin<<<1, 256, 0, s1>>>(spin, 1000000);
+    AddInto<<<n / 256, 256, 0, s1>>>(a, b, 3, n);             // a = 0 + 117 + 3 = 120
+    AddInto<<<n / 256, 256>>>(a, a, 0, n);                    // null stream: a = 240, after s1
+    std::vector<uint32_t> a_host(n);
+    CHECK(hipMemcpy(a_host.data(), a, n * 4, hipMemcpyDeviceToHost));
+    bad = 0;
+    for (size_t i = 0; i < n; ++i) bad += a_host[i] != 240;
+    Report("null stream after stream", bad, 0);
+
+    // ---- 6. host functions, stream queries, free behind queued work ----------------------------
+    volatile uint32_t host_word = 0, callback_word = 0;
+    Spin<<<1, 256, 0, s3>>>(spin, 1000000);
+    CHECK(hipLaunchHostFunc(s3, HostFn, (void *)&host_word));
+    CHECK(hipStreamAddCallback(s3, Callback, (void *)&callback_word, 0));
+    while (hipStreamQuery(s3) == hipErrorNotReady) std::this_thread::yield();
+    CHECK(hipStreamSynchronize(s3));
+    Report("host function and callback", host_word + callback_word, 78);
+    uint32_t *temp;
+    CHECK(hipMalloc(&temp, n * 4));
+    CHECK(hipMemsetD32Async((hipDeviceptr_t)temp, 9, n, s1));
+    Spin<<<1, 256, 0, s1>>>(spin, 500000);
+    AddInto<<<n / 256, 256, 0, s1>>>(a, temp, 0, n);          // a = 240 + 9 = 249
+    CHECK(hipFree(temp));                                     // must not pull the memory from under the kernel
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpy(a_host.data(), a, n * 4, hipMemcpyDeviceToHost));
+    bad = 0;
+    for (size_t i = 0; i < n; ++i) bad += a_host[i] != 249;
+    Report("free behind queued work", bad, 0);
+
+    // ---- 7. two threads, each with its own stream ------------------------------------------------
+    {
+        uint32_t *acc[2], *ones;
+        CHECK(hipMalloc(&ones, 1024 * 4));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)ones, 1, 1024, s1));
+        CHECK(hipStreamSynchronize(s1));
+        hipStream_t ts[2] = { s1, s2 };
+        std::thread th[2];
+        for (int t = 0; t < 2; ++t) {
+            CHECK(hipMalloc(&acc[t], 1024 * 4));
+            CHECK(hipMemset(acc[t], 0, 1024 * 4));
+            th[t] = std::thread([&, t]() {
+                for (uint32_t i = 0; i < 400; ++i) AddInto<<<4, 256, 0, ts[t]>>>(acc[t], ones, i * (t + 1), 1024);
+                CHECK(hipStreamSynchronize(ts[t]));
+            });
+        }
+        uint64_t sums = 0;
+        for (int t = 0; t < 2; ++t) {
+            th[t].join();
+            uint32_t first = 0;
+            CHECK(hipMemcpy(&first, acc[t] + 1023, 4, hipMemcpyDeviceToHost));
+            sums = sums * 1000003u + first;
+        }
+        // thread t: sum over i of (1 + i * (t + 1)) = 400 + (t + 1) * 79800
+        Report("two threads, two streams", sums, (uint64_t)(400 + 79800) * 1000003u + (400 + 2 * 79800));
+        CHECK(hipFree(acc[0])); CHECK(hipFree(acc[1])); CHECK(hipFree(ones));
+    }
+
+    // ---- 8. kernels of a loaded module ------------------------------------------------------------
+    if (module_path != nullptr) {
+        hipModule_t mod;
+        hipFunction_t scale, shift;
+        CHECK(hipModuleLoad(&mod, module_path));
+        CHECK(hipModuleGetFunction(&scale, mod, "ModScale"));
+        CHECK(hipModuleGetFunction(&shift, mod, "ModShift"));
+        uint32_t *m;
+        CHECK(hipMalloc(&m, 1024 * 4));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)m, 3, 1024, s1));
+        uint32_t factor = 7, count = 1024;
+        unsigned short add = 11;
+        void *params[] = { &m, &factor, &count };
+        CHECK(hipModuleLaunchKernel(scale, 4, 1, 1, 256, 1, 1, 0, s1, params, nullptr));   // 3 * 7 = 21
+        factor = 0;                                                                          // a copy was taken
+        struct { uint32_t *ptr; unsigned short add; uint32_t count; } packed { m, add, count };
+        size_t packed_bytes = sizeof packed;
+        void *extra[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, &packed, HIP_LAUNCH_PARAM_BUFFER_SIZE, &packed_bytes, HIP_LAUNCH_PARAM_END };
+        CHECK(hipModuleLaunchKernel(shift, 4, 1, 1, 256, 1, 1, 0, s1, nullptr, extra));     // 21 + 11 = 32
+        factor = 2;
+        void *params2[] = { &m, &factor, &count };
+        CHECK(hipExtModuleLaunchKernel(scale, 1024, 1, 1, 256, 1, 1, 0, s1, params2, nullptr, nullptr, nullptr, 0)); // 64
+        std::vector<uint32_t> m_host(1024);
+        CHECK(hipMemcpyAsync(m_host.data(), m, 1024 * 4, hipMemcpyDeviceToHost, s1));
+        CHECK(hipStreamSynchronize(s1));
+        bad = 0;
+        for (int i = 0; i < 1024; ++i) bad += m_host[i] != 64;
+        Report("module kernels", bad, 0);
+        CHECK(hipFree(m));
+        CHECK(hipModuleUnload(mod));
+    }
+
+    CHECK(hipEventDestroy(start)); CHECK(hipEventDestroy(produced)); CHECK(hipEventDestroy(stop));
+    CHECK(hipStreamDestroy(s1)); CHECK(hipStreamDestroy(s2)); CHECK(hipStreamDestroy(s3));
+    CHECK(hipFree(x)); CHECK(hipFree(y)); CHECK(hipFree(fills)); CHECK(hipFree(mixed_out)); CHECK(hipFree(wide_out));
+    CHECK(hipFree(counter_out)); CHECK(hipFree(a)); CHECK(hipFree(b)); CHECK(hipFree(spin));
+    CHECK(hipHostFree(pinned)); CHECK(hipHostFree(pinned_out));
+    printf("done\n");
+    return 0;
+}

@@ -8,7 +8,7 @@ Nothing is computed in Python; every call goes to the native libraries built by
 """
 import ctypes
 import os
-from ctypes import (CFUNCTYPE, POINTER, byref, c_double, c_float, c_int, c_int32, c_int64,
+from ctypes import (CFUNCTYPE, POINTER, byref, c_char_p, c_double, c_float, c_int, c_int32, c_int64,
                     c_size_t, c_uint32, c_uint64, c_void_p)
 
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
@@ -105,12 +105,21 @@ HALHIP_API = {
                                             c_uint32, c_int]),
     "HipMemcpyCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_void_p, c_size_t, c_int]),
     "HipMemsetCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_int, c_size_t]),
+    "HipMemsetWideCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_size_t, c_uint32]),
     "HipEventRecordCommandCreate": (XResult, [POINTER(c_uint64), c_void_p]),
     "HipEventWaitCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32]),
     "HipRecordedEventWaitCommandCreate": (XResult, [POINTER(c_uint64), c_uint64]),
     "HipKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32,
                                          c_uint32, c_uint32, c_uint32, POINTER(c_void_p),
                                          POINTER(c_size_t), c_size_t, c_uint32]),
+    "HipModuleKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32,
+                                               c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_size_t]),
+}
+
+SHIMHIP_API = {
+    "HipShimKernelArgLayout": (XResult, [c_void_p, c_size_t, c_char_p, POINTER(c_uint32), POINTER(c_uint32),
+                                         c_size_t, POINTER(c_size_t)]),
+    "HipShimGetStats": (XResult, [POINTER(c_uint64)]),
 }
 
 
@@ -148,6 +157,20 @@ def halhip():
         _halhip = _load("libhalhip.so")
         _bind(_halhip, HALHIP_API)
     return _halhip
+
+
+_shimhip = None
+
+
+def shimhip():
+    """libshimhip.so: the HIP interception shim. Loaded here only for its two test entry points;
+    a library loaded this way interposes nothing."""
+    global _shimhip
+    if _shimhip is None:
+        halhip()
+        _shimhip = _load("libshimhip.so")
+        _bind(_shimhip, SHIMHIP_API)
+    return _shimhip
 
 
 def check(res, what=""):

@@ -7,6 +7,10 @@ Produces, under xsched_amd/lib/:
     libhalhost.so   CPU hardware-queue adapter                         (g++)
     libhalhip.so    MI355X HIP adapter: Level-1/Level-2 queue, guarded
                     kernels, benchmark harness                         (hipcc, gfx950)
+    libshimhip.so   HIP interception shim: stream work of an unmodified
+                    HIP program becomes XQueue commands                (g++)
+    shim_app, shim_app_plain
+                    the shim's test program with and without the shim  (hipcc)
     xserver         scheduler daemon                                   (g++)
     traffic_probe   counter-run driver for the AXPY kernel             (hipcc)
 and, under oracle/, the checker libraries (see oracle/Makefile).
@@ -41,6 +45,7 @@ PREEMPT_SRCS = [
 ]
 HOST_SRCS = ["host/host_queue.cpp"]
 SERVER_SRCS = ["service/xserver.cpp"]
+SHIM_SRCS = ["shim/code_object.cpp", "shim/hip_shim.cpp"]
 HIP_SRCS = ["hip/hip_queue.hip", "hip/hip_command.hip", "hip/kernels_axpy.hip",
             "hip/kernels_gemm.hip", "hip/kernels_hist.hip", "bench/harness.hip"]
 
@@ -95,6 +100,23 @@ def build_hip(extra, jobs):
         return
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-o", os.path.join(LIB, "libhalhip.so")]
          + objs + ["-L", LIB, "-Wl,-rpath,$ORIGIN", "-lpreempt", "-pthread"])
+    # The shim is host code against the HIP headers. libamdhip64 is named after the adapter so
+    # that a program linked against the shim finds the runtime's entry points behind the shim's.
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    shim_flags = CXXFLAGS + extra + ["-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include"), "-Wno-attributes"]
+    shim_objs = _compile_all("g++", shim_flags, SHIM_SRCS, jobs)
+    _run(["g++", "-shared", "-o", os.path.join(LIB, "libshimhip.so")] + shim_objs
+         + ["-L", LIB, "-Wl,-rpath,$ORIGIN", "-lhalhip", "-lpreempt",
+            "-L", os.path.join(rocm, "lib"), "-Wl,--no-as-needed", "-lamdhip64", "-Wl,--as-needed", "-ldl", "-pthread"])
+    app = os.path.join(ROOT, "tests", "shim_app.hip")
+    if os.path.exists(app):
+        common = ["hipcc"] + HIPFLAGS + [app, "-pthread"]
+        _run(common + ["-o", os.path.join(LIB, "shim_app_plain")])
+        _run(common + ["-o", os.path.join(LIB, "shim_app"), "-L", LIB, "-Wl,-rpath,$ORIGIN",
+                       "-Wl,--no-as-needed", "-lshimhip"])
+    mod = os.path.join(ROOT, "tests", "shim_module.hip")
+    if os.path.exists(mod):
+        _run(["hipcc", "--offload-arch=gfx950", "-O3", "--genco", mod, "-o", os.path.join(LIB, "shim_module.co")])
     probe = os.path.join(CSRC, "bench", "traffic_probe.hip")
     if os.path.exists(probe):
         _run(["hipcc"] + HIPFLAGS + extra + [probe, "-o", os.path.join(LIB, "traffic_probe"),

@@ -39,6 +39,22 @@ private:
     void *dst_; int value_; size_t bytes_;
 };
 
+// Fills of 16- and 32-bit elements (reference hip_command.h:190-192).
+class HipMemsetWideCommand final : public HipCommand
+{
+public:
+    HipMemsetWideCommand(void *dst, uint32_t value, size_t count, uint32_t width)
+        : dst_(dst), value_(value), count_(count), width_(width) {}
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    {
+        if (width_ == 2) return hipMemsetD16Async((hipDeviceptr_t)dst_, (unsigned short)value_, count_, q.Stream());
+        return hipMemsetD32Async((hipDeviceptr_t)dst_, (int)value_, count_, q.Stream());
+    }
+private:
+    void *dst_; uint32_t value_; size_t count_; uint32_t width_;
+};
+
 // The user's event is the marker: always synchronizable (hip_command.h:197-219).
 class HipEventRecordCommand final : public HipCommand
 {
@@ -119,7 +135,39 @@ private:
     std::vector<void *> arg_ptrs_;
 };
 
+// A kernel of a loaded module (hipFunction_t). The arguments arrive as ONE buffer in which
+// every argument already sits at its offset of the kernel argument segment, the form
+// hipModuleLaunchKernel takes through its `extra` list (reference hip_command.h:124-186 keeps
+// the caller's parameter arrays instead and has to know HIP's internal structures for that:
+// kernel_param.cpp:347-390).
+class HipModuleKernelCommand final : public HipCommand
+{
+public:
+    HipModuleKernelCommand(hipFunction_t func, dim3 grid, dim3 block, uint32_t shmem,
+                           const void *packed, size_t bytes)
+        : func_(func), grid_(grid), block_(block), shmem_(shmem)
+        , storage_((const char *)packed, (const char *)packed + bytes) {}
+protected:
+    virtual hipError_t Enqueue(HipQueue &q, bool) override
+    {
+        size_t bytes = storage_.size();
+        void *extra[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, storage_.data(),
+                          HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END };
+        return hipModuleLaunchKernel(func_, grid_.x, grid_.y, grid_.z, block_.x, block_.y, block_.z,
+                                     shmem_, q.Stream(), nullptr, extra);
+    }
+private:
+    hipFunction_t func_; dim3 grid_, block_; uint32_t shmem_;
+    std::vector<char> storage_;
+};
+
 } // namespace
+
+std::shared_ptr<HwCommand> MakeRecordedEventWait(std::shared_ptr<HwCommand> record)
+{
+    if (record == nullptr || dynamic_cast<HipEventRecordCommand *>(record.get()) == nullptr) return nullptr;
+    return std::make_shared<HipRecordedEventWaitCommand>(std::move(record));
+}
 
 } // namespace xsched::hip
 
@@ -137,6 +185,29 @@ EXPORT_C_FUNC XResult HipMemsetCommandCreate(HwCommandHandle *cmd, void *dst, in
 {
     if (cmd == nullptr) return kXSchedErrorInvalidValue;
     *cmd = HwCommandManager::Add(std::make_shared<HipMemsetCommand>(dst, value, bytes));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipMemsetWideCommandCreate(HwCommandHandle *cmd, void *dst, uint32_t value,
+                                                 size_t count, uint32_t width_bytes)
+{
+    if (cmd == nullptr || (width_bytes != 2 && width_bytes != 4)) return kXSchedErrorInvalidValue;
+    if (((uintptr_t)dst & (width_bytes - 1)) != 0) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipMemsetWideCommand>(dst, value, count, width_bytes));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipModuleKernelCommandCreate(HwCommandHandle *cmd, void *function,
+                                                   uint32_t gx, uint32_t gy, uint32_t gz,
+                                                   uint32_t bx, uint32_t by, uint32_t bz,
+                                                   uint32_t shared_mem_bytes,
+                                                   const void *packed_args, size_t bytes)
+{
+    if (cmd == nullptr || function == nullptr || (bytes != 0 && packed_args == nullptr)) return kXSchedErrorInvalidValue;
+    if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || by == 0 || bz == 0 ||
+        (uint64_t)bx * by * bz > 1024) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipModuleKernelCommand>(
+        (hipFunction_t)function, dim3(gx, gy, gz), dim3(bx, by, bz), shared_mem_bytes, packed_args, bytes));
     return kXSchedSuccess;
 }
 

@@ -14,6 +14,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "shim_hooks.h"
 #include "xsched/hip/guard.h"
 #include "xsched/types.h"
 #include "xsched/utils/xassert.h"

@@ -1,0 +1,916 @@
+// libshimhip.so: HIP runtime entry points that route stream work through XQueues.
+//
+// Takes the place of reference platforms/hip/shim/src/{shim,intercept}.cpp. The reference
+// builds a stand-in for the whole of libamdhip64.so (every entry point generated, most of
+// them forwarding); this library defines only the entry points that matter for ordering
+// and sits IN FRONT of the real runtime: the real functions are found with
+// dlsym(RTLD_NEXT). Consequences worked out below:
+//   * The adapter (libhalhip.so) launches through the same names. A call whose return
+//     address lies in the adapter, the XQueue core, this library or the HIP runtime itself
+//     goes straight to the runtime.
+//   * Static constructors of other libraries call __hipRegisterFatBinary before this
+//     library's own constructors have run: all state is created on first use and never
+//     destroyed.
+//   * Whatever cannot be deferred safely is still ORDERED: the XQueue of the stream is
+//     drained and the call is handed to the runtime ("drain + direct"). That covers kernels
+//     whose argument layout is unknown (compressed code objects), copies from pageable host
+//     memory (the runtime reads the buffer before it returns; a deferred copy would read it
+//     later), cooperative launches, host callbacks and stream-ordered allocation.
+//   * Legacy null-stream semantics: work on the null stream waits for the XQueues of all
+//     blocking streams first (the reference keeps a map for this that is never filled:
+//     shim.cpp:21-32).
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <memory>
+#include <mutex>
+#include <shared_mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include <dlfcn.h>
+#include <link.h>
+
+#include <hip/hip_runtime_api.h>
+#include <hip/hip_ext.h>
+
+#include "code_object.h"
+#include "../hip/shim_hooks.h"
+#include "xsched/hip/hal.h"
+#include "xsched/hip/shim.h"
+#include "xsched/utils/log.h"
+#include "xsched/preempt/hal/hw_command.h"
+#include "xsched/preempt/hal/hw_queue.h"
+#include "xsched/preempt/xqueue/xqueue.h"
+
+using namespace xsched::preempt;
+using xsched::hip::codeobj::KernelLayout;
+
+namespace
+{
+
+// ---- the real runtime ----------------------------------------------------------------------
+
+void *RealSymbol(const char *name)
+{
+    void *sym = dlsym(RTLD_NEXT, name);
+    if (sym == nullptr) {
+        // This library was loaded after the runtime (dlopen from a running program): there
+        // is nothing "next", but the runtime is there under its own name.
+        static void *runtime = dlopen("libamdhip64.so", RTLD_NOW | RTLD_NOLOAD);
+        if (runtime == nullptr) runtime = dlopen("libamdhip64.so", RTLD_NOW);
+        if (runtime != nullptr) sym = dlsym(runtime, name);
+    }
+    if (sym == nullptr) {
+        fprintf(stderr, "[xsched shim] the HIP runtime does not export %s\n", name);
+        abort();
+    }
+    return sym;
+}
+
+#define REAL(name) ([]() { static auto fn = (decltype(&::name))RealSymbol(#name); return fn; }())
+// For names the HIP headers also overload with C++ templates: the C signature is spelled out.
+#define REAL_AS(name, ...) ([]() { static auto fn = (hipError_t (*)(__VA_ARGS__))RealSymbol(#name); return fn; }())
+
+// ---- who is calling ------------------------------------------------------------------------
+
+struct CodeRange { uintptr_t lo, hi; };
+
+int CollectRanges(struct dl_phdr_info *info, size_t, void *data)
+{
+    static const char *const kOwn[] = { "libhalhip.so", "libpreempt.so", "libshimhip.so", "libamdhip64.so" };
+    const char *name = info->dlpi_name ? info->dlpi_name : "";
+    const char *base = strrchr(name, '/');
+    base = base ? base + 1 : name;
+    bool own = false;
+    for (const char *lib : kOwn) own = own || strncmp(base, lib, strlen(lib)) == 0;
+    if (!own) return 0;
+    auto *ranges = (std::vector<CodeRange> *)data;
+    for (int i = 0; i < info->dlpi_phnum; ++i) {
+        const auto &ph = info->dlpi_phdr[i];
+        if (ph.p_type == PT_LOAD && (ph.p_flags & PF_X)) {
+            ranges->push_back({ (uintptr_t)(info->dlpi_addr + ph.p_vaddr), (uintptr_t)(info->dlpi_addr + ph.p_vaddr + ph.p_memsz) });
+        }
+    }
+    return 0;
+}
+
+/// True if `ret` is code of the adapter, the XQueue core, this library or the runtime.
+bool FromInside(const void *ret)
+{
+    static const std::vector<CodeRange> *ranges = []() {
+        auto *r = new std::vector<CodeRange>;
+        dl_iterate_phdr(CollectRanges, r);
+        return r;
+    }();
+    const uintptr_t a = (uintptr_t)ret;
+    for (const auto &r : *ranges) if (a >= r.lo && a < r.hi) return true;
+    return false;
+}
+
+#define CALLER_IS_INSIDE() FromInside(__builtin_return_address(0))
+
+// ---- state ---------------------------------------------------------------------------------
+
+struct Stats
+{
+    std::atomic<uint64_t> kernel_cmds { 0 }, kernel_drained { 0 }, kernel_direct { 0 };
+    std::atomic<uint64_t> mem_cmds { 0 }, mem_drained { 0 }, event_cmds { 0 }, event_waits { 0 };
+    std::atomic<uint64_t> known_kernels { 0 };
+};
+
+struct State
+{
+    Stats stats;
+
+    std::shared_mutex code_mtx;
+    // value returned by __hipRegisterFatBinary -> kernels of that binary, by name
+    std::unordered_map<const void *, std::shared_ptr<std::unordered_map<std::string, KernelLayout>>> binaries;
+    std::unordered_map<const void *, std::shared_ptr<const KernelLayout>> host_functions; // kernel stubs
+    std::unordered_map<const void *, std::shared_ptr<std::unordered_map<std::string, KernelLayout>>> modules; // hipModule_t
+    std::unordered_map<const void *, std::shared_ptr<const KernelLayout>> functions;      // hipFunction_t
+
+    std::mutex event_mtx;
+    std::unordered_map<hipEvent_t, std::shared_ptr<HwCommand>> events; // last record command per event
+
+    std::mutex stream_mtx;
+    std::unordered_map<hipStream_t, unsigned> stream_flags; // streams this library has seen created
+};
+
+void PrintStats();
+
+State &S()
+{
+    static State *state = []() {
+        auto *s = new State; // never destroyed: entry points may run during process exit
+        const char *v = getenv("XSCHED_SHIM_STATS");
+        if (v != nullptr && *v != 0 && strcmp(v, "0") != 0) atexit(PrintStats);
+        return s;
+    }();
+    return *state;
+}
+
+void PrintStats()
+{
+    const Stats &t = S().stats;
+    fprintf(stderr, "[xsched shim] kernel_cmds=%lu kernel_drained=%lu kernel_direct=%lu mem_cmds=%lu "
+            "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu\n",
+            (unsigned long)t.kernel_cmds, (unsigned long)t.kernel_drained, (unsigned long)t.kernel_direct,
+            (unsigned long)t.mem_cmds, (unsigned long)t.mem_drained, (unsigned long)t.event_cmds,
+            (unsigned long)t.event_waits, (unsigned long)t.known_kernels);
+}
+
+std::shared_ptr<XQueue> QueueOf(hipStream_t stream)
+{
+    if (stream == nullptr) return nullptr;
+    return HwQueueManager::GetXQueue((HwQueueHandle)(uintptr_t)stream); // reference handle.h:9-12
+}
+
+/// Takes a command out of the handle table and submits it.
+void SubmitHandle(const std::shared_ptr<XQueue> &xq, HwCommandHandle handle)
+{
+    xq->Submit(HwCommandManager::Del(handle));
+}
+
+/// Before work on the null stream: everything queued on blocking streams comes first.
+void WaitBlockingQueues()
+{
+    std::vector<std::shared_ptr<XQueue>> queues;
+    {
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        for (const auto &entry : S().stream_flags) {
+            if (entry.second & hipStreamNonBlocking) continue;
+            if (auto xq = QueueOf(entry.first)) queues.push_back(std::move(xq));
+        }
+    }
+    std::vector<std::shared_ptr<XQueueWaitAllCommand>> waits;
+    for (auto &xq : queues) waits.push_back(xq->SubmitWaitAll());
+    for (auto &w : waits) w->Wait();
+}
+
+// ---- code objects ---------------------------------------------------------------------------
+
+std::shared_ptr<std::unordered_map<std::string, KernelLayout>> ReadImage(const void *image, size_t bytes, const char *what)
+{
+    auto by_name = std::make_shared<std::unordered_map<std::string, KernelLayout>>();
+    std::vector<KernelLayout> kernels;
+    const auto status = xsched::hip::codeobj::ReadKernelLayouts(image, bytes, "gfx950", &kernels);
+    if (status != xsched::hip::codeobj::ParseStatus::kOk) {
+        XWARN("%s: kernel argument layouts not read (%s); its kernels are launched after draining their XQueue",
+              what, xsched::hip::codeobj::ToString(status));
+        return by_name;
+    }
+    for (auto &k : kernels) (*by_name)[k.name] = std::move(k);
+    return by_name;
+}
+
+// What hipcc's registration code passes to __hipRegisterFatBinary.
+struct FatBinaryWrapper { uint32_t magic; uint32_t version; const void *binary; void *unused; };
+constexpr uint32_t kFatBinaryMagic = 0x48495046; // "HIPF"
+
+template <typename Key>
+std::shared_ptr<const KernelLayout> Lookup(std::unordered_map<Key, std::shared_ptr<const KernelLayout>> &map, Key key)
+{
+    std::shared_lock<std::shared_mutex> lock(S().code_mtx);
+    auto it = map.find(key);
+    return it == map.end() ? nullptr : it->second;
+}
+
+// ---- launches -------------------------------------------------------------------------------
+
+/// Every explicit argument copied to its offset: the form hipModuleLaunchKernel's `extra` takes.
+std::vector<char> Pack(const KernelLayout &layout, void **params)
+{
+    std::vector<char> buf(layout.ExplicitBytes(), 0);
+    for (size_t i = 0; i < layout.args.size(); ++i) {
+        memcpy(buf.data() + layout.args[i].offset, params[i], layout.args[i].size);
+    }
+    return buf;
+}
+
+/// The packed argument buffer of an `extra` list, or false if the list has another form.
+bool ExtraBuffer(void **extra, const void **buf, size_t *bytes)
+{
+    *buf = nullptr;
+    const size_t *size_p = nullptr;
+    for (int i = 0; i < 8 && extra[i] != HIP_LAUNCH_PARAM_END; i += 2) {
+        if (extra[i] == HIP_LAUNCH_PARAM_BUFFER_POINTER) *buf = extra[i + 1];
+        else if (extra[i] == HIP_LAUNCH_PARAM_BUFFER_SIZE) size_p = (const size_t *)extra[i + 1];
+        else return false;
+    }
+    if (*buf == nullptr || size_p == nullptr) return false;
+    *bytes = *size_p;
+    return true;
+}
+
+bool SubmitModuleKernel(const std::shared_ptr<XQueue> &xq, hipFunction_t f,
+                        uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,
+                        size_t shmem, void **params, void **extra)
+{
+    HwCommandHandle cmd = 0;
+    XResult res;
+    if (extra != nullptr) {
+        const void *buf;
+        size_t bytes;
+        if (!ExtraBuffer(extra, &buf, &bytes)) return false;
+        res = HipModuleKernelCommandCreate(&cmd, f, gx, gy, gz, bx, by, bz, (uint32_t)shmem, buf, bytes);
+    } else {
+        auto layout = Lookup(S().functions, (const void *)f);
+        if (layout == nullptr || (params == nullptr && !layout->args.empty())) return false;
+        const std::vector<char> packed = Pack(*layout, params);
+        res = HipModuleKernelCommandCreate(&cmd, f, gx, gy, gz, bx, by, bz, (uint32_t)shmem, packed.data(), packed.size());
+    }
+    if (res != kXSchedSuccess) return false;
+    SubmitHandle(xq, cmd);
+    S().stats.kernel_cmds++;
+    return true;
+}
+
+// ---- copies ---------------------------------------------------------------------------------
+
+/// False for host memory the runtime does not know (pageable): a copy from or to it is done
+/// with the caller's buffer before the runtime returns, which a deferred copy cannot keep.
+bool StableForDeferredCopy(const void *ptr)
+{
+    hipPointerAttribute_t attr;
+    if (REAL(hipPointerGetAttributes)(&attr, ptr) != hipSuccess) {
+        (void)REAL(hipGetLastError)(); // the probe must not leave an error behind for the program
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeHost ||
+           attr.type == hipMemoryTypeManaged;
+}
+
+enum class Route { kDirect, kDrained, kCommand };
+
+/// Where a copy on `stream` goes; drains the XQueue when it has to.
+Route RouteCopy(hipStream_t stream, const void *dst, const void *src, hipMemcpyKind kind, std::shared_ptr<XQueue> *xq)
+{
+    if (stream == nullptr) { WaitBlockingQueues(); return Route::kDirect; }
+    *xq = QueueOf(stream);
+    if (*xq == nullptr) return Route::kDirect;
+    const bool deferrable = kind == hipMemcpyDeviceToDevice || (StableForDeferredCopy(dst) && StableForDeferredCopy(src));
+    if (deferrable) return Route::kCommand;
+    (*xq)->WaitAll();
+    S().stats.mem_drained++;
+    return Route::kDrained;
+}
+
+hipError_t CopyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind kind, hipStream_t stream)
+{
+    std::shared_ptr<XQueue> xq;
+    if (RouteCopy(stream, dst, src, kind, &xq) == Route::kCommand) {
+        HwCommandHandle cmd = 0;
+        if (HipMemcpyCommandCreate(&cmd, dst, src, bytes, (int)kind) == kXSchedSuccess) {
+            SubmitHandle(xq, cmd);
+            S().stats.mem_cmds++;
+            return hipSuccess;
+        }
+        xq->WaitAll();
+    }
+    return REAL(hipMemcpyAsync)(dst, src, bytes, kind, stream);
+}
+
+/// Drains the XQueue of `stream` (or the blocking queues for the null stream) so that a call
+/// handed to the runtime next keeps its place in the order.
+void DrainFor(hipStream_t stream)
+{
+    if (stream == nullptr) { WaitBlockingQueues(); return; }
+    if (auto xq = QueueOf(stream)) xq->WaitAll();
+}
+
+hipError_t FillAsync(void *dst, uint32_t value, size_t count, uint32_t width, hipStream_t stream)
+{
+    std::shared_ptr<XQueue> xq;
+    if (stream == nullptr) WaitBlockingQueues();
+    else xq = QueueOf(stream);
+    if (xq != nullptr) {
+        HwCommandHandle cmd = 0;
+        const XResult res = width == 1 ? HipMemsetCommandCreate(&cmd, dst, (int)value, count)
+                                       : HipMemsetWideCommandCreate(&cmd, dst, value, count, width);
+        if (res == kXSchedSuccess) {
+            SubmitHandle(xq, cmd);
+            S().stats.mem_cmds++;
+            return hipSuccess;
+        }
+        xq->WaitAll(); // let the runtime report what is wrong with the arguments
+    }
+    if (width == 1) return REAL(hipMemsetAsync)(dst, (int)value, count, stream);
+    if (width == 2) return REAL(hipMemsetD16Async)((hipDeviceptr_t)dst, (unsigned short)value, count, stream);
+    return REAL(hipMemsetD32Async)((hipDeviceptr_t)dst, (int)value, count, stream);
+}
+
+// ---- streams --------------------------------------------------------------------------------
+
+void OnStreamCreated(hipStream_t stream, unsigned flags)
+{
+    {
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        S().stream_flags[stream] = flags;
+    }
+    (void)XQueueManager::AutoCreate([&](HwQueueHandle *hwq) { return HipQueueCreate(hwq, stream); });
+}
+
+hipError_t RecordEvent(hipEvent_t event, hipStream_t stream, bool with_flags, unsigned flags)
+{
+    auto real = [&]() {
+        return with_flags ? REAL(hipEventRecordWithFlags)(event, stream, flags) : REAL(hipEventRecord)(event, stream);
+    };
+    if (event == nullptr) return real();
+    std::shared_ptr<XQueue> xq;
+    if (stream == nullptr) WaitBlockingQueues();
+    else xq = QueueOf(stream);
+    // Flags other than the default ask for an external-event record; that one is drained for.
+    if (xq != nullptr && with_flags && flags != 0) { xq->WaitAll(); xq = nullptr; }
+    if (xq == nullptr) {
+        {
+            std::lock_guard<std::mutex> lock(S().event_mtx);
+            S().events.erase(event); // the latest record of this event is the runtime's own
+        }
+        return real();
+    }
+    HwCommandHandle handle = 0;
+    if (HipEventRecordCommandCreate(&handle, event) != kXSchedSuccess) { xq->WaitAll(); return real(); }
+    auto cmd = HwCommandManager::Del(handle);
+    {
+        std::lock_guard<std::mutex> lock(S().event_mtx);
+        S().events[event] = cmd;
+    }
+    xq->Submit(cmd);
+    S().stats.event_cmds++;
+    return hipSuccess;
+}
+
+std::shared_ptr<HwCommand> RecordOf(hipEvent_t event)
+{
+    std::lock_guard<std::mutex> lock(S().event_mtx);
+    auto it = S().events.find(event);
+    return it == S().events.end() ? nullptr : it->second;
+}
+
+} // namespace
+
+// ============================================================================================
+// Entry points. Each one first lets calls from inside (adapter, XQueue core, runtime) through.
+// ============================================================================================
+
+extern "C" {
+
+// ---- code registration (reference shim.cpp:100-111) ------------------------------------------
+
+void **__hipRegisterFatBinary(const void *data)
+{
+    void **handle = REAL(__hipRegisterFatBinary)(data);
+    const auto *wrapper = (const FatBinaryWrapper *)data;
+    if (handle != nullptr && wrapper != nullptr && wrapper->magic == kFatBinaryMagic && wrapper->binary != nullptr) {
+        auto kernels = ReadImage(wrapper->binary, 0, "fat binary");
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        S().binaries[(const void *)handle] = std::move(kernels);
+    }
+    return handle;
+}
+
+void __hipRegisterFunction(void **modules, const void *hostFunction, char *deviceFunction,
+                           const char *deviceName, unsigned int threadLimit, uint3 *tid, uint3 *bid,
+                           dim3 *blockDim, dim3 *gridDim, int *wSize)
+{
+    if (deviceName != nullptr) {
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        auto bin = S().binaries.find((const void *)modules);
+        if (bin != S().binaries.end()) {
+            auto k = bin->second->find(deviceName);
+            if (k != bin->second->end()) {
+                S().host_functions[hostFunction] = std::make_shared<const KernelLayout>(k->second);
+                S().stats.known_kernels++;
+            }
+        }
+    }
+    REAL(__hipRegisterFunction)(modules, hostFunction, deviceFunction, deviceName, threadLimit, tid, bid,
+                                blockDim, gridDim, wSize);
+}
+
+hipError_t hipModuleLoadData(hipModule_t *module, const void *image)
+{
+    const hipError_t res = REAL(hipModuleLoadData)(module, image);
+    if (res == hipSuccess && module != nullptr && !CALLER_IS_INSIDE()) {
+        auto kernels = ReadImage(image, 0, "module image");
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        S().modules[(const void *)*module] = std::move(kernels);
+    }
+    return res;
+}
+
+hipError_t hipModuleLoadDataEx(hipModule_t *module, const void *image, unsigned int numOptions,
+                               hipJitOption *options, void **optionValues)
+{
+    const hipError_t res = REAL(hipModuleLoadDataEx)(module, image, numOptions, options, optionValues);
+    if (res == hipSuccess && module != nullptr && !CALLER_IS_INSIDE()) {
+        auto kernels = ReadImage(image, 0, "module image");
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        S().modules[(const void *)*module] = std::move(kernels);
+    }
+    return res;
+}
+
+hipError_t hipModuleLoad(hipModule_t *module, const char *fname)
+{
+    const hipError_t res = REAL(hipModuleLoad)(module, fname);
+    if (res == hipSuccess && module != nullptr && fname != nullptr && !CALLER_IS_INSIDE()) {
+        std::ifstream in(fname, std::ios::binary);
+        const std::vector<char> bytes((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+        auto kernels = ReadImage(bytes.data(), bytes.size(), fname);
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        S().modules[(const void *)*module] = std::move(kernels);
+    }
+    return res;
+}
+
+hipError_t hipModuleGetFunction(hipFunction_t *function, hipModule_t module, const char *kname)
+{
+    const hipError_t res = REAL(hipModuleGetFunction)(function, module, kname);
+    if (res == hipSuccess && function != nullptr && kname != nullptr) {
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        auto mod = S().modules.find((const void *)module);
+        if (mod != S().modules.end()) {
+            auto k = mod->second->find(kname);
+            if (k != mod->second->end()) {
+                S().functions[(const void *)*function] = std::make_shared<const KernelLayout>(k->second);
+                S().stats.known_kernels++;
+            }
+        }
+    }
+    return res;
+}
+
+hipError_t hipModuleUnload(hipModule_t module)
+{
+    if (!CALLER_IS_INSIDE()) {
+        // Launches of its kernels may still sit in XQueues.
+        (void)XQueueManager::ForEachWaitAll();
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        S().modules.erase((const void *)module);
+    }
+    return REAL(hipModuleUnload)(module);
+}
+
+// ---- kernel launches (reference shim.cpp:34-98) ----------------------------------------------
+
+hipError_t hipLaunchKernel(const void *function_address, dim3 numBlocks, dim3 dimBlocks, void **args,
+                           size_t sharedMemBytes, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipLaunchKernel)(function_address, numBlocks, dimBlocks, args, sharedMemBytes, stream);
+    std::shared_ptr<XQueue> xq;
+    if (stream == nullptr) WaitBlockingQueues();
+    else xq = QueueOf(stream);
+    if (xq == nullptr) {
+        S().stats.kernel_direct++;
+        return REAL(hipLaunchKernel)(function_address, numBlocks, dimBlocks, args, sharedMemBytes, stream);
+    }
+    auto layout = Lookup(S().host_functions, function_address);
+    if (layout != nullptr && (args != nullptr || layout->args.empty())) {
+        std::vector<size_t> sizes(layout->args.size());
+        for (size_t i = 0; i < sizes.size(); ++i) sizes[i] = layout->args[i].size;
+        HwCommandHandle cmd = 0;
+        const XResult res = HipKernelCommandCreate(&cmd, function_address, numBlocks.x, numBlocks.y, numBlocks.z,
+                                                   dimBlocks.x, dimBlocks.y, dimBlocks.z, args, sizes.data(),
+                                                   sizes.size(), (uint32_t)sharedMemBytes);
+        if (res == kXSchedSuccess) {
+            SubmitHandle(xq, cmd);
+            S().stats.kernel_cmds++;
+            return hipSuccess;
+        }
+    }
+    xq->WaitAll();
+    S().stats.kernel_drained++;
+    return REAL(hipLaunchKernel)(function_address, numBlocks, dimBlocks, args, sharedMemBytes, stream);
+}
+
+hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gridDimX, unsigned int gridDimY,
+                                 unsigned int gridDimZ, unsigned int blockDimX, unsigned int blockDimY,
+                                 unsigned int blockDimZ, unsigned int sharedMemBytes, hipStream_t stream,
+                                 void **kernelParams, void **extra)
+{
+    auto real = [&]() {
+        return REAL(hipModuleLaunchKernel)(f, gridDimX, gridDimY, gridDimZ, blockDimX, blockDimY, blockDimZ,
+                                           sharedMemBytes, stream, kernelParams, extra);
+    };
+    if (CALLER_IS_INSIDE()) return real();
+    std::shared_ptr<XQueue> xq;
+    if (stream == nullptr) WaitBlockingQueues();
+    else xq = QueueOf(stream);
+    if (xq == nullptr) { S().stats.kernel_direct++; return real(); }
+    if (SubmitModuleKernel(xq, f, gridDimX, gridDimY, gridDimZ, blockDimX, blockDimY, blockDimZ,
+                           sharedMemBytes, kernelParams, extra)) return hipSuccess;
+    xq->WaitAll();
+    S().stats.kernel_drained++;
+    return real();
+}
+
+hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX, uint32_t globalWorkSizeY,
+                                    uint32_t globalWorkSizeZ, uint32_t localWorkSizeX, uint32_t localWorkSizeY,
+                                    uint32_t localWorkSizeZ, size_t sharedMemBytes, hipStream_t hStream,
+                                    void **kernelParams, void **extra, hipEvent_t startEvent,
+                                    hipEvent_t stopEvent, uint32_t flags)
+{
+    auto real = [&]() {
+        return REAL(hipExtModuleLaunchKernel)(f, globalWorkSizeX, globalWorkSizeY, globalWorkSizeZ, localWorkSizeX,
+                                              localWorkSizeY, localWorkSizeZ, sharedMemBytes, hStream, kernelParams,
+                                              extra, startEvent, stopEvent, flags);
+    };
+    if (CALLER_IS_INSIDE()) return real();
+    std::shared_ptr<XQueue> xq;
+    if (hStream == nullptr) WaitBlockingQueues();
+    else xq = QueueOf(hStream);
+    if (xq == nullptr) { S().stats.kernel_direct++; return real(); }
+    // The sizes are in work-items; a launch of whole work-groups without timing events and
+    // flags is an ordinary module launch.
+    const bool plain = startEvent == nullptr && stopEvent == nullptr && flags == 0 &&
+                       localWorkSizeX != 0 && localWorkSizeY != 0 && localWorkSizeZ != 0 &&
+                       globalWorkSizeX % localWorkSizeX == 0 && globalWorkSizeY % localWorkSizeY == 0 &&
+                       globalWorkSizeZ % localWorkSizeZ == 0;
+    if (plain && SubmitModuleKernel(xq, f, globalWorkSizeX / localWorkSizeX, globalWorkSizeY / localWorkSizeY,
+                                    globalWorkSizeZ / localWorkSizeZ, localWorkSizeX, localWorkSizeY,
+                                    localWorkSizeZ, sharedMemBytes, kernelParams, extra)) return hipSuccess;
+    xq->WaitAll();
+    S().stats.kernel_drained++;
+    return real();
+}
+
+hipError_t hipLaunchCooperativeKernel(const void *f, dim3 gridDim, dim3 blockDimX, void **kernelParams,
+                                      unsigned int sharedMemBytes, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) {
+        DrainFor(stream);
+        if (QueueOf(stream) != nullptr) S().stats.kernel_drained++; else S().stats.kernel_direct++;
+    }
+    return REAL_AS(hipLaunchCooperativeKernel, const void *, dim3, dim3, void **, unsigned int, hipStream_t)(f, gridDim, blockDimX, kernelParams, sharedMemBytes, stream);
+}
+
+hipError_t hipExtLaunchKernel(const void *function_address, dim3 numBlocks, dim3 dimBlocks, void **args,
+                              size_t sharedMemBytes, hipStream_t stream, hipEvent_t startEvent,
+                              hipEvent_t stopEvent, int flags)
+{
+    if (!CALLER_IS_INSIDE()) {
+        DrainFor(stream);
+        if (QueueOf(stream) != nullptr) S().stats.kernel_drained++; else S().stats.kernel_direct++;
+    }
+    return REAL(hipExtLaunchKernel)(function_address, numBlocks, dimBlocks, args, sharedMemBytes, stream,
+                                    startEvent, stopEvent, flags);
+}
+
+// ---- memory (reference shim.cpp:113-150, shim.h:37-50) ----------------------------------------
+
+hipError_t hipMemcpyAsync(void *dst, const void *src, size_t sizeBytes, hipMemcpyKind kind, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemcpyAsync)(dst, src, sizeBytes, kind, stream);
+    return CopyAsync(dst, src, sizeBytes, kind, stream);
+}
+
+hipError_t hipMemcpyHtoDAsync(hipDeviceptr_t dst, const void *src, size_t sizeBytes, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemcpyHtoDAsync)(dst, src, sizeBytes, stream);
+    return CopyAsync((void *)dst, src, sizeBytes, hipMemcpyHostToDevice, stream);
+}
+
+hipError_t hipMemcpyDtoHAsync(void *dst, hipDeviceptr_t src, size_t sizeBytes, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemcpyDtoHAsync)(dst, src, sizeBytes, stream);
+    return CopyAsync(dst, (const void *)src, sizeBytes, hipMemcpyDeviceToHost, stream);
+}
+
+hipError_t hipMemcpyDtoDAsync(hipDeviceptr_t dst, hipDeviceptr_t src, size_t sizeBytes, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemcpyDtoDAsync)(dst, src, sizeBytes, stream);
+    return CopyAsync((void *)dst, (const void *)src, sizeBytes, hipMemcpyDeviceToDevice, stream);
+}
+
+// The copy is complete when this call returns, so there is nothing to defer
+// (reference shim.cpp:136-150).
+hipError_t hipMemcpyWithStream(void *dst, const void *src, size_t sizeBytes, hipMemcpyKind kind, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipMemcpyWithStream)(dst, src, sizeBytes, kind, stream);
+}
+
+hipError_t hipMemcpy2DAsync(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width,
+                            size_t height, hipMemcpyKind kind, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipMemcpy2DAsync)(dst, dpitch, src, spitch, width, height, kind, stream);
+}
+
+hipError_t hipMemcpyPeerAsync(void *dst, int dstDeviceId, const void *src, int srcDevice, size_t sizeBytes,
+                              hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipMemcpyPeerAsync)(dst, dstDeviceId, src, srcDevice, sizeBytes, stream);
+}
+
+// The synchronous calls work on the null stream.
+hipError_t hipMemcpy(void *dst, const void *src, size_t sizeBytes, hipMemcpyKind kind)
+{
+    if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
+    return REAL(hipMemcpy)(dst, src, sizeBytes, kind);
+}
+
+hipError_t hipMemset(void *dst, int value, size_t sizeBytes)
+{
+    if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
+    return REAL(hipMemset)(dst, value, sizeBytes);
+}
+
+hipError_t hipMemsetAsync(void *dst, int value, size_t sizeBytes, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemsetAsync)(dst, value, sizeBytes, stream);
+    return FillAsync(dst, (uint32_t)value, sizeBytes, 1, stream);
+}
+
+hipError_t hipMemsetD8Async(hipDeviceptr_t dest, unsigned char value, size_t count, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemsetD8Async)(dest, value, count, stream);
+    return FillAsync((void *)dest, value, count, 1, stream);
+}
+
+hipError_t hipMemsetD16Async(hipDeviceptr_t dest, unsigned short value, size_t count, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemsetD16Async)(dest, value, count, stream);
+    return FillAsync((void *)dest, value, count, 2, stream);
+}
+
+hipError_t hipMemsetD32Async(hipDeviceptr_t dst, int value, size_t count, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipMemsetD32Async)(dst, value, count, stream);
+    return FillAsync((void *)dst, (uint32_t)value, count, 4, stream);
+}
+
+// Commands that still sit in an XQueue may use the memory: they go first (reference
+// shim.cpp:121-127). Allocation does not touch queued work and is left alone.
+hipError_t hipFree(void *ptr)
+{
+    if (!CALLER_IS_INSIDE()) (void)XQueueManager::ForEachWaitAll();
+    return REAL(hipFree)(ptr);
+}
+
+hipError_t hipFreeAsync(void *dev_ptr, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipFreeAsync)(dev_ptr, stream);
+}
+
+hipError_t hipMallocAsync(void **dev_ptr, size_t size, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL_AS(hipMallocAsync, void **, size_t, hipStream_t)(dev_ptr, size, stream);
+}
+
+// ---- events (reference shim.cpp:152-257) ------------------------------------------------------
+
+hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipEventRecord)(event, stream);
+    return RecordEvent(event, stream, false, 0);
+}
+
+hipError_t hipEventRecordWithFlags(hipEvent_t event, hipStream_t stream, unsigned int flags)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipEventRecordWithFlags)(event, stream, flags);
+    return RecordEvent(event, stream, true, flags);
+}
+
+hipError_t hipEventQuery(hipEvent_t event)
+{
+    if (!CALLER_IS_INSIDE()) {
+        if (auto record = RecordOf(event)) {
+            return record->GetState() >= kCommandStateCompleted ? hipSuccess : hipErrorNotReady;
+        }
+    }
+    return REAL(hipEventQuery)(event);
+}
+
+hipError_t hipEventSynchronize(hipEvent_t event)
+{
+    if (!CALLER_IS_INSIDE()) {
+        if (auto record = RecordOf(event)) { record->Wait(); return hipSuccess; }
+    }
+    return REAL(hipEventSynchronize)(event);
+}
+
+hipError_t hipEventElapsedTime(float *ms, hipEvent_t start, hipEvent_t stop)
+{
+    if (!CALLER_IS_INSIDE()) {
+        // A record that has not reached the stream yet reads as "not ready" here as it would there.
+        for (hipEvent_t e : { start, stop }) {
+            auto record = RecordOf(e);
+            if (record != nullptr && record->GetState() < kCommandStateCompleted) return hipErrorNotReady;
+        }
+    }
+    return REAL(hipEventElapsedTime)(ms, start, stop);
+}
+
+hipError_t hipEventDestroy(hipEvent_t event)
+{
+    if (!CALLER_IS_INSIDE()) {
+        std::shared_ptr<HwCommand> record;
+        {
+            std::lock_guard<std::mutex> lock(S().event_mtx);
+            auto it = S().events.find(event);
+            if (it != S().events.end()) { record = it->second; S().events.erase(it); }
+        }
+        // The record command may still be waiting in its XQueue, and a replay after a level-2
+        // flush records the event again: it has to exist until the command has completed.
+        if (record != nullptr) record->Wait();
+    }
+    return REAL(hipEventDestroy)(event);
+}
+
+hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int flags)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipStreamWaitEvent)(stream, event, flags);
+    auto record = RecordOf(event);
+    if (record == nullptr) {
+        // Recorded by the runtime itself (or never): the runtime orders it, but only against
+        // what the waiting stream has been handed, so the wait keeps its place through a command.
+        std::shared_ptr<XQueue> xq = QueueOf(stream);
+        HwCommandHandle cmd = 0;
+        if (xq != nullptr && HipEventWaitCommandCreate(&cmd, event, flags) == kXSchedSuccess) {
+            SubmitHandle(xq, cmd);
+            return hipSuccess;
+        }
+        if (stream == nullptr) WaitBlockingQueues();
+        return REAL(hipStreamWaitEvent)(stream, event, flags);
+    }
+    S().stats.event_waits++;
+    std::shared_ptr<XQueue> xq = QueueOf(stream);
+    if (xq != nullptr) {
+        if (auto wait = xsched::hip::MakeRecordedEventWait(record)) {
+            xq->Submit(wait);
+            return hipSuccess;
+        }
+    }
+    // The waiting stream is the null stream or has no XQueue: wait here, on the host, for
+    // the record command, then let the runtime order the rest (reference shim.cpp:221-240).
+    if (stream == nullptr) WaitBlockingQueues();
+    record->Wait();
+    return REAL(hipStreamWaitEvent)(stream, event, flags);
+}
+
+// ---- streams (reference shim.cpp:259-320) -----------------------------------------------------
+
+hipError_t hipStreamCreate(hipStream_t *stream)
+{
+    const hipError_t res = REAL(hipStreamCreate)(stream);
+    if (res == hipSuccess && stream != nullptr && !CALLER_IS_INSIDE()) OnStreamCreated(*stream, hipStreamDefault);
+    return res;
+}
+
+hipError_t hipStreamCreateWithFlags(hipStream_t *stream, unsigned int flags)
+{
+    const hipError_t res = REAL(hipStreamCreateWithFlags)(stream, flags);
+    if (res == hipSuccess && stream != nullptr && !CALLER_IS_INSIDE()) OnStreamCreated(*stream, flags);
+    return res;
+}
+
+hipError_t hipStreamCreateWithPriority(hipStream_t *stream, unsigned int flags, int priority)
+{
+    const hipError_t res = REAL(hipStreamCreateWithPriority)(stream, flags, priority);
+    if (res == hipSuccess && stream != nullptr && !CALLER_IS_INSIDE()) OnStreamCreated(*stream, flags);
+    return res;
+}
+
+hipError_t hipStreamDestroy(hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) {
+        bool known;
+        {
+            std::lock_guard<std::mutex> lock(S().stream_mtx);
+            known = S().stream_flags.erase(stream) != 0;
+        }
+        if (known && QueueOf(stream) != nullptr) (void)XQueueManager::AutoDestroy((HwQueueHandle)(uintptr_t)stream);
+    }
+    return REAL(hipStreamDestroy)(stream);
+}
+
+hipError_t hipStreamSynchronize(hipStream_t stream)
+{
+    if (CALLER_IS_INSIDE()) return REAL(hipStreamSynchronize)(stream);
+    if (stream == nullptr) { WaitBlockingQueues(); return REAL(hipStreamSynchronize)(stream); }
+    auto xq = QueueOf(stream);
+    if (xq == nullptr) return REAL(hipStreamSynchronize)(stream);
+    xq->WaitAll();
+    return hipSuccess;
+}
+
+hipError_t hipStreamQuery(hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) {
+        // An XQueue is idle once everything has been handed to the stream; whether the device
+        // is done with it is the runtime's to say (the reference answers hipSuccess for an
+        // idle XQueue: shim.cpp:267-280).
+        if (auto xq = QueueOf(stream)) {
+            if (xq->Query() == kQueueStateReady) return hipErrorNotReady;
+        }
+    }
+    return REAL(hipStreamQuery)(stream);
+}
+
+hipError_t hipStreamAddCallback(hipStream_t stream, hipStreamCallback_t callback, void *userData, unsigned int flags)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipStreamAddCallback)(stream, callback, userData, flags);
+}
+
+hipError_t hipLaunchHostFunc(hipStream_t stream, hipHostFn_t fn, void *userData)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipLaunchHostFunc)(stream, fn, userData);
+}
+
+hipError_t hipDeviceSynchronize(void)
+{
+    if (!CALLER_IS_INSIDE()) (void)XQueueManager::ForEachWaitAll();
+    return REAL(hipDeviceSynchronize)();
+}
+
+#pragma GCC diagnostic push
+#pragma GCC diagnostic ignored "-Wdeprecated-declarations"
+hipError_t hipCtxSynchronize(void)
+{
+    if (!CALLER_IS_INSIDE()) (void)XQueueManager::ForEachWaitAll();
+    return REAL(hipCtxSynchronize)();
+}
+#pragma GCC diagnostic pop
+
+// ---- for tests and tools ----------------------------------------------------------------------
+
+XResult HipShimKernelArgLayout(const void *image, size_t bytes, const char *kernel, uint32_t *offsets,
+                               uint32_t *sizes, size_t cap, size_t *n_args)
+{
+    using xsched::hip::codeobj::ParseStatus;
+    if (image == nullptr || kernel == nullptr || n_args == nullptr) return kXSchedErrorInvalidValue;
+    if (cap != 0 && (offsets == nullptr || sizes == nullptr)) return kXSchedErrorInvalidValue;
+    std::vector<KernelLayout> kernels;
+    const ParseStatus status = xsched::hip::codeobj::ReadKernelLayouts(image, bytes, "gfx950", &kernels);
+    if (status == ParseStatus::kCompressed) return kXSchedErrorNotSupported;
+    if (status != ParseStatus::kOk) return kXSchedErrorInvalidValue;
+    for (const auto &k : kernels) {
+        if (k.name != kernel) continue;
+        *n_args = k.args.size();
+        for (size_t i = 0; i < k.args.size() && i < cap; ++i) { offsets[i] = k.args[i].offset; sizes[i] = k.args[i].size; }
+        return kXSchedSuccess;
+    }
+    return kXSchedErrorNotFound;
+}
+
+XResult HipShimGetStats(uint64_t *out)
+{
+    if (out == nullptr) return kXSchedErrorInvalidValue;
+    const Stats &t = S().stats;
+    out[0] = t.kernel_cmds; out[1] = t.kernel_drained; out[2] = t.kernel_direct; out[3] = t.mem_cmds;
+    out[4] = t.mem_drained; out[5] = t.event_cmds; out[6] = t.event_waits; out[7] = t.known_kernels;
+    return kXSchedSuccess;
+}
+
+} // extern "C"
