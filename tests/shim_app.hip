@@ -5,9 +5,12 @@
 //
 //   shim_app [module.co]          the checks (module checks only if a code object is given)
 //   shim_app --bench N            N launches of a tiny kernel on one stream, us per launch
+//   shim_app --load SECONDS       device-filling kernels back to back on one stream
+//   shim_app --probe N PERIOD_US  a short kernel every PERIOD_US, launch-to-completion latency
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdint>
 #include <cstdio>
@@ -95,9 +98,67 @@ static int Bench(int launches)
     return 0;
 }
 
+// Every thread runs `iters` dependent steps: with 2048 x 256 threads (all resident at once)
+// the device is full for about a millisecond at 30000 steps.
+__global__ void Busy(uint32_t *out, uint32_t iters)
+{
+    uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint32_t i = 0; i < iters; ++i) v = v * 1664525u + 1013904223u;
+    if (v == 0x12345678u) out[0] = v; // keeps the loop; practically never true
+}
+
+static int Load(double seconds)
+{
+    hipStream_t s;
+    uint32_t *out;
+    CHECK(hipStreamCreate(&s));
+    CHECK(hipMalloc(&out, 4));
+    printf("ready\n"); fflush(stdout);
+    const auto t0 = std::chrono::steady_clock::now();
+    uint64_t kernels = 0;
+    while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < seconds) {
+        for (int i = 0; i < 32; ++i) Busy<<<2048, 256, 0, s>>>(out, 30000);
+        CHECK(hipStreamSynchronize(s));
+        kernels += 32;
+    }
+    const double elapsed = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    printf("load kernels=%llu ms_per_kernel=%.3f\n", (unsigned long long)kernels, elapsed * 1e3 / kernels);
+    CHECK(hipFree(out));
+    CHECK(hipStreamDestroy(s));
+    return 0;
+}
+
+static int Probe(int count, int period_us)
+{
+    hipStream_t s;
+    uint32_t *out;
+    CHECK(hipStreamCreate(&s));
+    CHECK(hipMalloc(&out, 4));
+    for (int i = 0; i < 20; ++i) Busy<<<256, 256, 0, s>>>(out, 5000);
+    CHECK(hipStreamSynchronize(s));
+    printf("ready\n"); fflush(stdout);
+    std::vector<double> us(count);
+    for (int i = 0; i < count; ++i) {
+        const auto t0 = std::chrono::steady_clock::now();
+        Busy<<<256, 256, 0, s>>>(out, 5000);
+        CHECK(hipStreamSynchronize(s));
+        us[i] = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+        std::this_thread::sleep_for(std::chrono::microseconds(period_us));
+    }
+    std::sort(us.begin(), us.end());
+    // percentile p = sorted[floor(p * n)]
+    printf("probe n=%d p50_us=%.1f p99_us=%.1f max_us=%.1f\n", count, us[(size_t)(0.5 * count)],
+           us[(size_t)(0.99 * count)], us.back());
+    CHECK(hipFree(out));
+    CHECK(hipStreamDestroy(s));
+    return 0;
+}
+
 int main(int argc, char **argv)
 {
     if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
+    if (argc >= 3 && strcmp(argv[1], "--load") == 0) return Load(atof(argv[2]));
+    if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));
     const char *module_path = argc >= 2 ? argv[1] : nullptr;
 
     constexpr size_t n = 1 << 16;

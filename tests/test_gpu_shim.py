@@ -93,3 +93,81 @@ def test_launch_cost_through_the_shim():
     print(f"launch cost: plain submit {plain[0]:.2f} us, total {plain[1]:.2f} us per launch; "
           f"through the shim submit {through[0]:.2f} us, total {through[1]:.2f} us", file=sys.stderr, flush=True)
     assert through[1] < 60.0  # a regression guard, not a claim; typical values are far below
+
+
+def test_unmodified_binary_under_ld_preload(plain_output):
+    """The way a user runs a program that was not linked against the shim."""
+    shim = os.path.join(LIB, "libshimhip.so")
+    preload = " ".join(x for x in (os.environ.get("LD_PRELOAD", ""), shim) if x)
+    out, err = run("shim_app_plain", [MODULE], shim_env(1, LD_PRELOAD=preload))
+    assert out == plain_output
+    s = stats_of(err)
+    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 0
+
+
+def _percentiles(out):
+    m = re.search(r"probe n=(\d+) p50_us=([\d.]+) p99_us=([\d.]+) max_us=([\d.]+)", out)
+    assert m, out
+    return float(m.group(2)), float(m.group(3))
+
+
+def test_two_unmodified_processes_under_the_daemon():
+    """Two processes that know nothing of XSched, one filling the device with back-to-back
+    kernels (priority 0), one launching a short kernel every 2 ms (priority 1), both through the
+    shim and the scheduler daemon with HPF (reference examples/Linux/1_transparent_sched). The
+    low-priority process's queue must get suspended while the other has work; the latencies of
+    the short kernel alone, next to the other process without XSched, and under XSched are
+    printed for the record."""
+    import tempfile
+    import time
+    xserver = os.path.join(LIB, "xserver")
+    sock_dir = tempfile.mkdtemp(prefix="xsched-shim-")
+    base = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+
+    def start(binary, args, extra):
+        print(f"starting {binary} {args} with {extra}", flush=True)
+        return subprocess.Popen([os.path.join(LIB, binary)] + args, env=dict(base, **extra),
+                                stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+
+    def wait_ready(proc):
+        assert proc.stdout.readline().strip() == "ready"
+
+    # the short kernel alone
+    alone, _ = run("shim_app_plain", ["--probe", "300", "2000"], {})
+    # next to the other process, hardware scheduling only
+    load = start("shim_app_plain", ["--load", "1.6"], {})
+    wait_ready(load)
+    native, _ = run("shim_app_plain", ["--probe", "300", "2000"], {})
+    load_out, _ = load.communicate(timeout=60)
+    assert load.returncode == 0, load_out
+
+    server = subprocess.Popen([xserver, "HPF"], env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN"))
+    try:
+        deadline = time.time() + 5
+        while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
+            time.sleep(0.01)
+        assert os.path.exists(os.path.join(sock_dir, "xsched-1.sock")), "xserver did not come up"
+        common = {"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
+                  "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}
+        load = start("shim_app", ["--load", "1.6"], dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0",
+                                                        XSCHED_AUTO_XQUEUE_THRESHOLD="2", XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"))
+        wait_ready(load)
+        probe = start("shim_app", ["--probe", "300", "2000"], dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
+        probe_out, probe_err = probe.communicate(timeout=60)
+        load_out2, load_err = load.communicate(timeout=60)
+        assert probe.returncode == 0 and load.returncode == 0, (probe_err[-1000:], load_err[-1000:])
+    finally:
+        server.terminate()
+        try:
+            server.wait(timeout=5)
+        except subprocess.TimeoutExpired:
+            server.kill()
+    ls, ps = stats_of(load_err), stats_of(probe_err)
+    a, n, x = _percentiles(alone), _percentiles(native), _percentiles(probe_out)
+    print(f"short kernel p50/p99 us: alone {a[0]:.0f}/{a[1]:.0f}, next to the load without XSched {n[0]:.0f}/{n[1]:.0f}, "
+          f"under XSched {x[0]:.0f}/{x[1]:.0f}; load: {load_out.strip().splitlines()[-1]} | under XSched "
+          f"{load_out2.strip().splitlines()[-1]}; load queue deactivations {ls['deactivations']}",
+          file=sys.stderr, flush=True)
+    assert ps["deactivations"] == 0, "the high-priority process was suspended"
+    assert ls["deactivations"] > 50 and ls["reactivations"] > 50, "the daemon never suspended the low-priority process"
+    assert ps["kernel_cmds"] >= 300 and ls["kernel_cmds"] >= 32

@@ -103,7 +103,7 @@ def build_hip(extra, jobs):
     # The shim is host code against the HIP headers. libamdhip64 is named after the adapter so
     # that a program linked against the shim finds the runtime's entry points behind the shim's.
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    shim_flags = CXXFLAGS + extra + ["-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include"), "-Wno-attributes"]
+    shim_flags = CXXFLAGS + extra + ["-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include")]
     shim_objs = _compile_all("g++", shim_flags, SHIM_SRCS, jobs)
     _run(["g++", "-shared", "-o", os.path.join(LIB, "libshimhip.so")] + shim_objs
          + ["-L", LIB, "-Wl,-rpath,$ORIGIN", "-lhalhip", "-lpreempt",

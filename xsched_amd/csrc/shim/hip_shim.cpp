@@ -35,7 +35,6 @@
 #include <link.h>
 
 #include <hip/hip_runtime_api.h>
-#include <hip/hip_ext.h>
 
 #include "code_object.h"
 #include "../hip/shim_hooks.h"
@@ -120,6 +119,8 @@ struct Stats
     std::atomic<uint64_t> kernel_cmds { 0 }, kernel_drained { 0 }, kernel_direct { 0 };
     std::atomic<uint64_t> mem_cmds { 0 }, mem_drained { 0 }, event_cmds { 0 }, event_waits { 0 };
     std::atomic<uint64_t> known_kernels { 0 };
+    // summed over the hardware queues of streams at their destruction
+    std::atomic<uint64_t> queue_launches { 0 }, deactivations { 0 }, reactivations { 0 };
 };
 
 struct State
@@ -157,10 +158,12 @@ void PrintStats()
 {
     const Stats &t = S().stats;
     fprintf(stderr, "[xsched shim] kernel_cmds=%lu kernel_drained=%lu kernel_direct=%lu mem_cmds=%lu "
-            "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu\n",
+            "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu queue_launches=%lu "
+            "deactivations=%lu reactivations=%lu\n",
             (unsigned long)t.kernel_cmds, (unsigned long)t.kernel_drained, (unsigned long)t.kernel_direct,
             (unsigned long)t.mem_cmds, (unsigned long)t.mem_drained, (unsigned long)t.event_cmds,
-            (unsigned long)t.event_waits, (unsigned long)t.known_kernels);
+            (unsigned long)t.event_waits, (unsigned long)t.known_kernels, (unsigned long)t.queue_launches,
+            (unsigned long)t.deactivations, (unsigned long)t.reactivations);
 }
 
 std::shared_ptr<XQueue> QueueOf(hipStream_t stream)
@@ -549,6 +552,7 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gridDimX, unsigne
     return real();
 }
 
+// Declared in hip/hip_ext.h, which g++ does not take without diagnostics; the signature is the one there.
 hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX, uint32_t globalWorkSizeY,
                                     uint32_t globalWorkSizeZ, uint32_t localWorkSizeX, uint32_t localWorkSizeY,
                                     uint32_t localWorkSizeZ, size_t sharedMemBytes, hipStream_t hStream,
@@ -556,7 +560,8 @@ hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX, u
                                     hipEvent_t stopEvent, uint32_t flags)
 {
     auto real = [&]() {
-        return REAL(hipExtModuleLaunchKernel)(f, globalWorkSizeX, globalWorkSizeY, globalWorkSizeZ, localWorkSizeX,
+        return REAL_AS(hipExtModuleLaunchKernel, hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                       uint32_t, size_t, hipStream_t, void **, void **, hipEvent_t, hipEvent_t, uint32_t)(f, globalWorkSizeX, globalWorkSizeY, globalWorkSizeZ, localWorkSizeX,
                                               localWorkSizeY, localWorkSizeZ, sharedMemBytes, hStream, kernelParams,
                                               extra, startEvent, stopEvent, flags);
     };
@@ -828,7 +833,17 @@ hipError_t hipStreamDestroy(hipStream_t stream)
             std::lock_guard<std::mutex> lock(S().stream_mtx);
             known = S().stream_flags.erase(stream) != 0;
         }
-        if (known && QueueOf(stream) != nullptr) (void)XQueueManager::AutoDestroy((HwQueueHandle)(uintptr_t)stream);
+        if (known && QueueOf(stream) != nullptr) {
+            const HwQueueHandle hwq = (HwQueueHandle)(uintptr_t)stream;
+            QueueOf(stream)->WaitAll();
+            uint64_t counters[8] = {};
+            if (HipQueueGetStats(hwq, counters) == kXSchedSuccess) {
+                S().stats.queue_launches += counters[0];
+                S().stats.deactivations += counters[2];
+                S().stats.reactivations += counters[3];
+            }
+            (void)XQueueManager::AutoDestroy(hwq);
+        }
     }
     return REAL(hipStreamDestroy)(stream);
 }
