@@ -7,6 +7,7 @@
 //   shim_app --bench N            N launches of a tiny kernel on one stream, us per launch
 //   shim_app --load SECONDS       device-filling kernels back to back on one stream
 //   shim_app --probe N PERIOD_US  a short kernel every PERIOD_US, launch-to-completion latency
+//   shim_app --leak               leaves main() with streams, events and memory never released
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
@@ -154,8 +155,30 @@ static int Probe(int count, int period_us)
     return 0;
 }
 
+// What many programs do: nothing is destroyed, the last work is synchronised by an event only.
+static int Leak()
+{
+    hipStream_t s[2];
+    hipEvent_t done;
+    uint32_t *out, host = 0;
+    CHECK(hipStreamCreate(&s[0])); CHECK(hipStreamCreateWithFlags(&s[1], hipStreamNonBlocking));
+    CHECK(hipEventCreate(&done));
+    CHECK(hipMalloc(&out, 4));
+    uint32_t zero = 0;
+    CHECK(hipMemcpyToSymbol(HIP_SYMBOL(g_counter), &zero, 4));
+    for (int i = 0; i < 100; ++i) Bump<<<1, 64, 0, s[0]>>>();
+    ReadCounter<<<1, 1, 0, s[0]>>>(out);
+    CHECK(hipEventRecord(done, s[0]));
+    Busy<<<64, 256, 0, s[1]>>>(out + 0, 1000);   // never waited for
+    CHECK(hipEventSynchronize(done));
+    CHECK(hipMemcpy(&host, out, 4, hipMemcpyDeviceToHost));
+    printf("leak counter=%u\n", host);
+    return host == 100 ? 0 : 3;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc >= 2 && strcmp(argv[1], "--leak") == 0) return Leak();
     if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
     if (argc >= 3 && strcmp(argv[1], "--load") == 0) return Load(atof(argv[2]));
     if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));

@@ -171,3 +171,14 @@ def test_two_unmodified_processes_under_the_daemon():
     assert ps["deactivations"] == 0, "the high-priority process was suspended"
     assert ls["deactivations"] > 50 and ls["reactivations"] > 50, "the daemon never suspended the low-priority process"
     assert ps["kernel_cmds"] >= 300 and ls["kernel_cmds"] >= 32
+
+
+@pytest.mark.parametrize("level", [1, 2])
+def test_program_that_releases_nothing_exits_cleanly(level):
+    """Streams, events and memory are never released and one stream still has work when main()
+    returns: the process must end with the program's own exit code."""
+    out, _ = run("shim_app_plain", ["--leak"], {})
+    assert "leak counter=100" in out
+    out, err = run("shim_app", ["--leak"], shim_env(level))
+    assert "leak counter=100" in out
+    assert stats_of(err)["kernel_cmds"] == 102
