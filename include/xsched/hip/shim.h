@@ -13,9 +13,9 @@
  * Intercepted:
  *   kernels   hipLaunchKernel, hipModuleLaunchKernel, hipExtModuleLaunchKernel,
  *             hipLaunchCooperativeKernel, hipExtLaunchKernel              (shim.cpp:34-98)
- *   code      __hipRegisterFatBinary, __hipRegisterFunction, hipModuleLoad,
- *             hipModuleLoadData, hipModuleLoadDataEx, hipModuleGetFunction,
- *             hipModuleUnload                                             (shim.cpp:100-111)
+ *   code      __hipRegisterFatBinary, __hipRegisterFunction, __hipUnregisterFatBinary,
+ *             hipModuleLoad, hipModuleLoadData, hipModuleLoadDataEx,
+ *             hipModuleGetFunction, hipModuleUnload                       (shim.cpp:100-111)
  *   memory    hipMemcpyAsync, hipMemcpyWithStream, hipMemcpyHtoDAsync, hipMemcpyDtoHAsync,
  *             hipMemcpyDtoDAsync, hipMemcpy2DAsync, hipMemcpyPeerAsync, hipMemsetAsync,
  *             hipMemsetD8Async, hipMemsetD16Async, hipMemsetD32Async, hipMemcpy, hipMemset,
@@ -38,11 +38,12 @@ extern "C" {
 #endif
 
 /* The explicit arguments of `kernel` (its mangled name) as the code object `image` of
- * `bytes` bytes records them: a clang offload bundle as hipcc embeds it, or a bare AMDGPU
- * ELF file. Writes up to `cap` (offset, size) pairs and the argument count to `n_args`.
- * NotFound: no such kernel; NotSupported: compressed bundle; InvalidValue: not a code
- * object, or malformed. Takes the place of the comgr walk in reference
- * platforms/hip/hal/src/kernel_param.cpp:256-345. */
+ * `bytes` bytes records them: a clang offload bundle as hipcc embeds it (plain, or
+ * compressed with zstd or zlib), or a bare AMDGPU ELF file. Writes up to `cap`
+ * (offset, size) pairs and the argument count to `n_args`. NotFound: no such kernel;
+ * NotSupported: a compressed bundle that cannot be unpacked on this machine (no libzstd /
+ * libz); InvalidValue: not a code object, or malformed. Takes the place of the comgr walk
+ * in reference platforms/hip/hal/src/kernel_param.cpp:256-345. */
 XResult HipShimKernelArgLayout(const void *image, size_t bytes, const char *kernel,
                                uint32_t *offsets, uint32_t *sizes, size_t cap, size_t *n_args);
 

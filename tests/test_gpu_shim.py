@@ -73,6 +73,15 @@ def test_same_results_through_xqueues(plain_output, level, threshold, batch):
     assert s["mem_cmds"] >= 2 + 4 + 4 and s["mem_drained"] >= 5
 
 
+def test_program_with_compressed_device_code(plain_output):
+    """Large applications ship their code objects compressed; the launches must still become
+    commands (their argument layouts are read after unpacking), not drain-and-launch."""
+    out, err = run("shim_app_packed", [MODULE], shim_env(2))
+    assert out == plain_output
+    s = stats_of(err)
+    assert s["kernel_cmds"] == 1117 and s["kernel_drained"] == 0
+
+
 def test_without_auto_xqueue_everything_passes_through(plain_output):
     out, err = run("shim_app", [MODULE], {"XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"})
     assert out == plain_output
@@ -182,3 +191,31 @@ def test_program_that_releases_nothing_exits_cleanly(level):
     out, err = run("shim_app", ["--leak"], shim_env(level))
     assert "leak counter=100" in out
     assert stats_of(err)["kernel_cmds"] == 102
+
+
+def test_pytorch_program_under_the_preloaded_shim():
+    """A PyTorch-ROCm training loop on side streams (tests/shim_torch_workload.py; compressed
+    code objects, rocBLAS kernels launched from loaded modules, the caching allocator's events)
+    prints bit-identical losses and weights with the shim preloaded, and its launches were
+    XQueue commands."""
+    script = os.path.join(ROOT, "tests", "shim_torch_workload.py")
+
+    def torch_run(extra):
+        env = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+        env.update(extra)
+        print(f"running {script} with {extra}", flush=True)
+        proc = subprocess.run([sys.executable, script], env=env, capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, (proc.stdout[-2000:], proc.stderr[-3000:])
+        return proc.stdout, proc.stderr
+
+    plain, _ = torch_run({})
+    assert plain.strip().endswith("done")
+    shim = os.path.join(LIB, "libshimhip.so")
+    preload = " ".join(x for x in (os.environ.get("LD_PRELOAD", ""), shim) if x)
+    for level in (1, 2):
+        out, err = torch_run(shim_env(level, LD_PRELOAD=preload))
+        assert out == plain
+        s = stats_of(err)
+        print(f"level {level}: {s}", file=sys.stderr, flush=True)
+        assert s["kernel_cmds"] > 500 and s["kernel_drained"] == 0
+        assert s["event_waits"] >= 1 and s["mem_cmds"] > 0

@@ -140,6 +140,61 @@ def test_module_code_object():
         assert _layout(image, kernel)[:2] == (xs.kXSchedSuccess, args)
 
 
+def _packed_bundle(path):
+    """(compressed image as it sits in the file, the bundle it unpacks to) - unpacked here with
+    pyarrow's zstd codec, the library under test uses the system's libzstd."""
+    import pyarrow as pa
+    data = open(path, "rb").read()
+    at = data.find(b"CCOB")
+    assert at >= 0
+    version, method = struct.unpack_from("<HH", data, at + 4)
+    assert (version, method) == (3, 1), "hipcc of this image writes version 3 headers with zstd"
+    file_size, raw_size = struct.unpack_from("<QQ", data, at + 8)
+    packed = data[at:at + file_size]
+    raw = pa.Codec("zstd").decompress(packed[32:], decompressed_size=raw_size).to_pybytes()
+    assert raw.startswith(BUNDLE_MAGIC)
+    return packed, raw
+
+
+def test_compressed_bundles(app_bundle):
+    packed, raw = _packed_bundle(os.path.join(LIB, "shim_app_packed"))
+    end, device = 0, None
+    n = struct.unpack_from("<Q", raw, 24)[0]
+    p = 32
+    for _ in range(n):
+        off, size, tl = struct.unpack_from("<QQQ", raw, p)
+        if b"amdgcn" in raw[p + 24:p + 24 + tl] and size:
+            device = raw[off:off + size]
+        p += 24 + tl
+    want = _elf_metadata(device)
+    assert want == _elf_metadata(app_bundle[1])     # same program, same layouts
+    for kernel, args in want.items():
+        assert _layout(packed, kernel)[:2] == (xs.kXSchedSuccess, args)
+        assert _layout(packed, kernel, size=0)[:2] == (xs.kXSchedSuccess, args)   # size from the header
+    # the earlier header forms, built here around the same compressed bytes
+    body, raw_size = packed[32:], len(raw)
+    v2 = b"CCOB" + struct.pack("<HHII", 2, 1, 24 + len(body), raw_size) + packed[24:32] + body
+    v1 = b"CCOB" + struct.pack("<HHI", 1, 1, raw_size) + packed[24:32] + body
+    assert _layout(v2, "_Z5SaxpyfPKfPfm")[:2] == (xs.kXSchedSuccess, want["_Z5SaxpyfPKfPfm"])
+    assert _layout(v1, "_Z5SaxpyfPKfPfm")[:2] == (xs.kXSchedSuccess, want["_Z5SaxpyfPKfPfm"])
+    assert _layout(v1, "_Z5SaxpyfPKfPfm", size=0)[0] == xs.kXSchedErrorNotSupported   # version 1 has no length
+    # zlib (method 0)
+    import zlib
+    z = zlib.compress(raw)
+    v3z = b"CCOB" + struct.pack("<HHQQ", 3, 0, 32 + len(z), raw_size) + packed[24:32] + z
+    assert _layout(v3z, "_Z5SaxpyfPKfPfm")[:2] == (xs.kXSchedSuccess, want["_Z5SaxpyfPKfPfm"])
+    # damage: wrong sizes, cut data, unknown method or version
+    bad_raw = bytearray(packed); struct.pack_into("<Q", bad_raw, 16, raw_size + 1)
+    assert _layout(bytes(bad_raw), "_Z5SaxpyfPKfPfm")[0] == xs.kXSchedErrorNotSupported
+    assert _layout(packed[:len(packed) // 2], "_Z5SaxpyfPKfPfm")[0] == xs.kXSchedErrorInvalidValue
+    cut = bytearray(packed[:len(packed) - 40]); struct.pack_into("<Q", cut, 8, len(cut))
+    assert _layout(bytes(cut), "_Z5SaxpyfPKfPfm")[0] == xs.kXSchedErrorNotSupported
+    method9 = bytearray(packed); struct.pack_into("<H", method9, 6, 9)
+    assert _layout(bytes(method9), "_Z5SaxpyfPKfPfm")[0] == xs.kXSchedErrorNotSupported
+    version9 = bytearray(packed); struct.pack_into("<H", version9, 4, 9)
+    assert _layout(bytes(version9), "_Z5SaxpyfPKfPfm")[0] == xs.kXSchedErrorNotSupported
+
+
 def test_more_arguments_than_room(app_bundle):
     bundle, _ = app_bundle
     res, got, n = _layout(bundle, "_Z5Mixed4PairshPdi", cap=2)
@@ -158,7 +213,7 @@ def test_unknown_kernel_and_foreign_bytes(app_bundle):
     bundle, device = app_bundle
     assert _layout(bundle, "NoSuchKernel")[0] == xs.kXSchedErrorNotFound
     assert _layout(b"not a code object at all" * 4, "k")[0] == xs.kXSchedErrorInvalidValue
-    assert _layout(b"CCOB" + b"\0" * 60, "k")[0] == xs.kXSchedErrorNotSupported     # compressed bundle
+    assert _layout(b"CCOB" + b"\0" * 60, "k")[0] == xs.kXSchedErrorNotSupported     # compressed, version 0
     assert _layout(b"\x7fELF" + b"\x01\x01" + b"\0" * 58, "k")[0] == xs.kXSchedErrorInvalidValue  # 32-bit ELF
     host_only = BUNDLE_MAGIC + struct.pack("<QQQQ", 1, 64, 0, 4) + b"host"
     assert _layout(host_only + b"\0" * 32, "k")[0] == xs.kXSchedErrorInvalidValue    # no amdgcn entry

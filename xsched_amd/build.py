@@ -9,8 +9,9 @@ Produces, under xsched_amd/lib/:
                     kernels, benchmark harness                         (hipcc, gfx950)
     libshimhip.so   HIP interception shim: stream work of an unmodified
                     HIP program becomes XQueue commands                (g++)
-    shim_app, shim_app_plain
-                    the shim's test program with and without the shim  (hipcc)
+    shim_app, shim_app_plain, shim_app_packed
+                    the shim's test program with the shim, without it, and
+                    with compressed device code                        (hipcc)
     xserver         scheduler daemon                                   (g++)
     traffic_probe   counter-run driver for the AXPY kernel             (hipcc)
 and, under oracle/, the checker libraries (see oracle/Makefile).
@@ -114,6 +115,9 @@ def build_hip(extra, jobs):
         _run(common + ["-o", os.path.join(LIB, "shim_app_plain")])
         _run(common + ["-o", os.path.join(LIB, "shim_app"), "-L", LIB, "-Wl,-rpath,$ORIGIN",
                        "-Wl,--no-as-needed", "-lshimhip"])
+        # the same program with its device code compressed, as large applications ship it
+        _run(common + ["--offload-compress", "-o", os.path.join(LIB, "shim_app_packed"), "-L", LIB,
+                       "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed", "-lshimhip"])
     mod = os.path.join(ROOT, "tests", "shim_module.hip")
     if os.path.exists(mod):
         _run(["hipcc", "--offload-arch=gfx950", "-O3", "--genco", mod, "-o", os.path.join(LIB, "shim_module.co")])

@@ -3,6 +3,8 @@
 #include <cstring>
 #include <string_view>
 
+#include <dlfcn.h>
+
 namespace xsched::hip::codeobj
 {
 
@@ -279,6 +281,77 @@ ParseStatus ReadBundle(Span image, const char *arch, std::vector<KernelLayout> *
     return ReadElf(chosen, out);
 }
 
+// ---- compressed offload bundle ----------------------------------------------------------------
+
+// Header written by clang's offload bundler in front of the compressed bytes of a whole
+// bundle (clang/lib/Driver/OffloadBundler.cpp, CompressedOffloadBundle):
+//   "CCOB", u16 version, u16 method (0 zlib, 1 zstd), then
+//   version 1:                u32 uncompressed size, u64 hash            (20 bytes)
+//   version 2: u32 file size, u32 uncompressed size, u64 hash            (24 bytes)
+//   version 3: u64 file size, u64 uncompressed size, u64 hash            (32 bytes)
+// The decompressors are taken from the system's libzstd / libz at run time; a machine without
+// them reads such images as "compressed", which callers handle.
+typedef size_t (*ZstdDecompressFn)(void *dst, size_t dst_cap, const void *src, size_t src_size);
+typedef unsigned (*ZstdIsErrorFn)(size_t code);
+typedef int (*ZlibUncompressFn)(unsigned char *dst, unsigned long *dst_len, const unsigned char *src, unsigned long src_len);
+
+bool Decompress(uint16_t method, Span in, std::vector<uint8_t> *out)
+{
+    if (method == 1) {
+        static void *lib = dlopen("libzstd.so.1", RTLD_NOW | RTLD_LOCAL);
+        static auto decompress = lib ? (ZstdDecompressFn)dlsym(lib, "ZSTD_decompress") : nullptr;
+        static auto is_error = lib ? (ZstdIsErrorFn)dlsym(lib, "ZSTD_isError") : nullptr;
+        if (decompress == nullptr || is_error == nullptr) return false;
+        const size_t n = decompress(out->data(), out->size(), in.p, in.n);
+        return !is_error(n) && n == out->size();
+    }
+    if (method == 0) {
+        static void *lib = dlopen("libz.so.1", RTLD_NOW | RTLD_LOCAL);
+        static auto uncompress = lib ? (ZlibUncompressFn)dlsym(lib, "uncompress") : nullptr;
+        if (uncompress == nullptr) return false;
+        unsigned long n = out->size();
+        return uncompress(out->data(), &n, in.p, in.n) == 0 && n == out->size();
+    }
+    return false;
+}
+
+ParseStatus ReadCompressed(Span image, const char *arch, std::vector<KernelLayout> *out)
+{
+    uint16_t version, method;
+    if (!image.Get(4, &version) || !image.Get(6, &method)) return ParseStatus::kMalformed;
+    size_t header, file_size = 0, raw_size;
+    if (version == 1) {
+        uint32_t raw;
+        if (!image.Get(8, &raw)) return ParseStatus::kMalformed;
+        header = 20; raw_size = raw;
+    } else if (version == 2) {
+        uint32_t file, raw;
+        if (!image.Get(8, &file) || !image.Get(12, &raw)) return ParseStatus::kMalformed;
+        header = 24; file_size = file; raw_size = raw;
+    } else if (version == 3) {
+        uint64_t file, raw;
+        if (!image.Get(8, &file) || !image.Get(16, &raw)) return ParseStatus::kMalformed;
+        header = 32; file_size = file; raw_size = raw;
+    } else {
+        return ParseStatus::kCompressed;
+    }
+    if (raw_size == 0 || raw_size > ((size_t)1 << 32)) return ParseStatus::kMalformed;
+    size_t packed;
+    if (file_size != 0) {
+        if (file_size < header || !image.Has(0, file_size)) return ParseStatus::kMalformed;
+        packed = file_size - header;
+    } else {
+        if (image.n == kUnbounded) return ParseStatus::kCompressed; // version 1 does not say where it ends
+        if (image.n < header) return ParseStatus::kMalformed;
+        packed = image.n - header;
+    }
+    std::vector<uint8_t> raw(raw_size);
+    if (!Decompress(method, image.Sub(header, packed), &raw)) return ParseStatus::kCompressed;
+    const Span plain { raw.data(), raw.size() };
+    if (plain.Has(0, 24) && memcmp(plain.p, kBundleMagic, 24) == 0) return ReadBundle(plain, arch, out);
+    return ParseStatus::kNotCodeObject;
+}
+
 } // namespace
 
 const char *ToString(ParseStatus status)
@@ -286,7 +359,7 @@ const char *ToString(ParseStatus status)
     switch (status) {
     case ParseStatus::kOk: return "ok";
     case ParseStatus::kNotCodeObject: return "not a code object";
-    case ParseStatus::kCompressed: return "compressed offload bundle";
+    case ParseStatus::kCompressed: return "compressed offload bundle that could not be unpacked";
     case ParseStatus::kNoDeviceImage: return "bundle without an amdgcn image";
     case ParseStatus::kNoMetadata: return "no AMDGPU metadata note";
     case ParseStatus::kMalformed: return "malformed image";
@@ -300,7 +373,7 @@ ParseStatus ReadKernelLayouts(const void *image, size_t bytes, const char *arch,
     if (image == nullptr || out == nullptr) return ParseStatus::kNotCodeObject;
     const Span all { (const uint8_t *)image, bytes == 0 ? kUnbounded : bytes };
     if (!all.Has(0, 4)) return ParseStatus::kNotCodeObject;
-    if (memcmp(all.p, kCompressedMagic, 4) == 0) return ParseStatus::kCompressed;
+    if (memcmp(all.p, kCompressedMagic, 4) == 0) return ReadCompressed(all, arch, out);
     if (memcmp(all.p, "\177ELF", 4) == 0) return ReadElf(all, out);
     if (all.Has(0, 24) && memcmp(all.p, kBundleMagic, 24) == 0) return ReadBundle(all, arch, out);
     return ParseStatus::kNotCodeObject;

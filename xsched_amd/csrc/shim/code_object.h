@@ -38,7 +38,7 @@ enum class ParseStatus
 {
     kOk = 0,
     kNotCodeObject, // neither an offload bundle nor an ELF file
-    kCompressed,    // a compressed offload bundle ("CCOB"): not read
+    kCompressed,    // a compressed offload bundle ("CCOB") and no way to unpack it here
     kNoDeviceImage, // a bundle without an amdgcn entry
     kNoMetadata,    // ELF without the AMDGPU metadata note
     kMalformed,     // a header or the MessagePack data points outside the image
@@ -46,7 +46,8 @@ enum class ParseStatus
 
 const char *ToString(ParseStatus status);
 
-/// Reads the layouts of all kernels in `image`: a clang offload bundle (what
+/// Reads the layouts of all kernels in `image`: a clang offload bundle, plain or compressed
+/// with zstd / zlib (what
 /// __hipRegisterFatBinary and hipModuleLoadData receive from hipcc-built programs; the
 /// entry whose target names `arch` is taken, else the first amdgcn entry: explicit
 /// arguments are laid out alike for every target) or a bare code object (ELF).

@@ -123,14 +123,32 @@ struct Stats
     std::atomic<uint64_t> queue_launches { 0 }, deactivations { 0 }, reactivations { 0 };
 };
 
+// A registered fat binary is read when the first of its kernels is launched: a large program
+// registers thousands of kernels it never runs, and a compressed image costs its whole
+// decompression.
+struct FatBinary
+{
+    const void *image = nullptr;
+    bool read = false;
+    std::unordered_map<std::string, KernelLayout> kernels;
+};
+
+struct HostFunction
+{
+    std::shared_ptr<FatBinary> binary;
+    std::string device_name;
+    bool resolved = false;
+    std::shared_ptr<const KernelLayout> layout; // nullptr after resolution: unknown
+};
+
 struct State
 {
     Stats stats;
 
     std::shared_mutex code_mtx;
-    // value returned by __hipRegisterFatBinary -> kernels of that binary, by name
-    std::unordered_map<const void *, std::shared_ptr<std::unordered_map<std::string, KernelLayout>>> binaries;
-    std::unordered_map<const void *, std::shared_ptr<const KernelLayout>> host_functions; // kernel stubs
+    // value returned by __hipRegisterFatBinary -> that binary
+    std::unordered_map<const void *, std::shared_ptr<FatBinary>> binaries;
+    std::unordered_map<const void *, HostFunction> host_functions; // kernel stubs
     std::unordered_map<const void *, std::shared_ptr<std::unordered_map<std::string, KernelLayout>>> modules; // hipModule_t
     std::unordered_map<const void *, std::shared_ptr<const KernelLayout>> functions;      // hipFunction_t
 
@@ -220,6 +238,37 @@ std::shared_ptr<const KernelLayout> Lookup(std::unordered_map<Key, std::shared_p
     std::shared_lock<std::shared_mutex> lock(S().code_mtx);
     auto it = map.find(key);
     return it == map.end() ? nullptr : it->second;
+}
+
+/// The layout of a kernel registered through __hipRegisterFunction; reads its binary if
+/// nobody has yet.
+std::shared_ptr<const KernelLayout> LayoutOfHostFunction(const void *host_function)
+{
+    {
+        std::shared_lock<std::shared_mutex> lock(S().code_mtx);
+        auto it = S().host_functions.find(host_function);
+        if (it == S().host_functions.end()) return nullptr;
+        if (it->second.resolved) return it->second.layout;
+    }
+    std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+    auto it = S().host_functions.find(host_function);
+    if (it == S().host_functions.end()) return nullptr;
+    HostFunction &fn = it->second;
+    if (!fn.resolved) {
+        FatBinary &bin = *fn.binary;
+        if (!bin.read) {
+            bin.read = true;
+            auto kernels = ReadImage(bin.image, 0, "fat binary");
+            bin.kernels = std::move(*kernels);
+        }
+        auto k = bin.kernels.find(fn.device_name);
+        if (k != bin.kernels.end()) {
+            fn.layout = std::make_shared<const KernelLayout>(k->second);
+            S().stats.known_kernels++;
+        }
+        fn.resolved = true;
+    }
+    return fn.layout;
 }
 
 // ---- launches -------------------------------------------------------------------------------
@@ -409,11 +458,27 @@ void **__hipRegisterFatBinary(const void *data)
     void **handle = REAL(__hipRegisterFatBinary)(data);
     const auto *wrapper = (const FatBinaryWrapper *)data;
     if (handle != nullptr && wrapper != nullptr && wrapper->magic == kFatBinaryMagic && wrapper->binary != nullptr) {
-        auto kernels = ReadImage(wrapper->binary, 0, "fat binary");
+        auto binary = std::make_shared<FatBinary>();
+        binary->image = wrapper->binary;
         std::unique_lock<std::shared_mutex> lock(S().code_mtx);
-        S().binaries[(const void *)handle] = std::move(kernels);
+        S().binaries[(const void *)handle] = std::move(binary);
     }
     return handle;
+}
+
+// The image may go away with the library that holds it (dlclose): it is not read after this.
+void __hipUnregisterFatBinary(void **modules)
+{
+    {
+        std::unique_lock<std::shared_mutex> lock(S().code_mtx);
+        auto bin = S().binaries.find((const void *)modules);
+        if (bin != S().binaries.end()) {
+            bin->second->read = true;
+            bin->second->image = nullptr;
+            S().binaries.erase(bin);
+        }
+    }
+    REAL(__hipUnregisterFatBinary)(modules);
 }
 
 void __hipRegisterFunction(void **modules, const void *hostFunction, char *deviceFunction,
@@ -424,11 +489,10 @@ void __hipRegisterFunction(void **modules, const void *hostFunction, char *devic
         std::unique_lock<std::shared_mutex> lock(S().code_mtx);
         auto bin = S().binaries.find((const void *)modules);
         if (bin != S().binaries.end()) {
-            auto k = bin->second->find(deviceName);
-            if (k != bin->second->end()) {
-                S().host_functions[hostFunction] = std::make_shared<const KernelLayout>(k->second);
-                S().stats.known_kernels++;
-            }
+            HostFunction &fn = S().host_functions[hostFunction];
+            fn = HostFunction {};
+            fn.binary = bin->second;
+            fn.device_name = deviceName;
         }
     }
     REAL(__hipRegisterFunction)(modules, hostFunction, deviceFunction, deviceName, threadLimit, tid, bid,
@@ -512,7 +576,7 @@ hipError_t hipLaunchKernel(const void *function_address, dim3 numBlocks, dim3 di
         S().stats.kernel_direct++;
         return REAL(hipLaunchKernel)(function_address, numBlocks, dimBlocks, args, sharedMemBytes, stream);
     }
-    auto layout = Lookup(S().host_functions, function_address);
+    auto layout = LayoutOfHostFunction(function_address);
     if (layout != nullptr && (args != nullptr || layout->args.empty())) {
         std::vector<size_t> sizes(layout->args.size());
         for (size_t i = 0; i < sizes.size(); ++i) sizes[i] = layout->args[i].size;
