@@ -3,17 +3,19 @@
 //
 // MFMA-bound: 2*M*N*K flop. One work-group of 512 threads (8 wavefronts) owns one
 // 256x256 tile of C and walks K in steps of 64 through two LDS buffers:
-//   global -> registers (tile t+2 is requested while tile t is computed)
-//   registers -> LDS    A tile as [256 rows][64 k], B tile transposed to [256 cols][64 k],
-//                       both with rows padded to 72 bf16 so that the 128-bit fragment
-//                       reads of 32 consecutive rows fall into distinct banks; written to
-//                       the buffer that is not being read, one barrier per step
+//   global -> registers (tile t+2 is requested while tile t is computed), 128-bit loads for
+//                       both operands
+//   registers -> LDS    A tile as [256 rows][64 k], rows padded to 72 bf16 so that the 128-bit
+//                       fragment reads of 32 consecutive rows fall into distinct banks;
+//                       B tile as it sits in memory, [64 k][256 cols], rows padded to 272 bf16;
+//                       written to the buffer that is not being read, one barrier per step
 //   LDS -> MFMA         v_mfma_f32_32x32x16_bf16; wave (wm, wn) of the 2x4 wave grid
 //                       accumulates a 128x64 sub-tile = 4x2 blocks of 32x32
-// B is read from global memory as 32-bit words (two columns) over eight k rows and
-// transposed in registers with byte permutes, so that LDS holds k-contiguous
-// fragments for both operands. There is no split-K: every element of C is summed by
-// one wave in one fixed order, which makes a replayed tile bit-identical.
+// An MFMA operand wants eight consecutive k per lane. A has them contiguous in memory; for B
+// (k is the strided dimension) the transposing LDS read of gfx950, ds_read_b64_tr_b16, turns
+// four rows of four columns into four k of one column per lane, two of them per fragment.
+// There is no split-K: every element of C is summed by one wave in one fixed order, which
+// makes a replayed tile bit-identical.
 //
 // Guard: the tile is computed in registers and written once at the end, so a
 // work-group may give up at any K step without side effects. The preempt word is
@@ -39,7 +41,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTile = 256;          // tile edge (M and N)
 constexpr int kStepK = 64;          // K per step
-constexpr int kLdsStride = 72;      // bf16 per LDS row (64 + 8 padding)
+constexpr int kLdsStride = 72;      // bf16 per row of the A tile in LDS (64 + 8 padding)
+constexpr int kBStride = 272;       // bf16 per row of the B tile in LDS (256 + 16): four consecutive rows start in four different 32-byte bank groups
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 LdsS16x4;
 constexpr int kThreads = 512;
 constexpr int kPollSteps = 8;       // K steps between two looks at the preempt word
 constexpr int kXcds = 8;
@@ -88,7 +94,7 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
                              uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
 {
     __shared__ __attribute__((aligned(16))) uint16_t As[2][kTile * kLdsStride];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kTile * kLdsStride];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kStepK * kBStride];
     __shared__ uint32_t guard_word;
 
     const uint32_t tid = threadIdx.x;
@@ -102,7 +108,7 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     const size_t m0 = (size_t)tm * kTile, n0 = (size_t)tn * kTile;
 
     u32x4 a_reg[4];
-    uint32_t b_reg[2][8];
+    u32x4 b_vec[4];
 
     auto load_global = [&](int k0) {
 #pragma unroll
@@ -112,12 +118,10 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
             a_reg[i] = *(const u32x4 *)(A + (m0 + row) * (size_t)K + k0 + kc * 8);
         }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const uint32_t c = tid + kThreads * i;
-            const uint32_t npair = c & 127, kg = c >> 7;
-            const uint16_t *src = B + (size_t)(k0 + kg * 8) * N + n0 + npair * 2;
-#pragma unroll
-            for (int r = 0; r < 8; ++r) b_reg[i][r] = *(const uint32_t *)(src + (size_t)r * N);
+            const uint32_t krow = c >> 5, chunk = c & 31;
+            b_vec[i] = *(const u32x4 *)(B + (size_t)(k0 + krow) * N + n0 + chunk * 8);
         }
     };
 
@@ -129,33 +133,35 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
             *(u32x4 *)(As[buf] + row * kLdsStride + kc * 8) = a_reg[i];
         }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const uint32_t c = tid + kThreads * i;
-            const uint32_t npair = c & 127, kg = c >> 7;
-            u32x4 col0, col1;
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const uint32_t lo = b_reg[i][2 * p], hi = b_reg[i][2 * p + 1];
-                col0[p] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                col1[p] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
-            }
-            *(u32x4 *)(Bs[buf] + (npair * 2 + 0) * kLdsStride + kg * 8) = col0;
-            *(u32x4 *)(Bs[buf] + (npair * 2 + 1) * kLdsStride + kg * 8) = col1;
+            const uint32_t krow = c >> 5, chunk = c & 31;
+            *(u32x4 *)(Bs[buf] + krow * kBStride + chunk * 8) = b_vec[i];
         }
     };
 
     const uint32_t a_row0 = 128 * wm + (lane & 31);
-    const uint32_t b_col0 = 64 * wn + (lane & 31);
     const uint32_t khalf = 8 * (lane >> 5);
     auto load_a_frags = [&](int buf, int ks, bf16x8 *fa) {
         const uint32_t koff = ks * 16 + khalf;
 #pragma unroll
         for (int i = 0; i < 4; ++i) fa[i] = *(const bf16x8 *)(As[buf] + (a_row0 + 32 * i) * kLdsStride + koff);
     };
+    // B sits in LDS as it sits in memory, [k][n]. The transposing read hands lane l of every 16
+    // lanes the element (l & 3) of what lanes 4 * j + (l >> 2), j = 0..3, of the same 16 point
+    // at: with lane r pointing at row (r >> 2), columns 4 * (r & 3) .. + 3, lane l receives
+    // column l of rows 0..3. Two reads give the eight consecutive k of one fragment.
+    const uint32_t b_tr_row = 8 * (lane >> 5) + ((lane & 15) >> 2);
+    const uint32_t b_tr_col = 64 * wn + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     auto load_b_frags = [&](int buf, int ks, bf16x8 *fb) {
-        const uint32_t koff = ks * 16 + khalf;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) fb[j] = *(const bf16x8 *)(Bs[buf] + (b_col0 + 32 * j) * kLdsStride + koff);
+        for (int j = 0; j < 2; ++j) {
+            const uint16_t *p = Bs[buf] + (ks * 16 + b_tr_row) * kBStride + b_tr_col + 32 * j;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)p);
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)(p + 4 * kBStride));
+            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            fb[j] = __builtin_bit_cast(bf16x8, both);
+        }
     };
     auto load_frags = [&](int buf, int ks, bf16x8 *fa, bf16x8 *fb) {
         load_a_frags(buf, ks, fa);
@@ -249,6 +255,7 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         guard.Commit();
     }
 }
+
 
 class HipGemmCommand final : public HipGuardedCommand
 {
