@@ -18,13 +18,16 @@
  *             hipModuleGetFunction, hipModuleUnload                       (shim.cpp:100-111)
  *   memory    hipMemcpyAsync, hipMemcpyWithStream, hipMemcpyHtoDAsync, hipMemcpyDtoHAsync,
  *             hipMemcpyDtoDAsync, hipMemcpy2DAsync, hipMemcpyPeerAsync, hipMemsetAsync,
- *             hipMemsetD8Async, hipMemsetD16Async, hipMemsetD32Async, hipMemcpy, hipMemset,
- *             hipFree, hipFreeAsync, hipMallocAsync                       (shim.cpp:113-150, shim.h:37-50)
+ *             hipMemsetD8Async, hipMemsetD16Async, hipMemsetD32Async, hipMemcpy, hipMemcpyHtoD,
+ *             hipMemcpyDtoH, hipMemcpyDtoD, hipMemset, hipFree, hipFreeAsync,
+ *             hipMallocAsync                                              (shim.cpp:113-150, shim.h:37-50)
  *   events    hipEventRecord, hipEventRecordWithFlags, hipEventQuery, hipEventSynchronize,
  *             hipEventElapsedTime, hipEventDestroy, hipStreamWaitEvent    (shim.cpp:152-257)
  *   streams   hipStreamCreate, hipStreamCreateWithFlags, hipStreamCreateWithPriority,
  *             hipStreamDestroy, hipStreamSynchronize, hipStreamQuery, hipStreamAddCallback,
  *             hipLaunchHostFunc, hipDeviceSynchronize, hipCtxSynchronize  (shim.cpp:259-320)
+ *   graphs    hipStreamBeginCapture, hipStreamEndCapture (a capturing stream is left to the
+ *             runtime), hipGraphLaunch (ordered behind the stream's XQueue)
  *
  * The two functions below are for tests and tools; a program under the shim needs neither.
  */

@@ -342,6 +342,32 @@ int main(int argc, char **argv)
         CHECK(hipFree(acc[0])); CHECK(hipFree(acc[1])); CHECK(hipFree(ones));
     }
 
+    // ---- 7b. a graph captured from a stream and launched between ordinary launches --------------
+    {
+        uint32_t *gbuf, *gone;
+        CHECK(hipMalloc(&gbuf, 1024 * 4)); CHECK(hipMalloc(&gone, 1024 * 4));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)gbuf, 0, 1024, s1));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)gone, 1, 1024, s1));
+        AddInto<<<4, 256, 0, s1>>>(gbuf, gone, 1, 1024);                  // 2, still queued when the capture begins
+        hipGraph_t graph;
+        hipGraphExec_t exec;
+        CHECK(hipStreamBeginCapture(s1, hipStreamCaptureModeGlobal));
+        for (int i = 0; i < 3; ++i) AddInto<<<4, 256, 0, s1>>>(gbuf, gone, 9, 1024);   // + 30 per launch of the graph
+        CHECK(hipStreamEndCapture(s1, &graph));
+        CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        CHECK(hipGraphLaunch(exec, s1));                                  // 32
+        AddInto<<<4, 256, 0, s1>>>(gbuf, gbuf, 0, 1024);                  // 64, must follow the graph
+        CHECK(hipGraphLaunch(exec, s1));                                  // 94, must follow the kernel
+        std::vector<uint32_t> g_host(1024);
+        CHECK(hipMemcpyAsync(g_host.data(), gbuf, 1024 * 4, hipMemcpyDeviceToHost, s1));
+        CHECK(hipStreamSynchronize(s1));
+        bad = 0;
+        for (int i = 0; i < 1024; ++i) bad += g_host[i] != 94;
+        Report("captured graph in order", bad, 0);
+        CHECK(hipGraphExecDestroy(exec)); CHECK(hipGraphDestroy(graph));
+        CHECK(hipFree(gbuf)); CHECK(hipFree(gone));
+    }
+
     // ---- 8. kernels of a loaded module ------------------------------------------------------------
     if (module_path != nullptr) {
         hipModule_t mod;

@@ -184,9 +184,18 @@ void PrintStats()
             (unsigned long)t.deactivations, (unsigned long)t.reactivations);
 }
 
+constexpr unsigned kStreamCapturing = 1u << 31; // kept next to the stream's creation flags
+
 std::shared_ptr<XQueue> QueueOf(hipStream_t stream)
 {
     if (stream == nullptr) return nullptr;
+    {
+        // While a stream captures a graph its work is recorded, not run: the runtime has to see
+        // every call on the capturing thread, so the stream counts as one without an XQueue.
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        auto it = S().stream_flags.find(stream);
+        if (it != S().stream_flags.end() && (it->second & kStreamCapturing)) return nullptr;
+    }
     return HwQueueManager::GetXQueue((HwQueueHandle)(uintptr_t)stream); // reference handle.h:9-12
 }
 
@@ -199,13 +208,16 @@ void SubmitHandle(const std::shared_ptr<XQueue> &xq, HwCommandHandle handle)
 /// Before work on the null stream: everything queued on blocking streams comes first.
 void WaitBlockingQueues()
 {
-    std::vector<std::shared_ptr<XQueue>> queues;
+    std::vector<hipStream_t> blocking;
     {
         std::lock_guard<std::mutex> lock(S().stream_mtx);
         for (const auto &entry : S().stream_flags) {
-            if (entry.second & hipStreamNonBlocking) continue;
-            if (auto xq = QueueOf(entry.first)) queues.push_back(std::move(xq));
+            if ((entry.second & (hipStreamNonBlocking | kStreamCapturing)) == 0) blocking.push_back(entry.first);
         }
+    }
+    std::vector<std::shared_ptr<XQueue>> queues;
+    for (hipStream_t stream : blocking) {
+        if (auto xq = QueueOf(stream)) queues.push_back(std::move(xq));
     }
     std::vector<std::shared_ptr<XQueueWaitAllCommand>> waits;
     for (auto &xq : queues) waits.push_back(xq->SubmitWaitAll());
@@ -725,6 +737,24 @@ hipError_t hipMemcpy(void *dst, const void *src, size_t sizeBytes, hipMemcpyKind
     return REAL(hipMemcpy)(dst, src, sizeBytes, kind);
 }
 
+hipError_t hipMemcpyHtoD(hipDeviceptr_t dst, const void *src, size_t sizeBytes)
+{
+    if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
+    return REAL(hipMemcpyHtoD)(dst, src, sizeBytes);
+}
+
+hipError_t hipMemcpyDtoH(void *dst, hipDeviceptr_t src, size_t sizeBytes)
+{
+    if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
+    return REAL(hipMemcpyDtoH)(dst, src, sizeBytes);
+}
+
+hipError_t hipMemcpyDtoD(hipDeviceptr_t dst, hipDeviceptr_t src, size_t sizeBytes)
+{
+    if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
+    return REAL(hipMemcpyDtoD)(dst, src, sizeBytes);
+}
+
 hipError_t hipMemset(void *dst, int value, size_t sizeBytes)
 {
     if (!CALLER_IS_INSIDE()) WaitBlockingQueues();
@@ -933,6 +963,42 @@ hipError_t hipStreamQuery(hipStream_t stream)
         }
     }
     return REAL(hipStreamQuery)(stream);
+}
+
+// Stream capture: what is queued goes first, then the stream is the runtime's alone until the
+// capture ends. A graph launch is one stream-ordered operation: ordered by draining.
+hipError_t hipStreamBeginCapture(hipStream_t stream, hipStreamCaptureMode mode)
+{
+    if (!CALLER_IS_INSIDE() && stream != nullptr) {
+        if (auto xq = QueueOf(stream)) xq->WaitAll();
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        auto it = S().stream_flags.find(stream);
+        if (it != S().stream_flags.end()) it->second |= kStreamCapturing;
+    }
+    const hipError_t res = REAL(hipStreamBeginCapture)(stream, mode);
+    if (res != hipSuccess && stream != nullptr) {
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        auto it = S().stream_flags.find(stream);
+        if (it != S().stream_flags.end()) it->second &= ~kStreamCapturing;
+    }
+    return res;
+}
+
+hipError_t hipStreamEndCapture(hipStream_t stream, hipGraph_t *pGraph)
+{
+    const hipError_t res = REAL(hipStreamEndCapture)(stream, pGraph);
+    if (stream != nullptr) {
+        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        auto it = S().stream_flags.find(stream);
+        if (it != S().stream_flags.end()) it->second &= ~kStreamCapturing;
+    }
+    return res;
+}
+
+hipError_t hipGraphLaunch(hipGraphExec_t graphExec, hipStream_t stream)
+{
+    if (!CALLER_IS_INSIDE()) DrainFor(stream);
+    return REAL(hipGraphLaunch)(graphExec, stream);
 }
 
 hipError_t hipStreamAddCallback(hipStream_t stream, hipStreamCallback_t callback, void *userData, unsigned int flags)
