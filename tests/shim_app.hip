@@ -351,8 +351,12 @@ int main(int argc, char **argv)
         AddInto<<<4, 256, 0, s1>>>(gbuf, gone, 1, 1024);                  // 2, still queued when the capture begins
         hipGraph_t graph;
         hipGraphExec_t exec;
+        // Another stream is busy during the capture: whoever waits for its work on the program's
+        // behalf must not disturb a capture in the default (global) mode.
+        for (int i = 0; i < 40; ++i) Spin<<<1, 256, 0, s3>>>(spin, 20000);
         CHECK(hipStreamBeginCapture(s1, hipStreamCaptureModeGlobal));
         for (int i = 0; i < 3; ++i) AddInto<<<4, 256, 0, s1>>>(gbuf, gone, 9, 1024);   // + 30 per launch of the graph
+        std::this_thread::sleep_for(std::chrono::milliseconds(2));
         CHECK(hipStreamEndCapture(s1, &graph));
         CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
         CHECK(hipGraphLaunch(exec, s1));                                  // 32

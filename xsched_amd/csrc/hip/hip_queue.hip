@@ -17,6 +17,27 @@ using namespace xsched::protocol;
 namespace xsched::hip
 {
 
+namespace
+{
+
+/// While a stream of the process captures a graph in the default (global) mode, the runtime
+/// refuses waits, queries and allocations from every thread that has not declared itself
+/// relaxed, and invalidates the capture on top. The adapter's own waits and allocations
+/// concern its own streams and markers, never a capturing one (the shim leaves a capturing
+/// stream to the runtime), so they run relaxed; the thread's mode is put back afterwards
+/// because the thread may be the application's.
+class RelaxedCaptureScope
+{
+public:
+    RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
+    ~RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
+private:
+    hipStreamCaptureMode mode_ = hipStreamCaptureModeRelaxed;
+};
+
+} // namespace
+
+
 int64_t SyncSpinMicros()
 {
     static const int64_t us = []() {
@@ -155,6 +176,7 @@ void GuardState::Deactivate(hipStream_t op_stream)
 
 void GuardState::WaitFlagWritten(hipStream_t op_stream)
 {
+    RelaxedCaptureScope relaxed;
     if (!flag_on_host_ && !write_through_bar_) HIP_ASSERT(hipStreamSynchronize(op_stream));
 }
 
@@ -162,6 +184,7 @@ GuardState::Slot GuardState::AcquireSlot()
 {
     std::lock_guard<std::mutex> lock(mtx_);
     if (free_slots_.empty()) {
+        RelaxedCaptureScope relaxed;
         uint8_t *arena = nullptr;
         const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
         HIP_ASSERT(hipMalloc((void **)&arena, bytes));
@@ -228,6 +251,7 @@ hipError_t HipCommand::LaunchWrapper(HipQueue &q, bool replay)
 void HipCommand::Synchronize()
 {
     XASSERT(marker_ != nullptr, "Synchronize() needs EnableSynchronization() before launch");
+    RelaxedCaptureScope relaxed;
     const int64_t spin_us = SyncSpinMicros();
     if (spin_us > 0) {
         const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_us);
@@ -359,6 +383,7 @@ void *ScratchPool::Acquire(size_t bytes)
     // be in flight with it, so that a queue in steady state allocates nothing while its
     // kernels run.
     DeviceScope scope(device_);
+    RelaxedCaptureScope relaxed;
     void *first = nullptr;
     const int count = buffers_.empty() ? kInitialBuffers : 1;
     for (int i = 0; i < count; ++i) {
@@ -399,6 +424,7 @@ void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
 void HipQueue::Synchronize()
 {
     DeviceScope scope(device_);
+    RelaxedCaptureScope relaxed;
     const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(SyncSpinMicros());
     while (true) {
         const hipError_t err = hipStreamQuery(stream_);

@@ -20,6 +20,7 @@
 //     blocking streams first (the reference keeps a map for this that is never filled:
 //     shim.cpp:21-32).
 #include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -28,6 +29,7 @@
 #include <mutex>
 #include <shared_mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -970,7 +972,14 @@ hipError_t hipStreamQuery(hipStream_t stream)
 hipError_t hipStreamBeginCapture(hipStream_t stream, hipStreamCaptureMode mode)
 {
     if (!CALLER_IS_INSIDE() && stream != nullptr) {
-        if (auto xq = QueueOf(stream)) xq->WaitAll();
+        if (auto xq = QueueOf(stream)) {
+            // Not only everything queued: the launch thread may still be in the drain sequence
+            // it runs on its own after commands were launched from this thread, and that ends
+            // with a query of the stream. An idle XQueue means the thread sleeps.
+            xq->WaitAll();
+            const auto give_up = std::chrono::steady_clock::now() + std::chrono::seconds(2);
+            while (xq->Query() != kQueueStateIdle && std::chrono::steady_clock::now() < give_up) std::this_thread::yield();
+        }
         std::lock_guard<std::mutex> lock(S().stream_mtx);
         auto it = S().stream_flags.find(stream);
         if (it != S().stream_flags.end()) it->second |= kStreamCapturing;
