@@ -312,6 +312,34 @@ def config5(H, a):
     return line
 
 
+def shim_launch_cost():
+    """us per launch of a tiny kernel by an unmodified HIP program (tests/shim_app.hip, built into
+    xsched_amd/lib), natively and with the interception shim in front of the runtime (every
+    launch an XQueue command). Informational; None when the programs have not been built."""
+    import re
+    import subprocess
+    lib = os.path.join(os.path.dirname(os.path.abspath(__file__)), "xsched_amd", "lib")
+    out = {}
+    for key, binary, extra in (("native", "shim_app_plain", {}),
+                               ("through_shim", "shim_app", {"XSCHED_AUTO_XQUEUE": "ON", "XSCHED_SCHEDULER": "LCL",
+                                                             "XSCHED_POLICY": "HPF", "XLOG_LEVEL": "WARN"})):
+        path = os.path.join(lib, binary)
+        if not os.path.exists(path):
+            return None
+        env = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+        env.update(extra)
+        try:
+            proc = subprocess.run([path, "--bench", "20000"], env=env, capture_output=True, text=True, timeout=60)
+        except subprocess.TimeoutExpired:
+            return None
+        m = re.search(r"submit_us_per_launch=([\d.]+) total_us_per_launch=([\d.]+)", proc.stdout)
+        if proc.returncode != 0 or not m:
+            return None
+        out[key] = {"submit_us_per_launch": float(m.group(1)), "total_us_per_launch": float(m.group(2))}
+    out["launches"] = 20000
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -335,6 +363,8 @@ def main():
     from xsched_amd import harness as H
 
     line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
+    if a.config == 2 and not a.quick:
+        line["shim_launch_cost"] = shim_launch_cost()
     if a.config == 2 and not a.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
     else:
