@@ -157,7 +157,7 @@ struct State
     std::mutex event_mtx;
     std::unordered_map<hipEvent_t, std::shared_ptr<HwCommand>> events; // last record command per event
 
-    std::mutex stream_mtx;
+    std::shared_mutex stream_mtx; // read on every call that names a stream
     std::unordered_map<hipStream_t, unsigned> stream_flags; // streams this library has seen created
 };
 
@@ -194,7 +194,7 @@ std::shared_ptr<XQueue> QueueOf(hipStream_t stream)
     {
         // While a stream captures a graph its work is recorded, not run: the runtime has to see
         // every call on the capturing thread, so the stream counts as one without an XQueue.
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::shared_lock<std::shared_mutex> lock(S().stream_mtx);
         auto it = S().stream_flags.find(stream);
         if (it != S().stream_flags.end() && (it->second & kStreamCapturing)) return nullptr;
     }
@@ -212,7 +212,7 @@ void WaitBlockingQueues()
 {
     std::vector<hipStream_t> blocking;
     {
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::shared_lock<std::shared_mutex> lock(S().stream_mtx);
         for (const auto &entry : S().stream_flags) {
             if ((entry.second & (hipStreamNonBlocking | kStreamCapturing)) == 0) blocking.push_back(entry.first);
         }
@@ -414,7 +414,7 @@ hipError_t FillAsync(void *dst, uint32_t value, size_t count, uint32_t width, hi
 void OnStreamCreated(hipStream_t stream, unsigned flags)
 {
     {
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
         S().stream_flags[stream] = flags;
     }
     (void)XQueueManager::AutoCreate([&](HwQueueHandle *hwq) { return HipQueueCreate(hwq, stream); });
@@ -926,7 +926,7 @@ hipError_t hipStreamDestroy(hipStream_t stream)
     if (!CALLER_IS_INSIDE()) {
         bool known;
         {
-            std::lock_guard<std::mutex> lock(S().stream_mtx);
+            std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
             known = S().stream_flags.erase(stream) != 0;
         }
         if (known && QueueOf(stream) != nullptr) {
@@ -980,13 +980,13 @@ hipError_t hipStreamBeginCapture(hipStream_t stream, hipStreamCaptureMode mode)
             const auto give_up = std::chrono::steady_clock::now() + std::chrono::seconds(2);
             while (xq->Query() != kQueueStateIdle && std::chrono::steady_clock::now() < give_up) std::this_thread::yield();
         }
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
         auto it = S().stream_flags.find(stream);
         if (it != S().stream_flags.end()) it->second |= kStreamCapturing;
     }
     const hipError_t res = REAL(hipStreamBeginCapture)(stream, mode);
     if (res != hipSuccess && stream != nullptr) {
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
         auto it = S().stream_flags.find(stream);
         if (it != S().stream_flags.end()) it->second &= ~kStreamCapturing;
     }
@@ -997,7 +997,7 @@ hipError_t hipStreamEndCapture(hipStream_t stream, hipGraph_t *pGraph)
 {
     const hipError_t res = REAL(hipStreamEndCapture)(stream, pGraph);
     if (stream != nullptr) {
-        std::lock_guard<std::mutex> lock(S().stream_mtx);
+        std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
         auto it = S().stream_flags.find(stream);
         if (it != S().stream_flags.end()) it->second &= ~kStreamCapturing;
     }
