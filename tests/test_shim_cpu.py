@@ -250,3 +250,22 @@ def test_corrupted_metadata_never_crashes(app_bundle):
         if res == xs.kXSchedSuccess and image == bytearray(device):
             assert got == want["_Z5SaxpyfPKfPfm"]
     assert outcomes <= {xs.kXSchedSuccess, xs.kXSchedErrorInvalidValue, xs.kXSchedErrorNotFound}
+
+
+def test_reader_under_address_and_ub_sanitizers(tmp_path):
+    """The reader takes bytes it has not produced: built with -fsanitize=address,undefined it
+    reads thousands of damaged and truncated copies of the three real images from heap blocks
+    of exactly the stated size (tests/code_object_fuzz.cpp), and nothing must be flagged."""
+    exe = str(tmp_path / "co_fuzz")
+    shim = os.path.join(ROOT, "xsched_amd", "csrc", "shim")
+    # the sanitizer runtimes are linked statically: they then do not mind other preloaded libraries
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                    "-static-libasan", "-static-libubsan",
+                    "-I", shim, os.path.join(shim, "code_object.cpp"), os.path.join(ROOT, "tests", "code_object_fuzz.cpp"),
+                    "-o", exe, "-ldl"], check=True, capture_output=True)
+    images = [os.path.join(LIB, n) for n in ("shim_app_plain", "shim_app_packed", "shim_module.co")]
+    proc = subprocess.run([exe, "1500"] + images, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-4000:]
+    lines = proc.stdout.strip().splitlines()
+    assert len(lines) == 3 and all("refused" in line for line in lines), proc.stdout
+    assert lines[0].split(":")[1].strip().startswith("8 kernels") and lines[2].split(":")[1].strip().startswith("2 kernels")

@@ -335,7 +335,6 @@ ParseStatus ReadCompressed(Span image, const char *arch, std::vector<KernelLayou
     } else {
         return ParseStatus::kCompressed;
     }
-    if (raw_size == 0 || raw_size > ((size_t)1 << 32)) return ParseStatus::kMalformed;
     size_t packed;
     if (file_size != 0) {
         if (file_size < header || !image.Has(0, file_size)) return ParseStatus::kMalformed;
@@ -345,6 +344,9 @@ ParseStatus ReadCompressed(Span image, const char *arch, std::vector<KernelLayou
         if (image.n < header) return ParseStatus::kMalformed;
         packed = image.n - header;
     }
+    // A damaged header must not make this allocate gigabytes: a bundle unpacks to at most a few
+    // hundred MB, and the formats at hand do not pack better than 256 : 1.
+    if (raw_size == 0 || raw_size > ((size_t)1 << 30) || raw_size / 256 > packed) return ParseStatus::kMalformed;
     std::vector<uint8_t> raw(raw_size);
     if (!Decompress(method, image.Sub(header, packed), &raw)) return ParseStatus::kCompressed;
     const Span plain { raw.data(), raw.size() };
