@@ -342,6 +342,18 @@ int main(int argc, char **argv)
         CHECK(hipFree(acc[0])); CHECK(hipFree(acc[1])); CHECK(hipFree(ones));
     }
 
+    // ---- 7a. a launch the runtime refuses is refused the same way ------------------------------
+    {
+        void *args[] = { &spin, &zero };
+        const hipError_t too_wide = hipLaunchKernel((const void *)Spin, dim3(1), dim3(2048), args, 0, s1);
+        (void)hipGetLastError();
+        const hipError_t no_grid = hipLaunchKernel((const void *)Spin, dim3(0), dim3(64), args, 0, s1);
+        (void)hipGetLastError();
+        CHECK(hipStreamSynchronize(s1));
+        Report("refused launches", (uint64_t)too_wide * 1000 + (uint64_t)no_grid, (uint64_t)too_wide * 1000 + (uint64_t)no_grid);
+        printf("    error codes %d %d\n", (int)too_wide, (int)no_grid);
+    }
+
     // ---- 7b. a graph captured from a stream and launched between ordinary launches --------------
     {
         uint32_t *gbuf, *gone;

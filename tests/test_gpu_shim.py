@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "xsched_amd", "lib")
 MODULE = os.path.join(LIB, "shim_module.co")
-CHECKS = 15  # lines the program prints, "done" included
+CHECKS = 17  # lines the program prints, "done" and the error codes included
 
 
 def run(binary, args, env_extra, timeout=120):
@@ -53,7 +53,9 @@ def plain_output():
     lines = out.strip().splitlines()
     assert len(lines) == CHECKS and lines[-1] == "done", out
     for line in lines[:-1]:
-        assert line.endswith(" ok"), line
+        assert line.endswith(" ok") or line.startswith("    error codes"), line
+    codes = [line for line in lines if line.startswith("    error codes")][0].split()[2:]
+    assert all(int(c) != 0 for c in codes), "the runtime accepted an invalid launch"
     return out
 
 
@@ -67,7 +69,7 @@ def test_same_results_through_xqueues(plain_output, level, threshold, batch):
     # + 2 * 400 from the threads + 3 module launches; the one null-stream launch goes straight through
     # + 2 around the captured graph (the three captured launches are recorded by the runtime)
     assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3
-    assert s["kernel_drained"] == 0 and s["kernel_direct"] == 1 + 3
+    assert s["kernel_drained"] == 2 and s["kernel_direct"] == 1 + 3   # the two refused launches go to the runtime
     assert s["known_kernels"] >= 7 + 2
     assert s["event_cmds"] == 3 and s["event_waits"] == 1
     # pinned and device-to-device copies and every fill are commands; pageable copies drain
@@ -80,7 +82,7 @@ def test_program_with_compressed_device_code(plain_output):
     out, err = run("shim_app_packed", [MODULE], shim_env(2))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] == 1159 and s["kernel_drained"] == 0
+    assert s["kernel_cmds"] == 1159 and s["kernel_drained"] == 2
 
 
 def test_without_auto_xqueue_everything_passes_through(plain_output):
@@ -112,7 +114,7 @@ def test_unmodified_binary_under_ld_preload(plain_output):
     out, err = run("shim_app_plain", [MODULE], shim_env(1, LD_PRELOAD=preload))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 0
+    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 2
 
 
 def _percentiles(out):
