@@ -71,6 +71,22 @@ XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void
 XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t n, void *bins,
                                   uint32_t n_bins, int guard);
 
+/* A kernel of the caller's own that has the guard of xsched/hip/guard.h compiled in (see the
+ * head of that file for the three lines). The kernel's LAST parameter must be an XGuardArgs:
+ * `args` / `arg_sizes` describe the parameters in front of it (copied at creation), the guard
+ * arguments are supplied at every launch. The grid is one-dimensional, `n_workgroups`
+ * work-groups (at most 2^18); the kernel identifies its work-group to the guard by
+ * blockIdx.x. Property Deactivatable: at level 2 a launch can be flushed and is replayed by
+ * the reactivation, every work-group taking effect exactly once; at level 1 the guard lets
+ * every work-group through. Takes the place of the instrumentation the reference applies to
+ * CUDA kernels (platforms/cuda/hal/src/level2/instrument.cpp:224-231,
+ * platforms/cuda/hal/inject/inject.cu:43-83). */
+XResult HipGuardedKernelCommandCreate(HwCommandHandle *cmd, const void *host_func,
+                                      uint32_t n_workgroups,
+                                      uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                                      void **args, const size_t *arg_sizes, size_t n_args,
+                                      uint32_t shared_mem_bytes);
+
 /* ---- generic commands (level 1 semantics; they are drain points at level 2) -- */
 
 /* hipMemcpyAsync; `kind` is a hipMemcpyKind value. reference hip_command.h:188 */

@@ -304,3 +304,63 @@ def test_launches_of_a_flushed_epoch_do_not_run(xs, gpu, kind):
     q.close()
     assert np.array_equal(untouched, before), "a launch of a flushed epoch wrote something"
     assert np.array_equal(ran, after), "a launch of the next epoch did not run exactly once"
+
+
+def test_user_written_guarded_kernel_is_flushed_and_replayed_exactly_once(xs, gpu):
+    """A kernel outside the library (tests/user_guarded_kernel.hip: in place, not idempotent)
+    with the guard compiled in, submitted through HipGuardedKernelCommandCreate: suspended and
+    resumed at random while 120 launches go through a level-2 queue, every work-group of every
+    launch must have taken effect exactly once; the same commands at level 1 give the same bits."""
+    import ctypes
+    import os
+    torch = gpu
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(xs.__file__), "lib", "libuserguarded.so"))
+    lib.UserAffineKernel.restype = ctypes.c_void_p
+    func, chunk = lib.UserAffineKernel(), lib.UserAffineChunk()
+    n, times = (1 << 24) + 1234, 120
+    n_wg = (n + chunk - 1) // chunk
+    print(f"case user-guarded n={n} times={times} work-groups={n_wg}", flush=True)
+    y_h = oracle.fill_uniform(21, 2, 0, n)
+
+    def command(y, b):
+        y_ptr, b_val, n_val = ctypes.c_void_p(y.data_ptr()), ctypes.c_float(b), ctypes.c_size_t(n)
+        args = (ctypes.c_void_p * 3)(ctypes.addressof(y_ptr), ctypes.addressof(b_val), ctypes.addressof(n_val))
+        sizes = (ctypes.c_size_t * 3)(8, 4, 8)
+        cmd = c_uint64()
+        xs.check(xs.halhip().HipGuardedKernelCommandCreate(byref(cmd), func, n_wg, 256, 1, 1, args, sizes, 3, 0))
+        return cmd.value
+
+    def run(level, with_churn):
+        y = torch.from_numpy(y_h.copy()).cuda()
+        q = Queue(xs, torch, level=level, threshold=4, batch=2)
+        stop, result = threading.Event(), {}
+        t = threading.Thread(target=lambda: result.setdefault("cycles", churn(xs, q, stop, 3)))
+        if with_churn:
+            t.start()
+        for i in range(times):
+            q.submit(command(y, 1.0 + (i % 3)))
+        if with_churn:
+            time.sleep(0.05)
+            stop.set()
+            t.join()
+        q.wait()
+        st = hip_stats(xs, q.hwq)
+        got = y.cpu().numpy()
+        q.close()
+        return got, st
+
+    want = y_h.copy()
+    for i in range(times):
+        want = np.float32(0.5) * want + np.float32(1.0 + (i % 3))   # 0.5 * y is exact: one rounding, as the fma
+    plain, _ = run(1, False)
+    assert np.array_equal(plain.view(np.uint32), want.view(np.uint32))
+    got, st = run(2, True)
+    print("stats", st, flush=True)
+    assert st[2] > 0 and st[1] > 0, "no launch was flushed and replayed: the test did not exercise level 2"
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # argument checks
+    cmd = c_uint64()
+    h = xs.halhip()
+    assert h.HipGuardedKernelCommandCreate(byref(cmd), func, 0, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipGuardedKernelCommandCreate(byref(cmd), func, (1 << 18) + 1, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipGuardedKernelCommandCreate(byref(cmd), None, 4, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue

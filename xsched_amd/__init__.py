@@ -112,6 +112,8 @@ HALHIP_API = {
     "HipKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32,
                                          c_uint32, c_uint32, c_uint32, POINTER(c_void_p),
                                          POINTER(c_size_t), c_size_t, c_uint32]),
+    "HipGuardedKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32, c_uint32,
+                                                POINTER(c_void_p), POINTER(c_size_t), c_size_t, c_uint32]),
     "HipModuleKernelCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_uint32, c_uint32,
                                                c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_size_t]),
 }

@@ -118,6 +118,9 @@ def build_hip(extra, jobs):
         # the same program with its device code compressed, as large applications ship it
         _run(common + ["--offload-compress", "-o", os.path.join(LIB, "shim_app_packed"), "-L", LIB,
                        "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed", "-lshimhip"])
+    user = os.path.join(ROOT, "tests", "user_guarded_kernel.hip")
+    if os.path.exists(user):
+        _run(["hipcc"] + HIPFLAGS + extra + ["-shared", user, "-o", os.path.join(LIB, "libuserguarded.so")])
     mod = os.path.join(ROOT, "tests", "shim_module.hip")
     if os.path.exists(mod):
         _run(["hipcc", "--offload-arch=gfx950", "-O3", "--genco", mod, "-o", os.path.join(LIB, "shim_module.co")])

@@ -161,6 +161,46 @@ private:
     std::vector<char> storage_;
 };
 
+// A kernel of the caller's own with the guard of xsched/hip/guard.h compiled in. Its last
+// parameter is an XGuardArgs; the caller's arguments in front of it are copied at creation,
+// the guard arguments are appended at every launch (first or replay) as the queue then has
+// them. This is what binary instrumentation gives every CUDA kernel in the reference
+// (platforms/cuda/hal/src/level2/instrument.cpp:224-231, inject.cu:43-83); here the kernel's
+// author writes the three guard lines and any kernel becomes flushable at level 2.
+class HipUserGuardedCommand final : public HipGuardedCommand
+{
+public:
+    HipUserGuardedCommand(const void *func, uint32_t n_wg, dim3 block, void **args, const size_t *sizes,
+                          size_t n_args, uint32_t shmem)
+        : HipGuardedCommand(n_wg, 1), func_(func), block_(block), shmem_(shmem)
+    {
+        size_t total = 0;
+        for (size_t i = 0; i < n_args; ++i) total += ROUND_UP(sizes[i], 16);
+        storage_.resize(total);
+        arg_ptrs_.resize(n_args + 1);
+        size_t off = 0;
+        for (size_t i = 0; i < n_args; ++i) {
+            memcpy(storage_.data() + off, args[i], sizes[i]);
+            arg_ptrs_[i] = storage_.data() + off;
+            off += ROUND_UP(sizes[i], 16);
+        }
+    }
+protected:
+    // The kernel has one variant: below level 2 the guard finds the preempt word equal to the
+    // launch's epoch (nothing deactivates a level-1 queue) and no progress map.
+    virtual hipError_t LaunchKernel(hipStream_t stream, bool, const XGuardArgs &g) override
+    {
+        guard_args_ = g;
+        arg_ptrs_.back() = &guard_args_;
+        return hipLaunchKernel(func_, dim3(n_wg_), block_, arg_ptrs_.data(), shmem_, stream);
+    }
+private:
+    const void *func_; dim3 block_; uint32_t shmem_;
+    std::vector<char> storage_;
+    std::vector<void *> arg_ptrs_;
+    XGuardArgs guard_args_;
+};
+
 } // namespace
 
 std::shared_ptr<HwCommand> MakeRecordedEventWait(std::shared_ptr<HwCommand> record)
@@ -194,6 +234,22 @@ EXPORT_C_FUNC XResult HipMemsetWideCommandCreate(HwCommandHandle *cmd, void *dst
     if (cmd == nullptr || (width_bytes != 2 && width_bytes != 4)) return kXSchedErrorInvalidValue;
     if (((uintptr_t)dst & (width_bytes - 1)) != 0) return kXSchedErrorInvalidValue;
     *cmd = HwCommandManager::Add(std::make_shared<HipMemsetWideCommand>(dst, value, count, width_bytes));
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipGuardedKernelCommandCreate(HwCommandHandle *cmd, const void *host_func,
+                                                    uint32_t n_workgroups,
+                                                    uint32_t bx, uint32_t by, uint32_t bz,
+                                                    void **args, const size_t *arg_sizes, size_t n_args,
+                                                    uint32_t shared_mem_bytes)
+{
+    if (cmd == nullptr || host_func == nullptr || (n_args != 0 && (args == nullptr || arg_sizes == nullptr))) {
+        return kXSchedErrorInvalidValue;
+    }
+    if (n_workgroups == 0 || n_workgroups > GuardState::kMaxWorkGroups) return kXSchedErrorInvalidValue;
+    if (bx == 0 || by == 0 || bz == 0 || (uint64_t)bx * by * bz > 1024) return kXSchedErrorInvalidValue;
+    *cmd = HwCommandManager::Add(std::make_shared<HipUserGuardedCommand>(
+        host_func, n_workgroups, dim3(bx, by, bz), args, arg_sizes, n_args, shared_mem_bytes));
     return kXSchedSuccess;
 }
 
