@@ -38,6 +38,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "xsched/hip/guard_args.h"
+
 // The preempt word is replicated: copy c lives at flag[c * kXGuardFlagStrideWords],
 // c in [0, flag_mask]. Uncached reads of ONE address are served one after the other by
 // a single memory channel (about 27 ns each on MI355X), which would cap a kernel at
@@ -56,16 +58,6 @@
 // earlier launch (not just "none flushed") still has to check their progress bytes.
 #define kXGuardFlagStrideWords 64u /* 256 bytes between copies */
 
-struct XGuardArgs
-{
-    const uint32_t *flag;      // the queue's preempt word, copy 0 (deactivation count)
-    uint8_t        *done;      // progress map: done[w] == gen once work-group w has committed; may be null
-    uint32_t        epoch;     // deactivation count this launch was enqueued under
-    uint32_t        resume;    // nonzero: skip work-groups that have already committed
-    uint32_t        flag_mask; // number of copies of the preempt word minus one (2^k - 1)
-    uint32_t        gen;       // generation tag of this command in its progress map (1..255)
-    uint32_t       *flushed;   // the queue's "a work-group of this epoch was flushed" word; may be null
-};
 
 __device__ __forceinline__ const uint32_t *xguard_flag_copy(const XGuardArgs &g, uint32_t wg)
 {
@@ -140,6 +132,11 @@ __device__ __forceinline__ bool xguard_epoch_flushed(const XGuardArgs &g)
     return g.flushed != nullptr && (uint32_t)__builtin_amdgcn_readfirstlane((int)*g.flushed) == g.epoch;
 }
 
+/// An XGuardArgs of all zeroes switches the guard off: every work-group runs and nothing is
+/// recorded. It is what a program passes that launches a guarded kernel itself, with no
+/// queue behind the launch (`kernel<<<grid, block, 0, stream>>>(..., XGuardArgs{})`).
+__device__ __forceinline__ bool xguard_inert(const XGuardArgs &g) { return g.flag == nullptr; }
+
 /// Guard of a work-group that is ONE wavefront (blockDim == 64): the decision is
 /// wave-uniform by construction, no LDS or barrier is needed.
 class XGuardWave
@@ -150,6 +147,7 @@ public:
     /// False: this work-group must not run (flushed, or finished by an earlier launch).
     __device__ __forceinline__ bool Enter() const
     {
+        if (xguard_inert(g_)) return true;
         const bool earlier_flushed = xguard_epoch_flushed(g_);
         if (xguard_read_flag(xguard_flag_copy(g_, wg_)) != g_.epoch) {
             if ((threadIdx.x & 63) == 0) xguard_note_flush(g_);
@@ -181,6 +179,7 @@ public:
 
     __device__ __forceinline__ bool Enter() const
     {
+        if (xguard_inert(g_)) return true;
         if (threadIdx.x < 64) {
             const bool earlier_flushed = xguard_epoch_flushed(g_);
             bool go = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
@@ -199,6 +198,7 @@ public:
     /// at the same point; it contains two barriers.
     __device__ __forceinline__ bool StillCurrent() const
     {
+        if (xguard_inert(g_)) return true;
         __syncthreads();
         if (threadIdx.x == 0) {
             const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
@@ -215,6 +215,7 @@ public:
     /// has in front of its write-out.
     __device__ __forceinline__ bool WaveStillCurrent() const
     {
+        if (xguard_inert(g_)) return true;
         const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
         if (!current && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
         return current;
@@ -224,6 +225,7 @@ public:
     /// work between the calls: `pending = WavePollBegin(); ...; if (!WavePollEnd(pending))`.
     __device__ __forceinline__ uint32_t WavePollBegin() const
     {
+        if (xguard_inert(g_)) return g_.epoch;
         return xguard_read_flag_begin(xguard_flag_copy(g_, wg_));
     }
 

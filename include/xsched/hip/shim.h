@@ -10,6 +10,10 @@
  * (platforms/hip/shim/src/shim.cpp:21-322, entry points generated into
  * platforms/hip/shim/src/intercept.cpp), which replaces libamdhip64.so as a whole.
  *
+ * Kernels that have the guard of xsched/hip/guard.h compiled in (last parameter an
+ * XGuardArgs, one-dimensional grid) are submitted as guarded commands and can be flushed and
+ * replayed at level 2; all other kernels are drain points there, as in the reference.
+ *
  * Intercepted:
  *   kernels   hipLaunchKernel, hipModuleLaunchKernel, hipExtModuleLaunchKernel,
  *             hipLaunchCooperativeKernel, hipExtLaunchKernel              (shim.cpp:34-98)
@@ -57,7 +61,8 @@ XResult HipShimKernelArgLayout(const void *image, size_t bytes, const char *kern
  * [2] kernel launches passed straight through (no XQueue on the stream, null stream),
  * [3] copies and fills submitted as commands, [4] copies done after draining the XQueue,
  * [5] event records submitted as commands, [6] cross-queue event waits,
- * [7] kernels whose argument layout is known. */
+ * [7] kernels whose argument layout is known. (Guarded launches are among [0]; the line that
+ * XSCHED_SHIM_STATS=1 prints at exit also has them, and the queues' own counters.) */
 XResult HipShimGetStats(uint64_t *out);
 
 #ifdef __cplusplus

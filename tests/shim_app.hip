@@ -8,8 +8,16 @@
 //   shim_app --load SECONDS       device-filling kernels back to back on one stream
 //   shim_app --probe N PERIOD_US  a short kernel every PERIOD_US, launch-to-completion latency
 //   shim_app --leak               leaves main() with streams, events and memory never released
+//   shim_app --load-guarded SECONDS  like --load with a kernel that has the XSched guard compiled in
+//
+// The guard (xsched/hip/guard.h) is the one thing here that belongs to XSched: a kernel with
+// an XGuardArgs as its last parameter. The program launches it like any other kernel and
+// passes zeroes, which switch the guard off; with the shim in front, the queue supplies the
+// real arguments and the launch can be flushed and replayed at level 2.
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
+
+#include "xsched/hip/guard.h"
 
 #include <algorithm>
 #include <chrono>
@@ -108,6 +116,65 @@ __global__ void Busy(uint32_t *out, uint32_t iters)
     if (v == 0x12345678u) out[0] = v; // keeps the loop; practically never true
 }
 
+// The guarded load: every work-group spins like Busy, looks at the preempt word every 1024
+// steps (and leaves without a trace when the queue has been deactivated), and counts itself in
+// `runs` at the end: a work-group that took effect twice, or never, shows there.
+__global__ __launch_bounds__(256)
+void BusyGuarded(uint32_t *runs, uint32_t iters, XGuardArgs g)
+{
+    __shared__ uint32_t guard_word;
+    XGuardBlock guard(g, blockIdx.x, &guard_word);
+    if (!guard.Enter()) return;
+    uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint32_t done = 0; done < iters; done += 1024) {
+        // (not an affine map like Busy's: the compiler would fold 1024 steps of that into one)
+        for (uint32_t i = 0; i < 1024; ++i) v = (v ^ (v >> 13)) * 1664525u + 1013904223u;
+        if (!guard.StillCurrent()) return;
+    }
+    if (threadIdx.x == 0) runs[blockIdx.x] += 1 + (v == 0x12345678u);
+    guard.Commit();
+}
+
+// In place and not idempotent, for the checks: y = 0.5 * y + b over 1024 elements per work-group.
+__global__ __launch_bounds__(256)
+void AffineGuarded(float *y, float b, uint32_t n, XGuardArgs g)
+{
+    __shared__ uint32_t guard_word;
+    XGuardBlock guard(g, blockIdx.x, &guard_word);
+    if (!guard.Enter()) return;
+    for (uint32_t i = blockIdx.x * 1024 + threadIdx.x; i < (blockIdx.x + 1) * 1024 && i < n; i += 256) {
+        y[i] = __builtin_fmaf(0.5f, y[i], b);
+    }
+    guard.Commit();
+}
+
+static int LoadGuarded(double seconds)
+{
+    hipStream_t s;
+    uint32_t *runs;
+    constexpr uint32_t kGroups = 2048;
+    CHECK(hipStreamCreate(&s));
+    CHECK(hipMalloc(&runs, kGroups * 4));
+    CHECK(hipMemset(runs, 0, kGroups * 4));
+    printf("ready\n"); fflush(stdout);
+    const auto t0 = std::chrono::steady_clock::now();
+    uint32_t kernels = 0;
+    while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < seconds) {
+        for (int i = 0; i < 8; ++i) BusyGuarded<<<kGroups, 256, 0, s>>>(runs, 92160, XGuardArgs {});   // about 5 ms: long enough that waiting for its end hurts
+        CHECK(hipStreamSynchronize(s));
+        kernels += 8;
+    }
+    const double elapsed = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    std::vector<uint32_t> host(kGroups);
+    CHECK(hipMemcpy(host.data(), runs, kGroups * 4, hipMemcpyDeviceToHost));
+    uint32_t wrong = 0;
+    for (uint32_t w = 0; w < kGroups; ++w) wrong += host[w] != kernels;
+    printf("load kernels=%u ms_per_kernel=%.3f work_groups_not_exactly_once=%u\n", kernels, elapsed * 1e3 / kernels, wrong);
+    CHECK(hipFree(runs));
+    CHECK(hipStreamDestroy(s));
+    return wrong == 0 ? 0 : 4;
+}
+
 static int Load(double seconds)
 {
     hipStream_t s;
@@ -181,6 +248,7 @@ int main(int argc, char **argv)
     if (argc >= 2 && strcmp(argv[1], "--leak") == 0) return Leak();
     if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
     if (argc >= 3 && strcmp(argv[1], "--load") == 0) return Load(atof(argv[2]));
+    if (argc >= 3 && strcmp(argv[1], "--load-guarded") == 0) return LoadGuarded(atof(argv[2]));
     if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));
     const char *module_path = argc >= 2 ? argv[1] : nullptr;
 
@@ -340,6 +408,24 @@ int main(int argc, char **argv)
         // thread t: sum over i of (1 + i * (t + 1)) = 400 + (t + 1) * 79800
         Report("two threads, two streams", sums, (uint64_t)(400 + 79800) * 1000003u + (400 + 2 * 79800));
         CHECK(hipFree(acc[0])); CHECK(hipFree(acc[1])); CHECK(hipFree(ones));
+    }
+
+    // ---- 7c. a kernel with the XSched guard compiled in, launched like any other ----------------
+    {
+        constexpr uint32_t gn = 100000;
+        float *gy;
+        std::vector<float> gy_host(gn), gy_want(gn);
+        for (uint32_t i = 0; i < gn; ++i) gy_want[i] = gy_host[i] = (float)(i % 251) * 0.25f;
+        CHECK(hipMalloc(&gy, gn * 4));
+        CHECK(hipMemcpy(gy, gy_host.data(), gn * 4, hipMemcpyHostToDevice));
+        for (int rep = 0; rep < 50; ++rep) {
+            AffineGuarded<<<(gn + 1023) / 1024, 256, 0, s2>>>(gy, 1.0f + rep, gn, XGuardArgs {});
+            for (uint32_t i = 0; i < gn; ++i) gy_want[i] = 0.5f * gy_want[i] + (1.0f + rep);
+        }
+        CHECK(hipStreamSynchronize(s2));
+        CHECK(hipMemcpy(gy_host.data(), gy, gn * 4, hipMemcpyDeviceToHost));
+        Report("guarded kernel, 50 launches", Fnv(gy_host.data(), gn * 4), Fnv(gy_want.data(), gn * 4));
+        CHECK(hipFree(gy));
     }
 
     // ---- 7a. a launch the runtime refuses is refused the same way ------------------------------

@@ -122,8 +122,17 @@ def test_submit_moves_ownership_and_counts(xs):
     n = c_int64()
     xs.check(p.XQueueProfileHwCommandCount(xq, byref(n)))
     assert n.value == 1
+    # The queue turns idle when its launch thread comes back for the next command and finds
+    # none, which is a moment after the wait-all command has completed and WaitAll has returned
+    # (as in the reference: command_buffer.cpp:39-60).
+    import time
     st = c_int()
-    xs.check(p.XQueueQuery(xq, byref(st)))
+    deadline = time.time() + 2.0
+    while True:
+        xs.check(p.XQueueQuery(xq, byref(st)))
+        if st.value == xs.kQueueStateIdle or time.time() > deadline:
+            break
+        time.sleep(0.0005)
     assert st.value == xs.kQueueStateIdle
     xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hwq))
 

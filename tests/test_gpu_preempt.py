@@ -148,7 +148,12 @@ def test_resume_with_drop_commands(xs, gpu):
     xs.check(p.XQueueResume(q.xq, 1))  # kQueueResumeFlagDropCommands
     q.wait()
     state = c_int()
-    xs.check(p.XQueueQuery(q.xq, byref(state)))
+    deadline = time.time() + 2.0   # idle a moment after the wait has returned
+    while True:
+        xs.check(p.XQueueQuery(q.xq, byref(state)))
+        if state.value == xs.kQueueStateIdle or time.time() > deadline:
+            break
+        time.sleep(0.0005)
     assert state.value == xs.kQueueStateIdle
     got = y.cpu().numpy()
     assert np.all(got == 0.0)

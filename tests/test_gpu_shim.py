@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "xsched_amd", "lib")
 MODULE = os.path.join(LIB, "shim_module.co")
-CHECKS = 17  # lines the program prints, "done" and the error codes included
+CHECKS = 18  # lines the program prints, "done" and the error codes included
 
 
 def run(binary, args, env_extra, timeout=120):
@@ -68,7 +68,8 @@ def test_same_results_through_xqueues(plain_output, level, threshold, batch):
     # 3 saxpy + 2 argument shapes + 301 counter kernels + 2 spins + 4 adds on streams (checks 4-6)
     # + 2 * 400 from the threads + 3 module launches; the one null-stream launch goes straight through
     # + 2 around the captured graph (the three captured launches are recorded by the runtime)
-    assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3
+    assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3 + 50
+    assert s["guarded_cmds"] == 50   # the launches of the kernel that has the guard compiled in
     assert s["kernel_drained"] == 2 and s["kernel_direct"] == 1 + 3   # the two refused launches go to the runtime
     assert s["known_kernels"] >= 7 + 2
     assert s["event_cmds"] == 3 and s["event_waits"] == 1
@@ -82,7 +83,7 @@ def test_program_with_compressed_device_code(plain_output):
     out, err = run("shim_app_packed", [MODULE], shim_env(2))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] == 1159 and s["kernel_drained"] == 2
+    assert s["kernel_cmds"] == 1209 and s["kernel_drained"] == 2 and s["guarded_cmds"] == 50
 
 
 def test_without_auto_xqueue_everything_passes_through(plain_output):
@@ -127,31 +128,38 @@ def test_two_unmodified_processes_under_the_daemon():
     """Two processes that know nothing of XSched, one filling the device with back-to-back
     kernels (priority 0), one launching a short kernel every 2 ms (priority 1), both through the
     shim and the scheduler daemon with HPF (reference examples/Linux/1_transparent_sched). The
-    low-priority process's queue must get suspended while the other has work; the latencies of
-    the short kernel alone, next to the other process without XSched, and under XSched are
-    printed for the record."""
+    low-priority process's queue must get suspended while the other has work. Twice: with an
+    ordinary load kernel, which a suspension can only keep from being launched again, and with
+    one that has the guard compiled in (a zeroed XGuardArgs as its last argument in the
+    program's own launches), which a deactivation makes leave the device and the reactivation
+    replays; every work-group of it must still count itself exactly once per launch. The
+    latencies of the short kernel are printed for the record."""
     import tempfile
     import time
     xserver = os.path.join(LIB, "xserver")
     sock_dir = tempfile.mkdtemp(prefix="xsched-shim-")
     base = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+    probe_args = ["--probe", "300", "2000"]
 
     def start(binary, args, extra):
         print(f"starting {binary} {args} with {extra}", flush=True)
         return subprocess.Popen([os.path.join(LIB, binary)] + args, env=dict(base, **extra),
                                 stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
 
-    def wait_ready(proc):
-        assert proc.stdout.readline().strip() == "ready"
+    def next_to(load_binary, load_args, load_env, probe_binary, probe_env):
+        """Runs the probe while the load runs; returns (probe out, probe err, load out, load err)."""
+        load = start(load_binary, load_args, load_env)
+        assert load.stdout.readline().strip() == "ready"
+        probe = start(probe_binary, probe_args, probe_env)
+        probe_out, probe_err = probe.communicate(timeout=60)
+        load_out, load_err = load.communicate(timeout=60)
+        assert probe.returncode == 0 and load.returncode == 0, (probe_err[-1000:], load_out[-500:], load_err[-1000:])
+        return probe_out, probe_err, load_out, load_err
 
-    # the short kernel alone
-    alone, _ = run("shim_app_plain", ["--probe", "300", "2000"], {})
-    # next to the other process, hardware scheduling only
-    load = start("shim_app_plain", ["--load", "1.6"], {})
-    wait_ready(load)
-    native, _ = run("shim_app_plain", ["--probe", "300", "2000"], {})
-    load_out, _ = load.communicate(timeout=60)
-    assert load.returncode == 0, load_out
+    alone, _ = run("shim_app_plain", probe_args, {})
+    # hardware scheduling only
+    native = {kind: next_to("shim_app_plain", [flag, "1.6"], {}, "shim_app_plain", {})
+              for kind, flag in (("plain", "--load"), ("guarded", "--load-guarded"))}
 
     server = subprocess.Popen([xserver, "HPF"], env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN"))
     try:
@@ -161,28 +169,35 @@ def test_two_unmodified_processes_under_the_daemon():
         assert os.path.exists(os.path.join(sock_dir, "xsched-1.sock")), "xserver did not come up"
         common = {"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
                   "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}
-        load = start("shim_app", ["--load", "1.6"], dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0",
-                                                        XSCHED_AUTO_XQUEUE_THRESHOLD="2", XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"))
-        wait_ready(load)
-        probe = start("shim_app", ["--probe", "300", "2000"], dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
-        probe_out, probe_err = probe.communicate(timeout=60)
-        load_out2, load_err = load.communicate(timeout=60)
-        assert probe.returncode == 0 and load.returncode == 0, (probe_err[-1000:], load_err[-1000:])
+        low = dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
+                   XSCHED_AUTO_XQUEUE_BATCH_SIZE="1")
+        high = dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1")
+        under = {kind: next_to("shim_app", [flag, "1.6"], low, "shim_app", high)
+                 for kind, flag in (("plain", "--load"), ("guarded", "--load-guarded"))}
     finally:
         server.terminate()
         try:
             server.wait(timeout=5)
         except subprocess.TimeoutExpired:
             server.kill()
-    ls, ps = stats_of(load_err), stats_of(probe_err)
-    a, n, x = _percentiles(alone), _percentiles(native), _percentiles(probe_out)
-    print(f"short kernel p50/p99 us: alone {a[0]:.0f}/{a[1]:.0f}, next to the load without XSched {n[0]:.0f}/{n[1]:.0f}, "
-          f"under XSched {x[0]:.0f}/{x[1]:.0f}; load: {load_out.strip().splitlines()[-1]} | under XSched "
-          f"{load_out2.strip().splitlines()[-1]}; load queue deactivations {ls['deactivations']}",
-          file=sys.stderr, flush=True)
-    assert ps["deactivations"] == 0, "the high-priority process was suspended"
-    assert ls["deactivations"] > 50 and ls["reactivations"] > 50, "the daemon never suspended the low-priority process"
-    assert ps["kernel_cmds"] >= 300 and ls["kernel_cmds"] >= 32
+
+    a = _percentiles(alone)
+    print(f"short kernel alone: p50/p99 {a[0]:.0f}/{a[1]:.0f} us", file=sys.stderr, flush=True)
+    for kind in ("plain", "guarded"):
+        n, x = _percentiles(native[kind][0]), _percentiles(under[kind][0])
+        ls, ps = stats_of(under[kind][3]), stats_of(under[kind][1])
+        print(f"{kind} load: short kernel p50/p99 us next to it without XSched {n[0]:.0f}/{n[1]:.0f}, under XSched "
+              f"{x[0]:.0f}/{x[1]:.0f}; load without XSched: {native[kind][2].strip().splitlines()[-1]} | under XSched: "
+              f"{under[kind][2].strip().splitlines()[-1]}; its queue: deactivations {ls['deactivations']}, "
+              f"replayed launches {ls['replays']}, guarded commands {ls['guarded_cmds']}", file=sys.stderr, flush=True)
+        assert ps["deactivations"] == 0, "the high-priority process was suspended"
+        assert ls["deactivations"] > 50 and ls["reactivations"] > 50, "the daemon never suspended the low-priority process"
+        assert ps["kernel_cmds"] >= 300 and ls["kernel_cmds"] >= 32
+    gs = stats_of(under["guarded"][3])
+    assert gs["guarded_cmds"] == gs["kernel_cmds"] and gs["replays"] > 0, "no guarded launch was flushed and replayed"
+    assert "work_groups_not_exactly_once=0" in under["guarded"][2] and "work_groups_not_exactly_once=0" in native["guarded"][2]
+    # what the guard is for: the short kernel no longer waits for the load's 5 ms kernel to finish
+    assert _percentiles(under["guarded"][0])[1] < _percentiles(native["guarded"][0])[0] / 3
 
 
 @pytest.mark.parametrize("level", [1, 2])

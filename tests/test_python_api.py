@@ -39,6 +39,11 @@ def test_queue_life_cycle_through_the_reference_shaped_interface():
         assert XSched.XQueueSubmit(xq, cmd) == XResult.kXSchedSuccess
     assert XSched.XQueueWaitAll(xq) == XResult.kXSchedSuccess
     assert np.array_equal(c, a + b)
+    # idle a moment after WaitAll has returned: when the launch thread comes back and finds nothing
+    import time
+    deadline = time.time() + 2.0
+    while XSched.XQueueQuery(xq)[1] != XQueueState.kQueueStateIdle and time.time() < deadline:
+        time.sleep(0.0005)
     assert XSched.XQueueQuery(xq) == (XResult.kXSchedSuccess, XQueueState.kQueueStateIdle)
     res, count = XSched.XQueueProfileHwCommandCount(xq)
     assert res == XResult.kXSchedSuccess and count == 3

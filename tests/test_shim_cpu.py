@@ -122,6 +122,8 @@ def test_layouts_follow_the_c_signatures(app_bundle):
         # struct of 50 uint32_t by value, uint32_t *
         "_Z7SumWide4WidePj": [(0, 200), (200, 8)],
         "_Z4Bumpv": [],
+        # float *, float, uint32_t, then the 40-byte XGuardArgs the shim recognises by this name
+        "_Z13AffineGuardedPffj10XGuardArgs": [(0, 8), (8, 4), (12, 4), (16, 40)],
     }
     for kernel, args in by_hand.items():
         res, got, n = _layout(bundle, kernel)
@@ -268,4 +270,4 @@ def test_reader_under_address_and_ub_sanitizers(tmp_path):
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-4000:]
     lines = proc.stdout.strip().splitlines()
     assert len(lines) == 3 and all("refused" in line for line in lines), proc.stdout
-    assert lines[0].split(":")[1].strip().startswith("8 kernels") and lines[2].split(":")[1].strip().startswith("2 kernels")
+    assert lines[0].split(":")[1].strip().startswith("10 kernels") and lines[2].split(":")[1].strip().startswith("2 kernels")

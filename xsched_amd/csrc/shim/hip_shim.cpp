@@ -39,6 +39,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "code_object.h"
+#include "xsched/hip/guard_args.h"
 #include "../hip/shim_hooks.h"
 #include "xsched/hip/hal.h"
 #include "xsched/hip/shim.h"
@@ -120,9 +121,9 @@ struct Stats
 {
     std::atomic<uint64_t> kernel_cmds { 0 }, kernel_drained { 0 }, kernel_direct { 0 };
     std::atomic<uint64_t> mem_cmds { 0 }, mem_drained { 0 }, event_cmds { 0 }, event_waits { 0 };
-    std::atomic<uint64_t> known_kernels { 0 };
+    std::atomic<uint64_t> known_kernels { 0 }, guarded_cmds { 0 };
     // summed over the hardware queues of streams at their destruction
-    std::atomic<uint64_t> queue_launches { 0 }, deactivations { 0 }, reactivations { 0 };
+    std::atomic<uint64_t> queue_launches { 0 }, deactivations { 0 }, reactivations { 0 }, replays { 0 };
 };
 
 // A registered fat binary is read when the first of its kernels is launched: a large program
@@ -179,11 +180,12 @@ void PrintStats()
     const Stats &t = S().stats;
     fprintf(stderr, "[xsched shim] kernel_cmds=%lu kernel_drained=%lu kernel_direct=%lu mem_cmds=%lu "
             "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu queue_launches=%lu "
-            "deactivations=%lu reactivations=%lu\n",
+            "deactivations=%lu reactivations=%lu guarded_cmds=%lu replays=%lu\n",
             (unsigned long)t.kernel_cmds, (unsigned long)t.kernel_drained, (unsigned long)t.kernel_direct,
             (unsigned long)t.mem_cmds, (unsigned long)t.mem_drained, (unsigned long)t.event_cmds,
             (unsigned long)t.event_waits, (unsigned long)t.known_kernels, (unsigned long)t.queue_launches,
-            (unsigned long)t.deactivations, (unsigned long)t.reactivations);
+            (unsigned long)t.deactivations, (unsigned long)t.reactivations, (unsigned long)t.guarded_cmds,
+            (unsigned long)t.replays);
 }
 
 constexpr unsigned kStreamCapturing = 1u << 31; // kept next to the stream's creation flags
@@ -286,6 +288,18 @@ std::shared_ptr<const KernelLayout> LayoutOfHostFunction(const void *host_functi
 }
 
 // ---- launches -------------------------------------------------------------------------------
+
+/// True for a kernel whose last parameter is an XGuardArgs passed by value: the Itanium
+/// mangling of the parameter list then ends in "10XGuardArgs" and the last explicit argument
+/// has that struct's size. (A kernel declared extern "C" has no mangled parameter list and is
+/// not recognised.)
+bool TakesGuardArgs(const KernelLayout &layout)
+{
+    static const char kSuffix[] = "10XGuardArgs";
+    constexpr size_t kLen = sizeof kSuffix - 1;
+    if (layout.args.empty() || layout.args.back().size != sizeof(XGuardArgs)) return false;
+    return layout.name.size() > kLen && layout.name.compare(layout.name.size() - kLen, kLen, kSuffix) == 0;
+}
 
 /// Every explicit argument copied to its offset: the form hipModuleLaunchKernel's `extra` takes.
 std::vector<char> Pack(const KernelLayout &layout, void **params)
@@ -595,6 +609,18 @@ hipError_t hipLaunchKernel(const void *function_address, dim3 numBlocks, dim3 di
         std::vector<size_t> sizes(layout->args.size());
         for (size_t i = 0; i < sizes.size(); ++i) sizes[i] = layout->args[i].size;
         HwCommandHandle cmd = 0;
+        // A kernel whose last parameter is an XGuardArgs (its mangled name says so) has the
+        // work-group entry guard compiled in: with a one-dimensional grid it is submitted as a
+        // guarded command, the queue supplying the guard arguments in place of the caller's,
+        // and can be flushed and replayed at level 2.
+        if (TakesGuardArgs(*layout) && numBlocks.y == 1 && numBlocks.z == 1 &&
+            HipGuardedKernelCommandCreate(&cmd, function_address, numBlocks.x, dimBlocks.x, dimBlocks.y, dimBlocks.z,
+                                          args, sizes.data(), sizes.size() - 1, (uint32_t)sharedMemBytes) == kXSchedSuccess) {
+            SubmitHandle(xq, cmd);
+            S().stats.kernel_cmds++;
+            S().stats.guarded_cmds++;
+            return hipSuccess;
+        }
         const XResult res = HipKernelCommandCreate(&cmd, function_address, numBlocks.x, numBlocks.y, numBlocks.z,
                                                    dimBlocks.x, dimBlocks.y, dimBlocks.z, args, sizes.data(),
                                                    sizes.size(), (uint32_t)sharedMemBytes);
@@ -935,6 +961,7 @@ hipError_t hipStreamDestroy(hipStream_t stream)
             uint64_t counters[8] = {};
             if (HipQueueGetStats(hwq, counters) == kXSchedSuccess) {
                 S().stats.queue_launches += counters[0];
+                S().stats.replays += counters[1];
                 S().stats.deactivations += counters[2];
                 S().stats.reactivations += counters[3];
             }
