@@ -119,12 +119,12 @@ def contended_run(H, cfg, steps, warmup, bg_warm=8, bg_cmds=40):
                 "deadline_miss": int(res.fg_deadline_miss), "stats": list(res.stats)}
 
 
-def recorded_traffic(bg_n):
-    """HBM bytes per launch of the plain 2^28 AXPY kernel as recorded by the two
-    rocprofv3 counter runs summarised under profiles/ (counters cannot be read from
-    inside this process); None for any other size or when the summary is absent."""
-    path = os.path.join(ROOT, "profiles", "axpy_2p28_hbm_traffic.md")
-    if bg_n != 1 << 28 or not os.path.exists(path):
+def recorded_traffic(summary, applies=True):
+    """HBM bytes per launch of a kernel as recorded by the two rocprofv3 counter runs
+    summarised in profiles/<summary> (counters cannot be read from inside this process);
+    None when the workload is not the one that summary covers, or the summary is absent."""
+    path = os.path.join(ROOT, "profiles", summary)
+    if not applies or not os.path.exists(path):
         return None
     for ln in open(path):
         if ln.startswith("traffic_bytes_per_launch_plain:"):
@@ -170,7 +170,7 @@ def config2(H, a):
                   "contended_GBs": axpy_bytes(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e9,
                   "commands_in_timed_region": r["bg_cont_cmds"]}
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(bg_n),
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("axpy_2p28_hbm_traffic.md", bg_n == 1 << 28),
                         "kernel": "AxpyVec4Kernel", "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
                         "avg_launch_ms": per_launch_ms}
     if not a.quick:
@@ -212,7 +212,7 @@ def config3(H, a):
                   "contended_TFLOPs": gemm_flops(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e12,
                   "commands_in_timed_region": r["bg_cont_cmds"], "level2_stats": r["stats"]}
     line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
-                        "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": None, "kernel": "GemmBf16Kernel",
+                        "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": recorded_traffic("gemm_8192_hbm_traffic.md"), "kernel": "GemmBf16Kernel",
                         "algorithmic_flops_per_launch": gemm_flops(bg_n), "avg_launch_ms": per_launch_ms}
     if not a.quick:
         ms_plain = bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 20, 4)
@@ -265,7 +265,7 @@ def config4(H, a):
                       hist_bytes(bg_n) * head["bg_alone_cmds"] / head["bg_alone_elapsed"] / 1e9,
                   "contended_GBs": hist_bytes(bg_n) * head["bg_cont_cmds"] / head["bg_cont_elapsed"] / 1e9}
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "HistogramKernel + HistogramMergeKernel",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("histogram_2p26_hbm_traffic.md"), "kernel": "HistogramKernel + HistogramMergeKernel",
                         "algorithmic_bytes_per_launch": hist_bytes(bg_n), "avg_launch_ms": per_launch_ms,
                         "note": "one queue streaming guarded histogram commands back to back; a command is the "
                                 "counting kernel followed by the merge kernel, avg_launch_ms covers both"}

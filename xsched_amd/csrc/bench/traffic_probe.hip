@@ -1,14 +1,19 @@
 // Small driver for hardware-counter runs: launches a plain copy kernel of known size
-// (1 GiB read + 1 GiB written) and then the AXPY victim kernel through an XQueue in
-// its three forms (plain, guarded at level 1, guarded at level 2), a few times each.
+// (1 GiB read + 1 GiB written) and then a victim kernel through an XQueue, a few times:
+//   traffic_probe [n] [reps]          AXPY of n elements in its three forms (plain, guarded at
+//                                     level 1, guarded at level 2)
+//   traffic_probe [n] [reps] hist     histogram of 2^26 Zipf keys, plain and guarded at level 2
+//   traffic_probe [n] [reps] gemm     bf16 GEMM 8192^3, plain and guarded at level 2
 // Run it under `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`: the copy kernel's
-// counters give the scale factor of the counter, the AXPY rows the kernel's real HBM
+// counters give the scale factor of the counter, the other rows the kernels' real HBM
 // traffic per launch.
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 #include <hip/hip_runtime.h>
 
+#include "xsched/hip/bench.h"
 #include "xsched/hip/hal.h"
 #include "xsched/xsched.h"
 
@@ -44,6 +49,30 @@ int main(int argc, char **argv)
     CHECK_HIP(hipStreamSynchronize(stream));
 
     CHECK_X(XHintSetScheduler(kSchedulerAppManaged, kPolicyUnknown));
+    if (argc > 3) {
+        // The harness of bench.py fills the seeded inputs and streams `reps` background commands.
+        const bool hist = strcmp(argv[3], "hist") == 0;
+        for (int pass = 0; pass < 2; ++pass) {
+            XBenchConfig cfg;
+            memset(&cfg, 0, sizeof cfg);
+            cfg.n_bg = 1;
+            cfg.bg.kind = hist ? kXBenchHist : kXBenchGemm;
+            cfg.bg.guard = pass;                         // 0 plain, 1 guarded at level 2
+            cfg.bg.n = hist ? (uint64_t)1 << 26 : 8192;
+            cfg.bg.level = pass ? kPreemptLevelDeactivate : kPreemptLevelBlock;
+            cfg.bg.threshold = 2; cfg.bg.batch = 1;
+            cfg.fg = cfg.bg; cfg.fg.n = hist ? (uint64_t)1 << 20 : 1024; cfg.fg.period_us = 1000;
+            cfg.bg_burst = reps;
+            cfg.seed = 7;
+            XBench *b = XBenchCreate(&cfg);
+            if (b == nullptr) { fprintf(stderr, "XBenchCreate failed\n"); return 1; }
+            XBenchPhaseResult res;
+            CHECK_X(XBenchRunBackgroundAlone(b, reps, &res));
+            XBenchDestroy(b);
+        }
+        printf("traffic_probe: %s reps=%d copy_bytes_read=%zu copy_bytes_written=%zu\n", argv[3], reps, n * 4, n * 4);
+        return 0;
+    }
     HwQueueHandle hwq;
     XQueueHandle xq;
     CHECK_X(HipQueueCreate(&hwq, stream));
