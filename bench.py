@@ -340,6 +340,80 @@ def shim_launch_cost():
     return out
 
 
+def transparent_preemption():
+    """Two plain HIP processes (tests/shim_app.hip), one filling the device with 5 ms kernels that
+    have the guard compiled in (priority 0), one launching a short kernel every 2 ms (priority 1):
+    the short kernel's launch-to-completion latency alone, next to the load under hardware
+    scheduling, and with both processes under the interception shim, the scheduler daemon (HPF)
+    and level 2. Informational; None when something it needs has not been built or a run fails."""
+    import re
+    import subprocess
+    import tempfile
+    lib = os.path.join(os.path.dirname(os.path.abspath(__file__)), "xsched_amd", "lib")
+    need = [os.path.join(lib, n) for n in ("shim_app", "shim_app_plain", "xserver")]
+    if not all(os.path.exists(n) for n in need):
+        return None
+    base = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+    probe_args = ["--probe", "300", "2000"]
+
+    def percentiles(out):
+        m = re.search(r"probe n=(\d+) p50_us=([\d.]+) p99_us=([\d.]+)", out)
+        return {"p50": float(m.group(2)), "p99": float(m.group(3))} if m else None
+
+    def next_to(binary, load_env, probe_env):
+        load = subprocess.Popen([os.path.join(lib, binary), "--load-guarded", "1.6"], env=dict(base, **load_env),
+                                stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        try:
+            if load.stdout.readline().strip() != "ready":
+                return None
+            probe = subprocess.run([os.path.join(lib, binary)] + probe_args, env=dict(base, **probe_env),
+                                   capture_output=True, text=True, timeout=60)
+            load_out, load_err = load.communicate(timeout=60)
+        finally:
+            if load.poll() is None:
+                load.kill()
+        if probe.returncode != 0 or load.returncode != 0:
+            return None
+        m = re.search(r"ms_per_kernel=([\d.]+) work_groups_not_exactly_once=(\d+)", load_out)
+        stats = dict(item.split("=") for item in re.search(r"\[xsched shim\] (.*)", load_err).group(1).split()) \
+            if "[xsched shim]" in load_err else {}
+        return {"fg": percentiles(probe.stdout), "load_ms_per_kernel": float(m.group(1)) if m else None,
+                "load_work_groups_not_exactly_once": int(m.group(2)) if m else None,
+                "load_queue_deactivations": int(stats["deactivations"]) if stats else None,
+                "load_replayed_launches": int(stats["replays"]) if stats else None}
+
+    try:
+        alone = subprocess.run([os.path.join(lib, "shim_app_plain")] + probe_args, env=base, capture_output=True,
+                               text=True, timeout=60)
+        native = next_to("shim_app_plain", {}, {})
+        sock_dir = tempfile.mkdtemp(prefix="xsched-bench-")
+        server = subprocess.Popen([os.path.join(lib, "xserver"), "HPF"],
+                                  env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN"))
+        try:
+            deadline = time.time() + 5
+            while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
+                time.sleep(0.01)
+            common = {"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
+                      "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}
+            under = next_to("shim_app", dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
+                                             XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"),
+                            dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
+        finally:
+            server.terminate()
+            try:
+                server.wait(timeout=5)
+            except subprocess.TimeoutExpired:
+                server.kill()
+    except (OSError, subprocess.SubprocessError, AttributeError):
+        return None
+    if native is None or under is None or alone.returncode != 0:
+        return None
+    return {"workload": "fg: 256x256-thread kernel every 2 ms, 300 samples; load: 2048x256-thread guarded kernels of "
+                        "5 ms back to back; two processes, plain HIP host code, percentile = sorted[floor(p*n)]",
+            "fg_alone_us": percentiles(alone.stdout), "hardware_scheduling_only": native,
+            "under_xsched_shim_daemon_level2": under}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -365,6 +439,7 @@ def main():
     line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
     if a.config == 2 and not a.quick:
         line["shim_launch_cost"] = shim_launch_cost()
+        line["transparent_preemption"] = transparent_preemption()
     if a.config == 2 and not a.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
     else:
