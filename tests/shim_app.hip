@@ -116,8 +116,8 @@ __global__ void Busy(uint32_t *out, uint32_t iters)
     if (v == 0x12345678u) out[0] = v; // keeps the loop; practically never true
 }
 
-// The guarded load: every work-group spins like Busy, looks at the preempt word every 1024
-// steps (and leaves without a trace when the queue has been deactivated), and counts itself in
+// The guarded load: every work-group spins like Busy, looks at the preempt word every 256
+// steps (about every 14 us) (and leaves without a trace when the queue has been deactivated), and counts itself in
 // `runs` at the end: a work-group that took effect twice, or never, shows there.
 __global__ __launch_bounds__(256)
 void BusyGuarded(uint32_t *runs, uint32_t iters, XGuardArgs g)
@@ -126,9 +126,9 @@ void BusyGuarded(uint32_t *runs, uint32_t iters, XGuardArgs g)
     XGuardBlock guard(g, blockIdx.x, &guard_word);
     if (!guard.Enter()) return;
     uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
-    for (uint32_t done = 0; done < iters; done += 1024) {
-        // (not an affine map like Busy's: the compiler would fold 1024 steps of that into one)
-        for (uint32_t i = 0; i < 1024; ++i) v = (v ^ (v >> 13)) * 1664525u + 1013904223u;
+    for (uint32_t done = 0; done < iters; done += 256) {
+        // (not an affine map like Busy's: the compiler would fold the fixed number of steps into one)
+        for (uint32_t i = 0; i < 256; ++i) v = (v ^ (v >> 13)) * 1664525u + 1013904223u;
         if (!guard.StillCurrent()) return;
     }
     if (threadIdx.x == 0) runs[blockIdx.x] += 1 + (v == 0x12345678u);
