@@ -327,7 +327,15 @@ def test_user_written_guarded_kernel_is_flushed_and_replayed_exactly_once(xs, gp
     print(f"case user-guarded n={n} times={times} work-groups={n_wg}", flush=True)
     y_h = oracle.fill_uniform(21, 2, 0, n)
 
+    from xsched_amd.xsched_api import XSched, XResult
+
     def command(y, b):
+        if int(b) % 2:   # through the Python interface ...
+            res, cmd = XSched.HipGuardedKernelCommandCreate(
+                func, n_wg, (256, 1, 1), [ctypes.c_void_p(y.data_ptr()), ctypes.c_float(b), ctypes.c_size_t(n)])
+            assert res == XResult.kXSchedSuccess
+            return cmd
+        # ... and through the C entry point itself
         y_ptr, b_val, n_val = ctypes.c_void_p(y.data_ptr()), ctypes.c_float(b), ctypes.c_size_t(n)
         args = (ctypes.c_void_p * 3)(ctypes.addressof(y_ptr), ctypes.addressof(b_val), ctypes.addressof(n_val))
         sizes = (ctypes.c_size_t * 3)(8, 4, 8)

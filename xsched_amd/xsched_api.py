@@ -215,6 +215,21 @@ class XSched:
         return _res(res), cmd.value
 
     @staticmethod
+    def HipGuardedKernelCommandCreate(host_func: int, n_workgroups: int, block: Tuple[int, int, int],
+                                      args: list, shared_mem_bytes: int = 0) -> Tuple[XResult, HwCommandHandle]:
+        """A kernel of the caller's own that has the guard of xsched/hip/guard.h compiled in and an
+        XGuardArgs as its last parameter. `host_func` is the kernel's host-side address, `args` the
+        parameters in front of the XGuardArgs as ctypes values (c_void_p, c_float, c_size_t, ...);
+        they are copied before this returns."""
+        n = len(args)
+        ptrs = (ctypes.c_void_p * max(n, 1))(*[ctypes.addressof(a) for a in args])
+        sizes = (ctypes.c_size_t * max(n, 1))(*[ctypes.sizeof(a) for a in args])
+        cmd = ctypes.c_uint64(0)
+        res = _xs.halhip().HipGuardedKernelCommandCreate(ctypes.byref(cmd), ctypes.c_void_p(host_func), n_workgroups,
+                                                         block[0], block[1], block[2], ptrs, sizes, n, shared_mem_bytes)
+        return _res(res), cmd.value
+
+    @staticmethod
     def HostQueueCreate() -> Tuple[XResult, HwQueueHandle]:
         hwq = ctypes.c_uint64(0)
         res = _xs.halhost().HostQueueCreate(ctypes.byref(hwq))
