@@ -470,6 +470,35 @@ int main(int argc, char **argv)
         CHECK(hipFree(gbuf)); CHECK(hipFree(gone));
     }
 
+    // ---- 7d. the calls that are ordered but not deferred, between calls that are deferred ----------
+    {
+        constexpr uint32_t rows = 64, cols = 256;                      // a 64 x 256 matrix of uint32_t
+        uint32_t *m0, *m1, *pool_buf = nullptr;
+        CHECK(hipMalloc(&m0, rows * cols * 4)); CHECK(hipMalloc(&m1, rows * cols * 4));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)m0, 2, rows * cols, s1));
+        CHECK(hipMemsetD32Async((hipDeviceptr_t)m1, 0, rows * cols, s1));
+        AddInto<<<rows * cols / 256, 256, 0, s1>>>(m0, m0, 1, rows * cols);                    // m0 = 5
+        CHECK(hipMemcpy2DAsync(m1, cols * 4, m0, cols * 4, cols * 2, rows, hipMemcpyDeviceToDevice, s1)); // left half of m1 = 5
+        AddInto<<<rows * cols / 256, 256, 0, s1>>>(m1, m0, 0, rows * cols);                    // m1 = 10 | 5
+        CHECK(hipMallocAsync((void **)&pool_buf, rows * cols * 4, s1));
+        CHECK(hipMemcpyAsync(pool_buf, m1, rows * cols * 4, hipMemcpyDeviceToDevice, s1));
+        void *coop_args[] = { &pool_buf, &m0, &zero, &zero };
+        uint32_t count = rows * cols;
+        coop_args[3] = &count;
+        CHECK(hipLaunchCooperativeKernel((const void *)AddInto, dim3(rows * cols / 256), dim3(256), coop_args, 0, s1)); // + 5
+        CHECK(hipExtLaunchKernel((const void *)AddInto, dim3(rows * cols / 256), dim3(256), coop_args, 0, s1, nullptr, nullptr, 0)); // + 5
+        AddInto<<<rows * cols / 256, 256, 0, s1>>>(m1, pool_buf, 0, rows * cols);              // m1 += pool_buf
+        CHECK(hipFreeAsync(pool_buf, s1));
+        std::vector<uint32_t> m_host(rows * cols);
+        CHECK(hipMemcpyDtoH(m_host.data(), (hipDeviceptr_t)m1, rows * cols * 4));               // null stream, after s1
+        bad = 0;
+        for (uint32_t r = 0; r < rows; ++r) {
+            for (uint32_t c = 0; c < cols; ++c) bad += m_host[r * cols + c] != (c < cols / 2 ? 10u + 20u : 5u + 15u);
+        }
+        Report("ordered, not deferred calls", bad, 0);
+        CHECK(hipFree(m0)); CHECK(hipFree(m1));
+    }
+
     // ---- 8. kernels of a loaded module ------------------------------------------------------------
     if (module_path != nullptr) {
         hipModule_t mod;

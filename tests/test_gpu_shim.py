@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "xsched_amd", "lib")
 MODULE = os.path.join(LIB, "shim_module.co")
-CHECKS = 18  # lines the program prints, "done" and the error codes included
+CHECKS = 19  # lines the program prints, "done" and the error codes included
 
 
 def run(binary, args, env_extra, timeout=120):
@@ -68,9 +68,10 @@ def test_same_results_through_xqueues(plain_output, level, threshold, batch):
     # 3 saxpy + 2 argument shapes + 301 counter kernels + 2 spins + 4 adds on streams (checks 4-6)
     # + 2 * 400 from the threads + 3 module launches; the one null-stream launch goes straight through
     # + 2 around the captured graph (the three captured launches are recorded by the runtime)
-    assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3 + 50
+    # + 3 ordinary launches among the ordered-only calls (the cooperative and the ext launch drain)
+    assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3 + 50 + 3
     assert s["guarded_cmds"] == 50   # the launches of the kernel that has the guard compiled in
-    assert s["kernel_drained"] == 2 and s["kernel_direct"] == 1 + 3   # the two refused launches go to the runtime
+    assert s["kernel_drained"] == 2 + 2 and s["kernel_direct"] == 1 + 3   # refused launches; cooperative and ext launch
     assert s["known_kernels"] >= 7 + 2
     assert s["event_cmds"] == 3 and s["event_waits"] == 1
     # pinned and device-to-device copies and every fill are commands; pageable copies drain
@@ -83,7 +84,7 @@ def test_program_with_compressed_device_code(plain_output):
     out, err = run("shim_app_packed", [MODULE], shim_env(2))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] == 1209 and s["kernel_drained"] == 2 and s["guarded_cmds"] == 50
+    assert s["kernel_cmds"] == 1212 and s["kernel_drained"] == 4 and s["guarded_cmds"] == 50
 
 
 def test_without_auto_xqueue_everything_passes_through(plain_output):
@@ -115,7 +116,7 @@ def test_unmodified_binary_under_ld_preload(plain_output):
     out, err = run("shim_app_plain", [MODULE], shim_env(1, LD_PRELOAD=preload))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 2
+    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 4
 
 
 def _percentiles(out):
