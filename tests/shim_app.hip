@@ -251,6 +251,10 @@ int main(int argc, char **argv)
     if (argc >= 3 && strcmp(argv[1], "--load-guarded") == 0) return LoadGuarded(atof(argv[2]));
     if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));
     const char *module_path = argc >= 2 ? argv[1] : nullptr;
+    // Under the kernel-trace profiler the program without any library of this repository in it
+    // ends in a segmentation fault inside the exit handlers once it has used stream-ordered
+    // allocation; a profile run passes this switch and leaves section 7d out.
+    const bool skip_ordered_only = argc >= 3 && strcmp(argv[2], "--skip-ordered-only") == 0;
 
     constexpr size_t n = 1 << 16;
     hipStream_t s1, s2, s3;
@@ -471,7 +475,7 @@ int main(int argc, char **argv)
     }
 
     // ---- 7d. the calls that are ordered but not deferred, between calls that are deferred ----------
-    {
+    if (!skip_ordered_only) {
         constexpr uint32_t rows = 64, cols = 256;                      // a 64 x 256 matrix of uint32_t
         uint32_t *m0, *m1, *pool_buf = nullptr;
         CHECK(hipMalloc(&m0, rows * cols * 4)); CHECK(hipMalloc(&m1, rows * cols * 4));
