@@ -183,13 +183,18 @@ def config2(H, a):
                          "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
                          "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
         line["preempt_us"] = preempt_block(H, H.AXPY, bg_n, False)
-        # The other end of the AXPY trade-off (guard mode 3): a few long-lived waves per CU.
-        ms_sd = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 3)
-        sus, res, _ = preempt_latency(H, H.AXPY, bg_n, 2, 200, guard=3)
-        dev = device_drain(H, H.AXPY, bg_n, 2, 200, guard=3)
-        line["short_drain_variant"] = {
+        # For comparison: guarded launches on the plain kernel's grid (one wave per chunk,
+        # guard at work-group entry) instead of the two long-lived waves per CU.
+        os.environ["XSCHED_HIP_AXPY_GRID"] = "chunk"
+        try:
+            ms_cg = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 1)
+            sus, res, _ = preempt_latency(H, H.AXPY, bg_n, 2, 200)
+            dev = device_drain(H, H.AXPY, bg_n, 2, 200)
+        finally:
+            del os.environ["XSCHED_HIP_AXPY_GRID"]
+        line["chunk_grid_variant"] = {
             "level2_device_drain_p50": H.pct(dev, 0.5), "level2_device_drain_p99": H.pct(dev, 0.99),
-            "level2_GBs": axpy_bytes(bg_n) / ms_sd / 1e6, "level2_overhead_frac": 1.0 - ms_plain / ms_sd,
+            "level2_GBs": axpy_bytes(bg_n) / ms_cg / 1e6, "level2_overhead_frac": 1.0 - ms_plain / ms_cg,
             "level2_suspend_sync_p50": H.pct(sus, 0.5), "level2_suspend_sync_p99": H.pct(sus, 0.99),
             "level2_resume_p50": H.pct(res, 0.5), "level2_resume_p99": H.pct(res, 0.99)}
     return line

@@ -50,10 +50,12 @@ XResult HipQueueMarkEpochFlushed(HwQueueHandle hwq);
  *              command launches the plain variant.
  *          2 = always launch the guarded variant, even at level 1 (for measuring
  *              the cost of the guard).
- *          3 = like 1, but prefer the kernel's short-drain variant where it has one
- *              (AXPY: a few long-lived waves per CU instead of one wave per chunk: the
- *              device drains in 20-30 us instead of ~190 us after a deactivation, at
- *              ~8 % less bandwidth). Same as 1 for the other kernels. */
+ *          3 = same as 1 (kept for callers that asked for the AXPY's short-drain grid when
+ *              that was not yet its default).
+ * A guarded AXPY runs as two long-lived waves per CU that look at the preempt word in front
+ * of every chunk: after a deactivation the device drains in microseconds, at the bandwidth
+ * of the plain kernel. XSCHED_HIP_AXPY_GRID=chunk keeps the plain kernel's grid (one wave
+ * per chunk, guard at entry) for guarded launches as well: ~180 us of drain. */
 
 /* y[i] = fma(alpha, x[i], y[i]) in place, fp32, i < n. 128-bit loads/stores when
  * x and y are 16-byte aligned. */

@@ -76,6 +76,31 @@ def test_axpy_bit_exact(xs, gpu, n, level, guard):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("n", [1, 1024, 2048, 3 * 1024 + 1, 7 * 1024, 7 * 1024 * 513 + 2, (1 << 21) + 4099])
+@pytest.mark.parametrize("grid,steps", [("waves", 2), ("waves", 3), ("waves", 7), ("chunk", 1), ("chunk", 2), ("chunk", 3)])
+def test_axpy_guarded_grids_and_chunk_sizes(xs, gpu, monkeypatch, grid, steps, n):
+    """Both grids of a guarded AXPY with chunks of several steps, at lengths around the
+    chunk and step borders (a last chunk that is not full, 0..3 trailing scalars, fewer
+    chunks than waves, more steps in a chunk than the waves keep in flight)."""
+    torch = gpu
+    monkeypatch.setenv("XSCHED_HIP_AXPY_GRID", grid)
+    monkeypatch.setenv("XSCHED_HIP_AXPY_STEPS", str(steps))
+    print(f"case axpy-grid n={n} grid={grid} steps={steps}", flush=True)
+    x_h = oracle.fill_uniform(21, 1, 0, n)
+    y_h = oracle.fill_uniform(21, 2, 0, n)
+    x = torch.from_numpy(x_h.copy()).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, 2)
+    for _ in range(2):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    q.wait()
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    q.close()
+    want = oracle.axpy(0.5, x_h, y_h, 2)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_axpy_general_alpha_and_unaligned(xs, gpu):
     """alpha whose product is inexact (one rounding: fma) and a pointer that is only
     4-byte aligned (scalar fallback kernel)."""

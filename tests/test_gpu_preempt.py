@@ -35,12 +35,19 @@ def churn(xs, q, stop, seed, flags=0):
     return cycles
 
 
-@pytest.mark.parametrize("guard", [1, 3])          # 3 = few long-lived waves per CU
+# The grid of a guarded AXPY (long-lived waves with several steps of loads in flight, or one
+# wave per chunk with the guard at entry) and the steps of 1024 elements in a chunk: with
+# more than one step a chunk that has begun must be finished, or the replay would apply
+# its first steps twice.
+@pytest.mark.parametrize("grid,steps", [("waves", 1), ("waves", 2), ("waves", 7), ("chunk", 1), ("chunk", 4)])
 @pytest.mark.parametrize("suspend_flags", [0, 1])  # 1 = kQueueSuspendFlagSyncHwQueue
-def test_axpy_preempt_resume_bit_exact(xs, gpu, suspend_flags, guard):
+def test_axpy_preempt_resume_bit_exact(xs, gpu, monkeypatch, suspend_flags, grid, steps):
     torch = gpu
+    guard = 1
+    monkeypatch.setenv("XSCHED_HIP_AXPY_GRID", grid)
+    monkeypatch.setenv("XSCHED_HIP_AXPY_STEPS", str(steps))
     n, times = (1 << 24) + 5, 60
-    print(f"case axpy-preempt n={n} times={times} flags={suspend_flags} guard={guard}", flush=True)
+    print(f"case axpy-preempt n={n} times={times} flags={suspend_flags} grid={grid} steps={steps}", flush=True)
     x_h = oracle.fill_uniform(5, 1, 0, n)
     y_h = oracle.fill_uniform(5, 2, 0, n)
     x = torch.from_numpy(x_h).cuda()

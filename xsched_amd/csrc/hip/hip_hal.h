@@ -156,8 +156,7 @@ private:
 class HipGuardedCommand : public HipCommand
 {
 public:
-    /// guard_mode: 0 plain, 1 guarded at level >= 2, 2 guarded always, 3 like 1 with the
-    /// kernel's short-drain variant where it has one.
+    /// guard_mode: 0 plain, 1 guarded at level >= 2, 2 guarded always, 3 same as 1.
     HipGuardedCommand(uint32_t n_wg, int guard_mode)
         : HipCommand(guard_mode ? preempt::kCommandPropertyDeactivatable : preempt::kCommandPropertyNone)
         , n_wg_(n_wg), guard_mode_(guard_mode) {}

@@ -9,17 +9,19 @@
 // progress map after its last store.
 //
 // Two grids:
-//   one single-wave work-group per chunk (default). Short-lived waves give the best
-//       bandwidth (6.2-6.3 TB/s on MI355X) and let a concurrent kernel find free wave
-//       slots within microseconds. After a deactivation the device still has to start
-//       and retire every remaining work-group, empty: ~3.3 waves per nanosecond, so two
-//       launches of 262144 work-groups in flight drain in ~190 us.
-//   guard mode 3: a fixed number of waves per CU, each walking chunks c, c + G,
-//       c + 2G, ... and re-reading the preempt word while the next chunk's loads are in
-//       flight. Every wave stops at its next chunk and a launch queued behind has only G
-//       work-groups to retire: the device drains in 20-30 us. Long-lived waves stream
-//       at 5.3-5.8 TB/s, though (the same loss shows with larger chunks per work-group,
-//       or several waves per work-group), so this is the latency end of a trade-off.
+//   plain launches: one single-wave work-group per chunk. Short-lived waves stream at
+//       6.2-6.3 TB/s on MI355X and let a concurrent kernel find free wave slots within
+//       microseconds.
+//   guarded launches: two long-lived waves per CU, each walking chunks c, c + G,
+//       c + 2G, ... with the loads of three steps in flight, and reading the preempt word
+//       in front of every chunk. Same bandwidth as the plain grid (measured: 2 waves per CU
+//       6.2 TB/s, 1 per CU 4.1, 4 or more per CU 5.3-5.8 whatever the depth). After a
+//       deactivation every wave stops at its next chunk, about a microsecond away, and a
+//       launch queued behind has only G work-groups to retire: the device drains in 6 us
+//       (p50). With XSCHED_HIP_AXPY_GRID=chunk a guarded launch keeps the plain grid, with
+//       the guard at work-group entry: after a deactivation the device then still has to
+//       start and retire every remaining work-group, empty, at ~3.3 waves per nanosecond:
+//       two launches of 262144 work-groups in flight drain in ~180 us.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 #include "xsched/utils/env.h"
@@ -102,6 +104,12 @@ void AxpyVec4Kernel(float alpha, const float4 *x, float4 *y,
 
 // Guarded launches: grid-stride over chunks, see the head of this file. `n_chunks`
 // chunks of `steps` x 1024 elements; the progress map has one byte per chunk.
+// A wave walks its chunks c, c + G, c + 2G, ... step by step and keeps the loads of
+// kDepth steps in flight: step j is stored while steps j+1 .. j+kDepth-1 are on their
+// way and step j+kDepth is requested right behind the stores. The preempt word is read
+// in front of the first store of every chunk; a chunk that has begun is finished and
+// committed, so it is applied exactly once.
+template <uint32_t kDepth>
 __global__ __launch_bounds__(64)
 void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, uint32_t tail,
                           uint32_t steps, uint32_t n_chunks, XGuardArgs g)
@@ -109,62 +117,90 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
     constexpr uint32_t kVecPerStep = 4;
     constexpr uint32_t kStepVecs = kLanes * kVecPerStep;
     const uint32_t lane = threadIdx.x;
+    const uint32_t stride = gridDim.x;
     const uint32_t *flag = xguard_flag_copy(g, blockIdx.x);
     // an earlier launch of this epoch was flushed: this one must not run ahead of its replay
     if (xguard_epoch_flushed(g)) return;
 
-    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const uint64_t chunk_base = (uint64_t)c * steps * kStepVecs;
-        const bool full = chunk_base + (uint64_t)steps * kStepVecs <= n4;
-        const uint64_t base = chunk_base + lane;
-        float4 xv[kVecPerStep], yv[kVecPerStep];
-        if (full) {
+    // Ring slot d holds step ring_s[d] of chunk ring_c[d]; the slots follow each other in
+    // the wave's sequence of steps.
+    uint32_t ring_c[kDepth], ring_s[kDepth];
+    float4 xv[kDepth][kVecPerStep], yv[kDepth][kVecPerStep];
+    {
+        uint32_t c = blockIdx.x, st = 0;
+#pragma unroll
+        for (uint32_t d = 0; d < kDepth; ++d) {
+            ring_c[d] = c;
+            ring_s[d] = st;
+            if (++st == steps) { st = 0; c += stride; }
+        }
+    }
+#pragma unroll
+    for (uint32_t d = 0; d < kDepth; ++d) {
+        const uint32_t c = ring_c[d];
+        if (c < n_chunks && ((uint64_t)c + 1) * steps * kStepVecs <= n4) {
+            const uint64_t base = ((uint64_t)c * steps + ring_s[d]) * kStepVecs + lane;
 #pragma unroll
             for (uint32_t u = 0; u < kVecPerStep; ++u) {
-                xv[u] = ld_nt(&x[base + u * kLanes]);
-                yv[u] = ld_nt(&y[base + u * kLanes]);
+                xv[d][u] = ld_nt(&x[base + u * kLanes]);
+                yv[d][u] = ld_nt(&y[base + u * kLanes]);
             }
         }
-        // The scalar read of the preempt word waits for itself only: the vector loads
-        // above stay in flight across it. A flushed wave drops what it has loaded.
-        if (xguard_read_flag(flag) != g.epoch) {
-            if (lane == 0) xguard_note_flush(g);
-            return;
-        }
-        if (g.resume && g.done && xguard_committed(g, c)) continue;
+    }
 
-        if (full) {
+    bool skip = false;   // the chunk whose steps are passing by was committed before the flush
+    while (true) {
 #pragma unroll
-            for (uint32_t u = 0; u < kVecPerStep; ++u) {
-                st_nt(&y[base + u * kLanes], fma4(alpha, xv[u], yv[u]));
+        for (uint32_t d = 0; d < kDepth; ++d) {
+            const uint32_t c = ring_c[d];
+            const uint32_t st = ring_s[d];
+            if (c >= n_chunks) return;   // the sequence only grows: every later step is beyond, too
+            const bool full = ((uint64_t)c + 1) * steps * kStepVecs <= n4;
+            if (st == 0) {
+                // The scalar read of the preempt word waits for itself only: the vector loads
+                // stay in flight across it. A flushed wave drops what it has loaded.
+                if (xguard_read_flag(flag) != g.epoch) {
+                    if (lane == 0) xguard_note_flush(g);
+                    return;
+                }
+                skip = g.resume && g.done && xguard_committed(g, c);
+                if (!skip && !full) {
+                    // the last chunk of an array that does not fill it, and the 0..3 scalars behind
+                    const uint64_t chunk_base = (uint64_t)c * steps * kStepVecs;
+                    const uint64_t end = chunk_base + (uint64_t)steps * kStepVecs;
+                    for (uint64_t i = chunk_base + lane; i < end && i < n4; i += kLanes) {
+                        st_nt(&y[i], fma4(alpha, ld_nt(&x[i]), ld_nt(&y[i])));
+                    }
+                    if (c == n_chunks - 1 && lane < tail) {
+                        const float *xs = (const float *)(x + n4);
+                        float *ys = (float *)(y + n4);
+                        ys[lane] = __builtin_fmaf(alpha, xs[lane], ys[lane]);
+                    }
+                    if (g.done && lane == 0) xguard_commit(g, c);
+                }
             }
-            // Chunks of more than one step (arrays beyond 2^28 elements): the rest of the
-            // chunk, with registers of its own so that nothing is carried around the loop.
-            for (uint32_t s = 1; s < steps; ++s) {
-                const uint64_t b = base + (uint64_t)s * kStepVecs;
-                float4 xs[kVecPerStep], ys[kVecPerStep];
+            if (full && !skip) {
+                const uint64_t base = ((uint64_t)c * steps + st) * kStepVecs + lane;
 #pragma unroll
                 for (uint32_t u = 0; u < kVecPerStep; ++u) {
-                    xs[u] = ld_nt(&x[b + u * kLanes]);
-                    ys[u] = ld_nt(&y[b + u * kLanes]);
+                    st_nt(&y[base + u * kLanes], fma4(alpha, xv[d][u], yv[d][u]));
                 }
+                if (st == steps - 1 && g.done && lane == 0) xguard_commit(g, c);
+            }
+            // this slot's next step: kDepth steps further on in the sequence
+            uint32_t nc = c, ns = st + kDepth;
+            while (ns >= steps) { ns -= steps; nc += stride; }
+            ring_c[d] = nc;
+            ring_s[d] = ns;
+            if (nc < n_chunks && ((uint64_t)nc + 1) * steps * kStepVecs <= n4) {
+                const uint64_t nb = ((uint64_t)nc * steps + ns) * kStepVecs + lane;
 #pragma unroll
                 for (uint32_t u = 0; u < kVecPerStep; ++u) {
-                    st_nt(&y[b + u * kLanes], fma4(alpha, xs[u], ys[u]));
+                    xv[d][u] = ld_nt(&x[nb + u * kLanes]);
+                    yv[d][u] = ld_nt(&y[nb + u * kLanes]);
                 }
-            }
-        } else {
-            const uint64_t end = chunk_base + (uint64_t)steps * kStepVecs;
-            for (uint64_t i = chunk_base + lane; i < end && i < n4; i += kLanes) {
-                st_nt(&y[i], fma4(alpha, ld_nt(&x[i]), ld_nt(&y[i])));
-            }
-            if (c == n_chunks - 1 && lane < tail) {
-                const float *xs = (const float *)(x + n4);
-                float *ys = (float *)(y + n4);
-                ys[lane] = __builtin_fmaf(alpha, xs[lane], ys[lane]);
             }
         }
-        if (g.done && lane == 0) xguard_commit(g, c);
     }
 }
 
@@ -192,8 +228,9 @@ class HipAxpyCommand final : public HipGuardedCommand
 public:
     /// steps: chunk size per work-group in units of 1024 elements.
     HipAxpyCommand(float alpha, const float *x, float *y, size_t n, uint32_t steps, uint32_t n_wg,
-                   int guard_mode)
-        : HipGuardedCommand(n_wg, guard_mode), alpha_(alpha), x_(x), y_(y), n_(n), steps_(steps) {}
+                   int guard_mode, bool chunk_grid)
+        : HipGuardedCommand(n_wg, guard_mode), alpha_(alpha), x_(x), y_(y), n_(n), steps_(steps)
+        , chunk_grid_(chunk_grid) {}
 
 protected:
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
@@ -201,10 +238,10 @@ protected:
         if (n_ == 0) return hipSuccess;
         const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
         const dim3 grid(n_wg_), block(kLanes);
-        if (aligned && guarded && guard_mode_ == 3) {
+        if (aligned && guarded && !chunk_grid_) {
             const uint32_t waves = PersistentWaves();
             const dim3 pgrid(n_wg_ < waves ? n_wg_ : waves);
-            hipLaunchKernelGGL(AxpyPersistentKernel, pgrid, block, 0, stream, alpha_, (const float4 *)x_,
+            hipLaunchKernelGGL(AxpyPersistentKernel<3>, pgrid, block, 0, stream, alpha_, (const float4 *)x_,
                                (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
         } else if (aligned) {
             const uint64_t n4 = n_ / 4;
@@ -236,7 +273,7 @@ private:
     static uint32_t PersistentWaves()
     {
         static const uint32_t waves = []() {
-            int64_t per_cu = 8;
+            int64_t per_cu = 2;
             GetEnvInt64("XSCHED_HIP_AXPY_WAVES_PER_CU", per_cu);
             if (per_cu < 1) per_cu = 1;
             if (per_cu > 64) per_cu = 64;
@@ -254,6 +291,7 @@ private:
     float *y_;
     const size_t n_;
     const uint32_t steps_;
+    const bool chunk_grid_;   // guarded launches keep the one-wave-per-chunk grid
 };
 
 } // namespace axpy
@@ -286,6 +324,6 @@ EXPORT_C_FUNC XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, co
     const uint64_t per_wg = (uint64_t)steps * 1024;
     const uint32_t n_wg = n == 0 ? 1 : (uint32_t)((n + per_wg - 1) / per_wg);
     *cmd = HwCommandManager::Add(std::make_shared<axpy::HipAxpyCommand>(
-        alpha, (const float *)x, (float *)y, n, steps, n_wg, guard));
+        alpha, (const float *)x, (float *)y, n, steps, n_wg, guard, GetEnv("XSCHED_HIP_AXPY_GRID") == "chunk"));
     return kXSchedSuccess;
 }
