@@ -87,9 +87,9 @@ int main(int argc, char **argv)
         CHECK_X(XQueueWaitAll(xq));
     };
     run(0);                                                   // AxpyVec4Kernel<false, 4>
-    run(2);                                                   // AxpyVec4Kernel<true, 4>, no progress map
+    run(2);                                                   // AxpyPersistentKernel, no progress map
     CHECK_X(XQueueSetPreemptLevel(xq, kPreemptLevelDeactivate));
-    run(1);                                                   // AxpyVec4Kernel<true, 4> with progress map
+    run(1);                                                   // AxpyPersistentKernel with progress map
     CHECK_X(XQueueDestroy(xq));
     CHECK_X(HwQueueDestroy(hwq));
     printf("traffic_probe: n=%zu reps=%d copy_bytes_read=%zu copy_bytes_written=%zu axpy_algorithmic_bytes=%zu\n",
