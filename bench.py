@@ -171,7 +171,8 @@ def config2(H, a):
                   "commands_in_timed_region": r["bg_cont_cmds"]}
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("axpy_2p28_hbm_traffic.md", bg_n == 1 << 28),
-                        "kernel": "AxpyVec4Kernel", "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
+                        "kernel": "AxpyPersistentKernel<3, false>" if bg_n >= 1 << 23 else "AxpyVec4Kernel<false, 4>",
+                        "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
                         "avg_launch_ms": per_launch_ms}
     if not a.quick:
         ms_plain = bg_ms_per_launch(H, H.AXPY, bg_n, 1, 0)

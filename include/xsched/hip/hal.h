@@ -54,8 +54,9 @@ XResult HipQueueMarkEpochFlushed(HwQueueHandle hwq);
  *              that was not yet its default).
  * A guarded AXPY runs as two long-lived waves per CU that look at the preempt word in front
  * of every chunk: after a deactivation the device drains in microseconds, at the bandwidth
- * of the plain kernel. XSCHED_HIP_AXPY_GRID=chunk keeps the plain kernel's grid (one wave
- * per chunk, guard at entry) for guarded launches as well: ~180 us of drain. */
+ * of the plain kernel (which uses the same grid from 2^23 elements on). With
+ * XSCHED_HIP_AXPY_GRID=chunk every AXPY runs as one short-lived wave per chunk, the guard at
+ * its entry: ~180 us of drain. */
 
 /* y[i] = fma(alpha, x[i], y[i]) in place, fp32, i < n. 128-bit loads/stores when
  * x and y are 16-byte aligned. */

@@ -86,7 +86,7 @@ int main(int argc, char **argv)
         }
         CHECK_X(XQueueWaitAll(xq));
     };
-    run(0);                                                   // AxpyVec4Kernel<false, 4>
+    run(0);                                                   // plain: AxpyPersistentKernel<3, false> from 2^23 elements on
     run(2);                                                   // AxpyPersistentKernel, no progress map
     CHECK_X(XQueueSetPreemptLevel(xq, kPreemptLevelDeactivate));
     run(1);                                                   // AxpyPersistentKernel with progress map

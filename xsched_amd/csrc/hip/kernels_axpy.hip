@@ -9,19 +9,22 @@
 // progress map after its last store.
 //
 // Two grids:
-//   plain launches: one single-wave work-group per chunk. Short-lived waves stream at
-//       6.2-6.3 TB/s on MI355X and let a concurrent kernel find free wave slots within
-//       microseconds.
-//   guarded launches: two long-lived waves per CU, each walking chunks c, c + G,
-//       c + 2G, ... with the loads of three steps in flight, and reading the preempt word
-//       in front of every chunk. Same bandwidth as the plain grid (measured: 2 waves per CU
-//       6.2 TB/s, 1 per CU 4.1, 4 or more per CU 5.3-5.8 whatever the depth). After a
-//       deactivation every wave stops at its next chunk, about a microsecond away, and a
-//       launch queued behind has only G work-groups to retire: the device drains in 6 us
-//       (p50). With XSCHED_HIP_AXPY_GRID=chunk a guarded launch keeps the plain grid, with
-//       the guard at work-group entry: after a deactivation the device then still has to
-//       start and retire every remaining work-group, empty, at ~3.3 waves per nanosecond:
-//       two launches of 262144 work-groups in flight drain in ~180 us.
+//   one single-wave work-group per chunk: plain launches of arrays below 2^23 elements.
+//       Every chunk is in flight at once, which is what a short array wants; on long
+//       arrays these short-lived waves stream at 6.2-6.3 TB/s on MI355X.
+//   two long-lived waves per CU, each walking chunks c, c + G, c + 2G, ... with the loads
+//       of three steps in flight: guarded launches, and plain launches of long arrays.
+//       Same bandwidth (measured: 2 waves per CU 6.2 TB/s, 1 per CU 4.1, 4 or more per CU
+//       5.3-5.8 whatever the depth), and nearly all wave slots stay free: a short kernel of
+//       another queue that arrives meanwhile finishes ~10 us earlier than beside a grid of
+//       262144 work-groups. A guarded launch reads the preempt word in front of every chunk:
+//       after a deactivation every wave stops at its next chunk, about a microsecond away,
+//       and a launch queued behind has only G work-groups to retire: the device drains in
+//       6 us (p50).
+//   XSCHED_HIP_AXPY_GRID=chunk keeps the first grid for everything, with the guard at
+//       work-group entry: after a deactivation the device then still has to start and retire
+//       every remaining work-group, empty, at ~3.3 waves per nanosecond: two launches of
+//       262144 work-groups in flight drain in ~180 us.
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 #include "xsched/utils/env.h"
@@ -109,7 +112,7 @@ void AxpyVec4Kernel(float alpha, const float4 *x, float4 *y,
 // way and step j+kDepth is requested right behind the stores. The preempt word is read
 // in front of the first store of every chunk; a chunk that has begun is finished and
 // committed, so it is applied exactly once.
-template <uint32_t kDepth>
+template <uint32_t kDepth, bool kGuard>
 __global__ __launch_bounds__(64)
 void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, uint32_t tail,
                           uint32_t steps, uint32_t n_chunks, XGuardArgs g)
@@ -118,9 +121,9 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
     constexpr uint32_t kStepVecs = kLanes * kVecPerStep;
     const uint32_t lane = threadIdx.x;
     const uint32_t stride = gridDim.x;
-    const uint32_t *flag = xguard_flag_copy(g, blockIdx.x);
+    const uint32_t *flag = kGuard ? xguard_flag_copy(g, blockIdx.x) : nullptr;
     // an earlier launch of this epoch was flushed: this one must not run ahead of its replay
-    if (xguard_epoch_flushed(g)) return;
+    if (kGuard && xguard_epoch_flushed(g)) return;
 
     // Ring slot d holds step ring_s[d] of chunk ring_c[d]; the slots follow each other in
     // the wave's sequence of steps.
@@ -159,11 +162,13 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
             if (st == 0) {
                 // The scalar read of the preempt word waits for itself only: the vector loads
                 // stay in flight across it. A flushed wave drops what it has loaded.
-                if (xguard_read_flag(flag) != g.epoch) {
-                    if (lane == 0) xguard_note_flush(g);
-                    return;
+                if (kGuard) {
+                    if (xguard_read_flag(flag) != g.epoch) {
+                        if (lane == 0) xguard_note_flush(g);
+                        return;
+                    }
+                    skip = g.resume && g.done && xguard_committed(g, c);
                 }
-                skip = g.resume && g.done && xguard_committed(g, c);
                 if (!skip && !full) {
                     // the last chunk of an array that does not fill it, and the 0..3 scalars behind
                     const uint64_t chunk_base = (uint64_t)c * steps * kStepVecs;
@@ -176,7 +181,7 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
                         float *ys = (float *)(y + n4);
                         ys[lane] = __builtin_fmaf(alpha, xs[lane], ys[lane]);
                     }
-                    if (g.done && lane == 0) xguard_commit(g, c);
+                    if (kGuard && g.done && lane == 0) xguard_commit(g, c);
                 }
             }
             if (full && !skip) {
@@ -185,7 +190,7 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
                 for (uint32_t u = 0; u < kVecPerStep; ++u) {
                     st_nt(&y[base + u * kLanes], fma4(alpha, xv[d][u], yv[d][u]));
                 }
-                if (st == steps - 1 && g.done && lane == 0) xguard_commit(g, c);
+                if (kGuard && st == steps - 1 && g.done && lane == 0) xguard_commit(g, c);
             }
             // this slot's next step: kDepth steps further on in the sequence
             uint32_t nc = c, ns = st + kDepth;
@@ -238,10 +243,15 @@ protected:
         if (n_ == 0) return hipSuccess;
         const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
         const dim3 grid(n_wg_), block(kLanes);
+        const uint32_t waves = PersistentWaves();
         if (aligned && guarded && !chunk_grid_) {
-            const uint32_t waves = PersistentWaves();
             const dim3 pgrid(n_wg_ < waves ? n_wg_ : waves);
-            hipLaunchKernelGGL(AxpyPersistentKernel<3>, pgrid, block, 0, stream, alpha_, (const float4 *)x_,
+            hipLaunchKernelGGL((AxpyPersistentKernel<3, true>), pgrid, block, 0, stream, alpha_, (const float4 *)x_,
+                               (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
+        } else if (aligned && !guarded && !chunk_grid_ && n_wg_ >= 16 * waves) {
+            // A long array: the same few long-lived waves stream it as fast as one wave per
+            // chunk does and leave nearly all wave slots to whatever else runs on the device.
+            hipLaunchKernelGGL((AxpyPersistentKernel<3, false>), dim3(waves), block, 0, stream, alpha_, (const float4 *)x_,
                                (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
         } else if (aligned) {
             const uint64_t n4 = n_ / 4;
