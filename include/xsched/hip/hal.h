@@ -64,8 +64,11 @@ XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, v
                              size_t n, int guard);
 
 /* C[M,N] = A[M,K] * B[K,N]; A, B, C row-major bf16, fp32 accumulation in ascending
- * k, round-to-nearest-even on store. M, N multiples of 256 and K a multiple of 64
- * use the 256x256-tile MFMA kernel; other shapes are refused (InvalidValue). */
+ * k, round-to-nearest-even on store. M, N multiples of 128 and K a multiple of 64; other
+ * shapes are refused (InvalidValue). The MFMA kernel works on 256x256 tiles of C, or on
+ * 128x128 tiles when M or N is no multiple of 256 or the large tiles would cover at most half
+ * of the compute units (XSCHED_HIP_GEMM_TILE=128|256 overrides that); every element is
+ * summed in the same order either way. */
 XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void *B, void *C,
                                  int M, int N, int K, int guard);
 

@@ -261,9 +261,18 @@ def _gemm_case(xs, torch, a_bits, b_bits, M, N, K, level, guard):
     return got
 
 
+@pytest.fixture(params=[128, 256])
+def gemm_tile(request, monkeypatch):
+    """The GEMM works on 256x256 tiles of C, or on 128x128 tiles when the large ones would not
+    fill the device (every shape of these tests) or do not fit the shape. The variable forces
+    one of them where the shape allows both."""
+    monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(request.param))
+    return request.param
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 512, 128), (512, 256, 192)])
 @pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
-def test_gemm_exact_on_small_integers(xs, gpu, M, N, K, level, guard):
+def test_gemm_exact_on_small_integers(xs, gpu, gemm_tile, M, N, K, level, guard):
     """Inputs are integers in [-4, 4]: every product and partial sum is an integer below
     2^24, so fp32 accumulation is exact in any order and the bf16 result is determined;
     any indexing or layout mistake changes it."""
@@ -279,7 +288,35 @@ def test_gemm_exact_on_small_integers(xs, gpu, M, N, K, level, guard):
     assert np.array_equal(got, want)
 
 
-def test_gemm_rounding_to_bf16_is_the_oracles(xs, gpu):
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (384, 128, 128), (128, 640, 192), (896, 384, 64)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_gemm_shapes_that_only_small_tiles_fit(xs, gpu, M, N, K, level, guard):
+    """M or N a multiple of 128 but not of 256; integers as above, so the result is determined."""
+    print(f"case gemm-int-small M={M} N={N} K={K} level={level} guard={guard}", flush=True)
+    rng = np.random.default_rng(8)
+    a_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b_i = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    a_bits, b_bits = oracle.f32_to_bf16_bits(a_i), oracle.f32_to_bf16_bits(b_i)
+    got = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, level, guard)
+    want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K)
+    assert np.array_equal(got, want)
+
+
+def test_gemm_both_tile_sizes_give_the_same_bits(xs, gpu, monkeypatch):
+    """Seeded normal inputs, where the order of the fp32 additions shows in the last bits:
+    both tile sizes feed every element's products to the matrix cores in the same order."""
+    M, N, K = 512, 768, 1024
+    print(f"case gemm-tiles M={M} N={N} K={K}", flush=True)
+    a_bits = oracle.fill_normal_bf16(17, 1, 0, M * K)
+    b_bits = oracle.fill_normal_bf16(17, 2, 0, K * N)
+    out = {}
+    for tile in (128, 256):
+        monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
+        out[tile] = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, 2, 1)
+    assert np.array_equal(out[128], out[256])
+
+
+def test_gemm_rounding_to_bf16_is_the_oracles(xs, gpu, gemm_tile):
     """Every C[i][j] here is ONE product a_i * b_j (the other 63 terms of the sum are 0 * 0),
     so the fp32 accumulator holds it exactly and the stored bf16 shows the rounding alone:
     ties to even, carries into the exponent, overflow to infinity, denormal results,
@@ -319,7 +356,7 @@ def test_gemm_rounding_to_bf16_is_the_oracles(xs, gpu):
     assert np.count_nonzero(~nan_want) > 60000
 
 
-def test_gemm_normal_inputs_within_tolerance(xs, gpu):
+def test_gemm_normal_inputs_within_tolerance(xs, gpu, gemm_tile):
     """Seeded N(0,1)-like inputs: the MFMA's internal summation order is not the
     oracle's, so the comparison is on values. Tolerance: one bf16 unit in the last
     place of the result (2^-8 relative) plus fp32 accumulation noise 2^-20*sqrt(K)."""

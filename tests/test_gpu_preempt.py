@@ -106,8 +106,10 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     assert np.array_equal(got.astype(np.uint64), one * times)
 
 
-def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu):
+@pytest.mark.parametrize("tile", [128, 256])
+def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile):
     torch = gpu
+    monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
     M = N = K = 2048
     times = 12
     print(f"case gemm-preempt {M}^3 times={times}", flush=True)

@@ -39,14 +39,13 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTile = 256;          // tile edge (M and N)
+constexpr int kLargeTile = 256;     // edge of the large tile of C (M and N)
+constexpr int kSmallTile = 128;     // edge of the small one
 constexpr int kStepK = 64;          // K per step
 constexpr int kLdsStride = 72;      // bf16 per row of the A tile in LDS (64 + 8 padding)
-constexpr int kBStride = 272;       // bf16 per row of the B tile in LDS (256 + 16): four consecutive rows start in four different 32-byte bank groups
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4 LdsS16x4;
-constexpr int kThreads = 512;
 constexpr int kPollSteps = 8;       // K steps between two looks at the preempt word
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 4;       // tile rows walked together
@@ -88,11 +87,23 @@ __device__ __forceinline__ void TileOf(uint32_t wg, uint32_t tiles_m, uint32_t t
 // t % 2, the registers holding tile t + 1 are written to the other buffer and the global
 // loads of tile t + 2 are issued; the fragments of the next 16-wide k slice are read from
 // LDS before the MFMAs of the current slice are issued.
-template <bool kGuard>
-__global__ __launch_bounds__(kThreads)
+//
+// kTile x kTile is the tile of C, kWavesM x kWavesN the wave grid over it; a wave owns
+// kBlocksM x kBlocksN blocks of 32x32. Two shapes are built: 256 with 2x4 waves (4x2 blocks
+// per wave), and 128 with 2x2 waves (2x2 blocks) for outputs of too few large tiles to fill
+// the device. Every element is summed in the same order in both.
+template <bool kGuard, int kTile, int kWavesM, int kWavesN>
+__global__ __launch_bounds__(64 * kWavesM * kWavesN)
 void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                              uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
 {
+    constexpr int kThreads = 64 * kWavesM * kWavesN;
+    constexpr int kBlocksM = kTile / (32 * kWavesM);
+    constexpr int kBlocksN = kTile / (32 * kWavesN);
+    constexpr int kBStride = kTile + 16;               // bf16 per row of the B tile in LDS: four consecutive rows start in four different 32-byte bank groups
+    constexpr int kAChunks = kTile * (kStepK / 8) / kThreads; // 16-byte pieces of the A tile per thread
+    constexpr int kBChunks = kStepK * (kTile / 8) / kThreads; // and of the B tile
+    static_assert(kBlocksN == 2, "the transposing B reads below cover two 32-column blocks per wave");
     __shared__ __attribute__((aligned(16))) uint16_t As[2][kTile * kLdsStride];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kStepK * kBStride];
     __shared__ uint32_t guard_word;
@@ -100,52 +111,52 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
-    const uint32_t wm = wave >> 2;
-    const uint32_t wn = wave & 3;
+    const uint32_t wm = wave / kWavesN;
+    const uint32_t wn = wave % kWavesN;
 
     uint32_t tm, tn;
     TileOf(blockIdx.x, (uint32_t)M / kTile, (uint32_t)N / kTile, tm, tn);
     const size_t m0 = (size_t)tm * kTile, n0 = (size_t)tn * kTile;
 
-    u32x4 a_reg[4];
-    u32x4 b_vec[4];
+    u32x4 a_reg[kAChunks];
+    u32x4 b_vec[kBChunks];
 
     auto load_global = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kAChunks; ++i) {
             const uint32_t c = tid + kThreads * i;
             const uint32_t row = c >> 3, kc = c & 7;
             a_reg[i] = *(const u32x4 *)(A + (m0 + row) * (size_t)K + k0 + kc * 8);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kBChunks; ++i) {
             const uint32_t c = tid + kThreads * i;
-            const uint32_t krow = c >> 5, chunk = c & 31;
+            const uint32_t krow = c / (kTile / 8), chunk = c % (kTile / 8);
             b_vec[i] = *(const u32x4 *)(B + (size_t)(k0 + krow) * N + n0 + chunk * 8);
         }
     };
 
     auto store_lds = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kAChunks; ++i) {
             const uint32_t c = tid + kThreads * i;
             const uint32_t row = c >> 3, kc = c & 7;
             *(u32x4 *)(As[buf] + row * kLdsStride + kc * 8) = a_reg[i];
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kBChunks; ++i) {
             const uint32_t c = tid + kThreads * i;
-            const uint32_t krow = c >> 5, chunk = c & 31;
+            const uint32_t krow = c / (kTile / 8), chunk = c % (kTile / 8);
             *(u32x4 *)(Bs[buf] + krow * kBStride + chunk * 8) = b_vec[i];
         }
     };
 
-    const uint32_t a_row0 = 128 * wm + (lane & 31);
+    const uint32_t a_row0 = 32 * kBlocksM * wm + (lane & 31);
     const uint32_t khalf = 8 * (lane >> 5);
     auto load_a_frags = [&](int buf, int ks, bf16x8 *fa) {
         const uint32_t koff = ks * 16 + khalf;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa[i] = *(const bf16x8 *)(As[buf] + (a_row0 + 32 * i) * kLdsStride + koff);
+        for (int i = 0; i < kBlocksM; ++i) fa[i] = *(const bf16x8 *)(As[buf] + (a_row0 + 32 * i) * kLdsStride + koff);
     };
     // B sits in LDS as it sits in memory, [k][n]. The transposing read hands lane l of every 16
     // lanes the element (l & 3) of what lanes 4 * j + (l >> 2), j = 0..3, of the same 16 point
@@ -168,11 +179,11 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         load_b_frags(buf, ks, fb);
     };
 
-    f32x16 acc[4][2];
+    f32x16 acc[kBlocksM][kBlocksN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBlocksM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < kBlocksN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -197,14 +208,14 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     //   slice 3: fragment reads of slice 0 of the NEXT tile from the other buffer
     // Both fragment sets are double-buffered in registers (40 of them): the reads of slice
     // s + 1 are issued before the MFMAs of slice s.
-    bf16x8 fa[2][4], fb[2][2];
+    bf16x8 fa[2][kBlocksM], fb[2][kBlocksN];
     load_frags(0, 0, fa[0], fb[0]);
 
     auto mfma_slice = [&](int set) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < kBlocksM; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < kBlocksN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
@@ -238,13 +249,13 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     }
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kBlocksM; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < kBlocksN; ++j) {
             const size_t col = n0 + 64 * wn + 32 * j + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const size_t row = m0 + 128 * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const size_t row = m0 + 32 * kBlocksM * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 C[row * (size_t)N + col] = f32_to_bf16_rne(acc[i][j][r]);
             }
         }
@@ -260,16 +271,23 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
 class HipGemmCommand final : public HipGuardedCommand
 {
 public:
-    HipGemmCommand(const void *A, const void *B, void *C, int M, int N, int K, int guard_mode)
-        : HipGuardedCommand((uint32_t)(M / kTile) * (uint32_t)(N / kTile), guard_mode)
-        , A_((const uint16_t *)A), B_((const uint16_t *)B), C_((uint16_t *)C), M_(M), N_(N), K_(K) {}
+    HipGemmCommand(const void *A, const void *B, void *C, int M, int N, int K, int tile, int guard_mode)
+        : HipGuardedCommand((uint32_t)(M / tile) * (uint32_t)(N / tile), guard_mode)
+        , A_((const uint16_t *)A), B_((const uint16_t *)B), C_((uint16_t *)C), M_(M), N_(N), K_(K), tile_(tile) {}
 
 protected:
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
     {
-        const dim3 grid(n_wg_), block(kThreads);
-        if (guarded) hipLaunchKernelGGL(GemmBf16Kernel<true>, grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
-        else         hipLaunchKernelGGL(GemmBf16Kernel<false>, grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+        const dim3 grid(n_wg_);
+        if (tile_ == kLargeTile) {
+            const dim3 block(512);
+            if (guarded) hipLaunchKernelGGL((GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+            else         hipLaunchKernelGGL((GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+        } else {
+            const dim3 block(256);
+            if (guarded) hipLaunchKernelGGL((GemmBf16Kernel<true, kSmallTile, 2, 2>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+            else         hipLaunchKernelGGL((GemmBf16Kernel<false, kSmallTile, 2, 2>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+        }
         return hipGetLastError();
     }
 
@@ -277,7 +295,28 @@ private:
     const uint16_t *A_, *B_;
     uint16_t *C_;
     const int M_, N_, K_;
+    const int tile_;
 };
+
+/// The tile edge for an M x N output: large tiles do more arithmetic per byte read from LDS,
+/// but each one keeps a single compute unit busy, so an output of few large tiles leaves most
+/// of the device idle. Small tiles when the large ones would cover at most half of the compute
+/// units, or when M or N is no multiple of the large edge. XSCHED_HIP_GEMM_TILE=128|256
+/// overrides the choice where the shape allows.
+inline int TileFor(int M, int N)
+{
+    const bool large_fits = M % kLargeTile == 0 && N % kLargeTile == 0;
+    if (!large_fits) return kSmallTile;
+    int64_t forced = 0;
+    if (GetEnvInt64("XSCHED_HIP_GEMM_TILE", forced) && (forced == kSmallTile || forced == kLargeTile)) return (int)forced;
+    static const int cus = []() {
+        int dev = 0, n = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        return n > 0 ? n : 256;
+    }();
+    const int64_t large_tiles = (int64_t)(M / kLargeTile) * (N / kLargeTile);
+    return large_tiles * 2 <= cus ? kSmallTile : kLargeTile;
+}
 
 } // namespace gemm
 
@@ -291,15 +330,16 @@ EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void 
     if (cmd == nullptr || A == nullptr || B == nullptr || C == nullptr || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
-    if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kTile || N % gemm::kTile || K % gemm::kStepK) {
-        XWARN("HipGemmBf16CommandCreate: M and N must be multiples of 256 and K of 64 (got %d %d %d)", M, N, K);
+    if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kSmallTile || N % gemm::kSmallTile || K % gemm::kStepK) {
+        XWARN("HipGemmBf16CommandCreate: M and N must be multiples of 128 and K of 64 (got %d %d %d)", M, N, K);
         return kXSchedErrorInvalidValue;
     }
+    const int tile = gemm::TileFor(M, N);
     if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) return kXSchedErrorInvalidValue;
     // one progress-map byte per tile
-    if ((uint64_t)(M / gemm::kTile) * (uint64_t)(N / gemm::kTile) > GuardState::kMaxWorkGroups) {
+    if ((uint64_t)(M / tile) * (uint64_t)(N / tile) > GuardState::kMaxWorkGroups) {
         return kXSchedErrorInvalidValue;
     }
-    *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, guard));
+    *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, tile, guard));
     return kXSchedSuccess;
 }
