@@ -557,29 +557,36 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
         acc[0] += w.x & 0xFFFFu; acc[1] += w.y & 0xFFFFu; acc[2] += w.z & 0xFFFFu; acc[3] += w.w & 0xFFFFu;
         acc[4] += w.x >> 16;     acc[5] += w.y >> 16;     acc[6] += w.z >> 16;     acc[7] += w.w >> 16;
     };
-    // The first eight rows are requested before the guard's uncached read of the preempt
-    // word: the kernel is short, and the round trips overlap. Reading has no side effect
-    // (after a flushed counting launch the words are stale, and nothing is done with them).
+    // The first eight rows are requested before the guard's reads: the kernel is short, and
+    // the round trips overlap. Reading has no side effect (after a flushed counting launch
+    // the words are stale, and nothing is done with them).
     u32x4 first[8];
 #pragma unroll
     for (uint32_t i = 0; i < 8; ++i) first[i] = load_words(row + i * kRows);
 
     if (kGuard) {
-        // A flushed counting launch leaves partials missing; then this launch is flushed
-        // too (the preempt word only ever counts up), but make sure: every counting group
-        // must have committed. Their progress bytes are requested ahead of the guard too.
+        // A flushed counting launch leaves partials missing: every counting group must have
+        // committed. Their progress bytes are requested ahead of the other reads.
         uint8_t tag[kMaxPartials / kThreads];
 #pragma unroll
         for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) {
             const uint32_t p = tid + i * kThreads;
             tag[i] = g.done != nullptr && p < n_part ? __builtin_nontemporal_load(&g.done[p]) : (uint8_t)g.gen;
         }
-        XGuardBlock guard(g, first_wg + blockIdx.x, &guard_word);
-        if (!guard.Enter()) return;
+        // This kernel does not look at the preempt word itself: it runs for a few
+        // microseconds, and what it must not do is run after a counting launch that was
+        // flushed. Every flushed group has left its epoch in the `flushed` word, and the tags
+        // say whether every partial is there; its own tag says whether it ran before the flush.
+        if (tid == 0) {
+            bool go = !xguard_epoch_flushed(g);
+            if (go && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) go = false;
+            guard_word = go ? 1u : 0u;
+        }
         int all = 1;
 #pragma unroll
         for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) all &= tag[i] == (uint8_t)g.gen;
-        if (!__syncthreads_and(all)) return;
+        const int complete = __syncthreads_and(all);   // also publishes guard_word
+        if (!complete || guard_word == 0) return;
     }
     if (tid < kHotBins) hot_total[tid] = 0;
 
