@@ -101,6 +101,30 @@ def test_axpy_guarded_grids_and_chunk_sizes(xs, gpu, monkeypatch, grid, steps, n
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("steps,n", [(1, (1 << 23) + 7), (3, 8192 * 3072 + 1029), (2, 8192 * 2048)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_axpy_long_arrays(xs, gpu, monkeypatch, steps, n, level, guard):
+    """From 8192 chunks on a plain launch runs on the long-lived waves as well (shorter arrays
+    use one wave per chunk): lengths just past that border, with one and several steps per
+    chunk, a ragged end and an exact fit."""
+    torch = gpu
+    monkeypatch.setenv("XSCHED_HIP_AXPY_STEPS", str(steps))
+    print(f"case axpy-long n={n} steps={steps} level={level} guard={guard}", flush=True)
+    x_h = oracle.fill_uniform(23, 1, 0, n)
+    y_h = oracle.fill_uniform(23, 2, 0, n)
+    x = torch.from_numpy(x_h).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, level)
+    for _ in range(2):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, guard))
+    q.wait()
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    q.close()
+    want = oracle.axpy(0.5, x_h, y_h, 2)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_axpy_general_alpha_and_unaligned(xs, gpu):
     """alpha whose product is inexact (one rounding: fma) and a pointer that is only
     4-byte aligned (scalar fallback kernel)."""
