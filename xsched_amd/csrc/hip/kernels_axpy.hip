@@ -153,7 +153,8 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
 
     bool skip = false;   // the chunk whose steps are passing by was committed before the flush
     while (true) {
-#pragma unroll
+        // no unroll pragma here: the constant trip count is unrolled anyway, and with the
+        // pragma the compiler warns about a copy of the loop that it drops afterwards
         for (uint32_t d = 0; d < kDepth; ++d) {
             const uint32_t c = ring_c[d];
             const uint32_t st = ring_s[d];
