@@ -326,6 +326,25 @@ def test_gemm_shapes_that_only_small_tiles_fit(xs, gpu, M, N, K, level, guard):
     assert np.array_equal(got, want)
 
 
+def test_gemm_seeded_random_shapes(xs, gpu, monkeypatch):
+    """Ten seeded shapes (M, N multiples of 128 up to 1152, K multiples of 64 up to 448), each
+    with the tile sizes its shape allows; integer inputs, so every result is determined."""
+    rng = np.random.default_rng(2024)
+    for case in range(10):
+        M, N = (int(v) * 128 for v in rng.integers(1, 10, 2))
+        K = int(rng.integers(1, 8)) * 64
+        a_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+        b_i = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        a_bits, b_bits = oracle.f32_to_bf16_bits(a_i), oracle.f32_to_bf16_bits(b_i)
+        want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K)
+        tiles = (128, 256) if M % 256 == 0 and N % 256 == 0 else (128,)
+        for tile in tiles:
+            print(f"case gemm-random {case}: M={M} N={N} K={K} tile={tile}", flush=True)
+            monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
+            got = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, 2, 1)
+            assert np.array_equal(got, want), (M, N, K, tile)
+
+
 def test_gemm_both_tile_sizes_give_the_same_bits(xs, gpu, monkeypatch):
     """Seeded normal inputs, where the order of the fp32 additions shows in the last bits:
     both tile sizes feed every element's products to the matrix cores in the same order."""
