@@ -221,19 +221,25 @@ def config3(H, a):
                         "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": recorded_traffic("gemm_8192_hbm_traffic.md"), "kernel": "GemmBf16Kernel",
                         "algorithmic_flops_per_launch": gemm_flops(bg_n), "avg_launch_ms": per_launch_ms}
     if not a.quick:
-        # Three alternating rounds, the median of each form: the clock under this load moves
-        # by a few percent within seconds, more than the guard costs.
-        rounds = [(bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 20, 4), bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 20, 4),
-                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 20, 4)) for _ in range(3)]
-        ms_plain, ms_guard, ms_l2 = (sorted(r[i] for r in rounds)[1] for i in range(3))
+        # Seven alternating rounds of 12 launches per form. The clock under this load moves by a
+        # few percent within seconds, more than the guard costs: the overheads are medians of
+        # the per-round ratios (forms measured within a second of each other), the rates are
+        # medians of each form.
+        rounds = [(bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 12, 4), bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 12, 4),
+                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 12, 4)) for _ in range(7)]
+        ms_plain, ms_guard, ms_l2 = (sorted(r[i] for r in rounds)[3] for i in range(3))
+        guard_frac = sorted(1.0 - r[0] / r[1] for r in rounds)
+        l2_frac = sorted(1.0 - r[0] / r[2] for r in rounds)
 
         def tf(ms):
             return gemm_flops(bg_n) / ms / 1e9
         line["guard"] = {"plain_TFLOPs": tf(ms_plain), "guarded_TFLOPs": tf(ms_guard), "level2_TFLOPs": tf(ms_l2),
                          "plain_mfma_util": tf(ms_plain) / MFMA_BF16_PEAK_TF,
                          "guarded_mfma_util": tf(ms_guard) / MFMA_BF16_PEAK_TF,
-                         "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
-                         "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
+                         "guard_overhead_frac": guard_frac[3], "level2_overhead_frac": l2_frac[3],
+                         "guard_overhead_frac_min_max": [guard_frac[0], guard_frac[-1]],
+                         "level2_overhead_frac_min_max": [l2_frac[0], l2_frac[-1]],
+                         "rounds": len(rounds), "launches_per_round_and_form": 12}
         line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, False)
     return line
 
