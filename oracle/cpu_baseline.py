@@ -1,13 +1,31 @@
 """ORACLE - test infrastructure only: runs the headline workload on CPU cores, on a
 bounded sample, and reports it in bench.py's `cpu_baseline` format. Preferred: the
 reference's own XQueue core, scheduler and policy (oracle/_ref/libxqueue_ref.so, kind
-"reference") driving scalar CPU kernels through oracle/host_bench.cpp; without that build,
-the compact port of the host loop in oracle/xsched_port.cpp (kind "port")."""
+"reference") driving scalar CPU kernels through oracle/host_bench.cpp. Without that build
+there is no CPU baseline: the call raises."""
 import ctypes
 import os
 from ctypes import POINTER, byref, c_double, c_int, c_int64, c_uint64
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
+
+
+def host_cpu():
+    """(model name, logical cores of the machine, cores this process may run on)."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 0
+    return model, os.cpu_count() or 0, usable
 
 
 def _pct(samples, p):
@@ -20,18 +38,18 @@ def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100, which="au
     20 ms at priority 2, level 1, HPF), with both arrays scaled down by 2^scale_log2 so
     that the sample takes on the order of ten seconds of CPU work."""
     ref_path = os.path.join(_DIR, "_ref", "libxqueue_ref.so")
-    path = os.path.join(_DIR, "libxsched_port.so")
     if which == "auto":
-        which = "reference" if os.path.exists(ref_path) else "port"
+        which = "reference"
     if which == "reference":
+        if not os.path.exists(ref_path):
+            raise RuntimeError(f"{ref_path} missing: it is built from the reference sources by "
+                               "`make -C oracle ref` where that tree is present")
         os.environ.setdefault("XLOG_LEVEL", "ERRO")
         fn = ctypes.CDLL(ref_path, mode=ctypes.RTLD_LOCAL).hostbench_run_fg_bg_axpy
     elif which == "shipped":
         fn = ctypes.CDLL(os.path.join(_DIR, "libhostbench.so"), mode=ctypes.RTLD_LOCAL).hostbench_run_fg_bg_axpy
     else:
-        if not os.path.exists(path):
-            raise RuntimeError(f"{path} missing: run `make -C oracle`")
-        fn = ctypes.CDLL(path).port_run_fg_bg_axpy
+        raise ValueError("which must be auto, reference or shipped")
     fn.restype = c_int
     fn.argtypes = [c_uint64, c_uint64, c_int64, c_int, c_int, c_int, POINTER(c_double), POINTER(c_double),
                    POINTER(c_uint64), POINTER(c_double), POINTER(c_uint64)]
@@ -48,16 +66,16 @@ def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100, which="au
         "value": _pct(cont, 0.99),
         "unit": "us",
         "cores": 7,
-        "kind": "port" if which == "port" else "reference" if which == "reference" else "shipped-host",
+        "host_cpu_model": host_cpu()[0], "host_logical_cores": host_cpu()[1], "host_usable_cores": host_cpu()[2],
+        "kind": "reference" if which == "reference" else "shipped-host",
         "sample": ("%s (2 XQueues, level 1, HPF, bg window 4/2, fg 8/4), scalar single-threaded fmaf AXPY per "
                    "queue; bg 2^%d and fg 2^%d elements (1/%d of the GPU sizes), fg every 20 ms, %d fg samples; "
                    "threads: 2 executors + 2 launch workers + 1 scheduler + 2 submitters"
-                   % ({"port": "oracle/xsched_port.cpp: CPU restatement of XSched's host loop",
-                       "reference": "oracle/_ref/libxqueue_ref.so: XSched's own XQueue core, local scheduler and "
+                   % ({"reference": "oracle/_ref/libxqueue_ref.so: XSched's own XQueue core, local scheduler and "
                                     "HPF policy compiled from the reference sources, driving this repository's "
                                     "host adapter through oracle/host_bench.cpp",
                        "shipped-host": "shipped libpreempt.so + libhalhost.so through oracle/host_bench.cpp"}
-                      ["port" if which == "port" else "reference" if which == "reference" else "shipped-host"],
+                      ["reference" if which == "reference" else "shipped-host"],
                       28 - scale_log2, 22 - scale_log2, 1 << scale_log2, len(cont))),
         "fg_alone_p50_us": _pct(alone, 0.5), "fg_alone_p99_us": _pct(alone, 0.99),
         "fg_contended_p50_us": _pct(cont, 0.5), "fg_contended_p99_us": _pct(cont, 0.99),

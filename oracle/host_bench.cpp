@@ -33,7 +33,11 @@ using Clock = std::chrono::steady_clock;
 #define HB_CHECK(call) do { XResult r_ = (call); if (r_ != kXSchedSuccess) return (int)r_; } while (0)
 } // namespace
 
-// Same meaning of arguments and outputs as port_run_fg_bg_axpy() in xsched_port.cpp.
+// bg_n / fg_n: elements of the background / foreground AXPY; one foreground command every
+// period_us, `samples` of them alone and `samples` beside the background stream; the
+// background window is bg_threshold / bg_batch (foreground 8 / 4). Outputs: the two latency
+// arrays (microseconds), background commands completed and seconds of the contended phase,
+// and a checksum over every 97th element of the foreground result.
 extern "C" __attribute__((visibility("default")))
 int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, int samples,
                              int bg_threshold, int bg_batch, double *alone_us, double *contended_us,

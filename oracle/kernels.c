@@ -3,24 +3,36 @@
  * percentile rule. Nothing in the shipped libraries links or calls this file; it is
  * used by tests/, by the smoke check and by the CPU-baseline leg of bench.py.
  *
- * What pins each function (besides the GPU parity tests it serves):
- *   oracle_vecadd      c = a + b is one IEEE-754 operation per element: any correct
- *                      implementation is bit-identical. Known-answer shape of the
- *                      reference's own test: k chained additions of ones give k
+ * What pins each function (tests/test_oracle_kernels.py, CPU only; the known answers in
+ * tests/golden/kernel_vectors.json were computed by tests/golden/make_kernel_vectors.py
+ * with Python integers, fractions and decimals, not with this file):
+ *   oracle_vecadd      c = a + b is one IEEE-754 operation per element: equal to numpy's
+ *                      addition bit for bit, and the known-answer shape of the reference's
+ *                      own test: k chained additions of ones give k
  *                      (platforms/example/test/src/vecadd.cpp:91-102).
- *   oracle_axpy        y = fma(alpha, x, y): one correctly rounded libm fmaf per
- *                      element. For alpha = 0.5 the product is exact, so it also
- *                      equals multiply-then-add (checked against numpy in tests).
- *   oracle_gemm_bf16   triple loop, ascending k, fmaf accumulation, RNE to bf16.
- *                      Pinned against numpy float64 matmul (tolerance) and, on
- *                      small-integer inputs where every partial sum is exact, bit for
- *                      bit against integer matmul.
- *   oracle_histogram   bins[key]++ ; pinned against numpy.bincount.
+ *   oracle_axpy        y = fma(alpha, x, y): one correctly rounded libm fmaf per element.
+ *                      alpha = 0.5 (product exact): equal to numpy's multiply-then-add bit
+ *                      for bit; five other alphas: equal to the exact rational
+ *                      alpha * x + y rounded once (fixture), on inputs where
+ *                      multiply-then-add gives different bits.
+ *   oracle_gemm_bf16   triple loop, ascending k, fmaf accumulation, RNE to bf16. On
+ *                      small-integer inputs (every partial sum exact) equal to integer
+ *                      matmul; the summation order by a sum whose value depends on it
+ *                      (2^24 + 63 ones); float64 matmul within the fp32 error bound;
+ *                      oracle_f32_to_bf16 against ties, carries and the overflow to
+ *                      infinity decided by exact distances (fixture).
+ *   oracle_histogram   bins[key]++ ; equal to numpy.bincount, keys outside the range
+ *                      ignored, bins not cleared, counters wrap modulo 2^32.
  *   oracle_percentile  sorted[floor(p*n)] - the reference's rule
- *                      (utils/include/xsched/utils/data.h:57-65); pinned by closed-form
- *                      cases in tests.
- *   synthetic inputs   integer hashing + exact int->float conversion; pinned by
- *                      committed first-values fixtures and distribution checks.
+ *                      (utils/include/xsched/utils/data.h:57-65); closed-form cases
+ *                      (n = 1; n = 100, p = 0.99 -> index 99; p * n integral; ties).
+ *   synthetic inputs   SplitMix64 against its published vector (seed 0: E220A8397B1DCDAF,
+ *                      6E789E6AA1B965F4, 06C45D188009454F); stream keys, the first 16
+ *                      uniform and normal values, the first 32 Zipf keys, the Zipf table
+ *                      (60-digit decimals) and bins 0..15 of 2^22 keys against the
+ *                      fixture; the table also against what the distribution fixes
+ *                      (monotone, ends at 2^32 - 1, P(0) = 1 / H(65536, 1.1), increments
+ *                      in the ratio (k + 1)^-1.1, 13.8 % of the keys in bin 0).
  * The reference has no GEMM, histogram or AXPY kernel: these three are new work
  * whose definition is the header include/xsched/hip/hal.h.
  */

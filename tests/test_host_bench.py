@@ -1,8 +1,7 @@
 """The headline workload on CPU cores, through the public C API only (oracle/host_bench.cpp),
-over three host loops: the reference's own XQueue core + local scheduler + HPF policy
-(where that build is present), the shipped core, and the compact port used when the
-reference build is absent. All three must leave bit-identical foreground output: k in-place
-AXPYs of the seeded arrays, checked against the kernel oracle."""
+over two host loops: the reference's own XQueue core + local scheduler + HPF policy
+(where that build is present) and the shipped core. Both must leave bit-identical foreground
+output: k in-place AXPYs of the seeded arrays, checked against the kernel oracle."""
 import ctypes
 import os
 from ctypes import POINTER, byref, c_double, c_int, c_int64, c_uint64
@@ -16,7 +15,6 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIBS = {
     "reference": (os.path.join(ROOT, "oracle", "_ref", "libxqueue_ref.so"), "hostbench_run_fg_bg_axpy"),
     "shipped": (os.path.join(ROOT, "oracle", "libhostbench.so"), "hostbench_run_fg_bg_axpy"),
-    "port": (os.path.join(ROOT, "oracle", "libxsched_port.so"), "port_run_fg_bg_axpy"),
 }
 FG_N, BG_N, SAMPLES = 1 << 12, 1 << 16, 20
 
@@ -28,7 +26,7 @@ def expected_checksum():
     return int(y[::97].view(np.uint32).astype(np.uint64).sum())
 
 
-@pytest.mark.parametrize("which", ["reference", "shipped", "port"])
+@pytest.mark.parametrize("which", ["reference", "shipped"])
 def test_host_loops_agree_bit_for_bit(which):
     path, sym = LIBS[which]
     if not os.path.exists(path):
