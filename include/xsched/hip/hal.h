@@ -77,6 +77,23 @@ XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void
 XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t n, void *bins,
                                   uint32_t n_bins, int guard);
 
+/* The same histogram (bins[keys[i]] += 1, bins not cleared) enqueued on `stream` (a
+ * hipStream_t; NULL = the default stream) directly, as two plain kernel launches, by an entry
+ * point that allocates nothing: no hipMalloc / hipFree, no pool, no XQueue, no command object.
+ * No counterpart in the reference. It is for callers that cannot allocate device memory where
+ * they call it: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation. The partial histograms that HipHistogramCommandCreate keeps in a buffer of its
+ * queue's pool live in a static device array of 16.03 MiB (128 partials) instead, which every
+ * GPU the library has run this call on holds until the process ends. Limits and rules:
+ *   - n <= 2^25 keys (InvalidValue and a warning above that); n_bins <= 65536;
+ *   - every call on one GPU uses that GPU's one array: calls whose kernels can overlap on a
+ *     GPU (different streams, no ordering between them) race; calls on one stream do not;
+ *   - nothing of the array has to be zero: each launch overwrites all it reads;
+ *   - the launches are not flushable (no guard): level-2 preemption does not apply.
+ * Returns after enqueueing; the caller synchronises the stream. */
+XResult HipHistogramLaunchNoAlloc(void *stream, const void *keys, size_t n, void *bins,
+                                  uint32_t n_bins);
+
 /* A kernel of the caller's own that has the guard of xsched/hip/guard.h compiled in (see the
  * head of that file for the three lines). The kernel's LAST parameter must be an XGuardArgs:
  * `args` / `arg_sizes` describe the parameters in front of it (copied at creation), the guard

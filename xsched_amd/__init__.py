@@ -103,6 +103,7 @@ HALHIP_API = {
                                            c_int, c_int, c_int, c_int]),
     "HipHistogramCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_size_t, c_void_p,
                                             c_uint32, c_int]),
+    "HipHistogramLaunchNoAlloc": (XResult, [c_void_p, c_void_p, c_size_t, c_void_p, c_uint32]),
     "HipMemcpyCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_void_p, c_size_t, c_int]),
     "HipMemsetCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_int, c_size_t]),
     "HipMemsetWideCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_uint32, c_size_t, c_uint32]),

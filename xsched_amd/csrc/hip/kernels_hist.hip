@@ -706,6 +706,99 @@ inline uint64_t MergeMinKeys()
 
 using namespace xsched::hip;
 
+// ---- the entry point that allocates nothing -------------------------------------------
+//
+// The partial histograms of HipHistogramLaunchNoAlloc() live in this array instead of a
+// buffer from a queue's pool. Every GPU the library runs on holds its own copy at its own
+// address for the life of the process; in host code the array's NAME is only a handle for
+// hipGetSymbolAddress(), never a device pointer.
+namespace
+{
+constexpr uint32_t kNoAllocMaxGroups = 128;                       // counting work-groups
+constexpr uint64_t kNoAllocMaxKeys = (uint64_t)kNoAllocMaxGroups * hist::kMaxChunk; // 2^25
+constexpr size_t kNoAllocScratchWords = (size_t)kNoAllocMaxGroups * hist::kPartialWords;
+
+static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];          // 16.03 MiB
+
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_scratch_mtx;
+uint32_t *g_scratch_ptr[kNoAllocMaxDevices] = {};
+
+/// Device address of `scratch` on `device`, which must be the calling thread's current device.
+/// Looked up once per device; nullptr (and a warning) if the runtime refuses.
+uint32_t *ScratchOnCurrentDevice(int device)
+{
+    std::lock_guard<std::mutex> lock(g_scratch_mtx);
+    if (g_scratch_ptr[device] != nullptr) return g_scratch_ptr[device];
+    uint32_t *ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+        XWARN("hipGetSymbolAddress(scratch) on device %d failed: %d (%s)", device, (int)err, hipGetErrorString(err));
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+    return ptr;
+}
+} // namespace
+
+EXPORT_C_FUNC XResult HipHistogramLaunchNoAlloc(void *stream_ptr, const void *keys, size_t n, void *bins,
+                                                uint32_t n_bins)
+{
+    if (bins == nullptr || (n != 0 && keys == nullptr)) return kXSchedErrorInvalidValue;
+    if (n_bins == 0 || n_bins > 65536) return kXSchedErrorInvalidValue;
+    if (n > kNoAllocMaxKeys) {
+        XWARN("HipHistogramLaunchNoAlloc: %zu keys exceed the limit of %llu keys that the static "
+              "scratch array holds partial histograms for", n, (unsigned long long)kNoAllocMaxKeys);
+        return kXSchedErrorInvalidValue;
+    }
+    if (n == 0) return kXSchedSuccess;
+
+    hipStream_t stream = (hipStream_t)stream_ptr;
+    int device = -1, current = -1;
+    if (hipGetDevice(&current) != hipSuccess) return kXSchedErrorHardware;
+    if (stream == nullptr) device = current;
+    else if (hipStreamGetDevice(stream, &device) != hipSuccess) { (void)hipGetLastError(); return kXSchedErrorInvalidValue; }
+    if (device < 0 || device >= kNoAllocMaxDevices) return kXSchedErrorNotSupported;
+    // Symbol lookup and launch both act on the current device: it has to be the stream's.
+    if (device != current && hipSetDevice(device) != hipSuccess) return kXSchedErrorHardware;
+
+    XResult res = kXSchedSuccess;
+    uint32_t *partials = ScratchOnCurrentDevice(device);
+    if (partials == nullptr) {
+        res = kXSchedErrorHardware;
+    } else {
+        // As few groups as the limit allows, each with a whole number of load units; every
+        // group stores its complete partial (all-zero after an overflow recount), so nothing
+        // of an earlier call's contents is read and nothing has to be cleared.
+        uint32_t chunk = hist::ChunkFor(n, hist::kMergeMinChunk);
+        uint64_t n_wg = (n + chunk - 1) / chunk;
+        if (n_wg > kNoAllocMaxGroups) {
+            const uint64_t per = (n + kNoAllocMaxGroups - 1) / kNoAllocMaxGroups;
+            chunk = (uint32_t)((per + hist::kMinChunk - 1) / hist::kMinChunk * hist::kMinChunk);
+            n_wg = (n + chunk - 1) / chunk;
+        }
+        XASSERT(n_wg <= kNoAllocMaxGroups && chunk <= hist::kMaxChunk, "group count %llu / chunk %u out of range",
+                (unsigned long long)n_wg, chunk);
+        const XGuardArgs inert {};
+        const dim3 block(hist::kThreads);
+        hipLaunchKernelGGL((hist::HistogramKernel<false, true>), dim3((uint32_t)n_wg), block, 0, stream,
+                           (const int32_t *)keys, (uint64_t)n, (uint32_t *)bins, n_bins, chunk, partials, inert);
+        hipError_t err = hipGetLastError();
+        if (err == hipSuccess) {
+            hipLaunchKernelGGL(hist::HistogramMergeKernel<false>, dim3(hist::kMergeGroups), block, 0, stream,
+                               (const uint32_t *)partials, (uint32_t)n_wg, (uint32_t *)bins, n_bins, (uint32_t)n_wg, inert);
+            err = hipGetLastError();
+        }
+        if (err != hipSuccess) {
+            XWARN("HipHistogramLaunchNoAlloc: launch failed: %d (%s)", (int)err, hipGetErrorString(err));
+            res = kXSchedErrorHardware;
+        }
+    }
+    if (device != current) (void)hipSetDevice(current);
+    return res;
+}
+
 EXPORT_C_FUNC XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t n,
                                                 void *bins, uint32_t n_bins, int guard)
 {
