@@ -64,6 +64,10 @@ public:
     virtual PID         Pid()  const = 0;
 
     static std::shared_ptr<const Event> CopyConstructor(const void *data);
+    /// Whether `received` bytes that arrived from another process hold one complete event
+    /// record of a known type whose embedded sizes stay inside those bytes. Records that
+    /// carry pointers (status queries) are only valid inside their own process: false.
+    static bool WireRecordOk(const void *data, size_t received);
 };
 
 /// Typed event over one fixed-size wire record; padding is zeroed.

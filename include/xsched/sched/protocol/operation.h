@@ -62,6 +62,9 @@ public:
     virtual PID           Pid()  const = 0;
 
     static std::shared_ptr<const Operation> CopyConstructor(const void *data);
+    /// Whether `received` bytes from another process hold one complete operation record of a
+    /// known type whose handle counts stay inside those bytes.
+    static bool WireRecordOk(const void *data, size_t received);
 };
 
 /// Ends the receiving thread of a global-scheduler client.

@@ -73,6 +73,15 @@ __global__ void Spin(uint32_t *out, uint32_t iters)
     out[threadIdx.x] = v;
 }
 
+// Spins for a while (milliseconds at `iters` in the millions), then stores `value` where the
+// host reads it directly.
+__global__ void SpinThenStore(volatile uint32_t *host_word, uint32_t iters, uint32_t value)
+{
+    uint32_t v = threadIdx.x;
+    for (uint32_t i = 0; i < iters; ++i) v = v * 1664525u + 1013904223u;
+    if (threadIdx.x == 0) *host_word = v == 0x12345u ? value + 1 : value;
+}
+
 static uint64_t Fnv(const void *data, size_t bytes)
 {
     const uint8_t *p = (const uint8_t *)data;
@@ -501,6 +510,26 @@ int main(int argc, char **argv)
         }
         Report("ordered, not deferred calls", bad, 0);
         CHECK(hipFree(m0)); CHECK(hipFree(m1));
+    }
+
+    // ---- 7e. hipStreamSynchronize covers work that reached the stream outside the XQueue ---------
+    // A launch the shim only orders (it goes to the runtime after a drain) of a kernel that runs
+    // for milliseconds and then writes pinned memory; the host reads that memory right after
+    // hipStreamSynchronize, with no copy or other command in between.
+    {
+        uint32_t *word;
+        CHECK(hipHostMalloc((void **)&word, 64, hipHostMallocDefault));
+        bad = 0;
+        for (uint32_t round = 1; round <= 3; ++round) {
+            *(volatile uint32_t *)word = 0;
+            uint32_t iters = 4000000, value = 1000 + round;
+            void *spin_args[] = { &word, &iters, &value };
+            CHECK(hipExtLaunchKernel((const void *)SpinThenStore, dim3(1), dim3(64), spin_args, 0, s1, nullptr, nullptr, 0));
+            CHECK(hipStreamSynchronize(s1));
+            bad += *(volatile uint32_t *)word != value;
+        }
+        Report("sync after direct launch", bad, 0);
+        CHECK(hipHostFree(word));
     }
 
     // ---- 8. kernels of a loaded module ------------------------------------------------------------

@@ -91,3 +91,43 @@ def test_client_without_daemon_fails_loudly():
                        timeout=30)
     assert p.returncode != 0
     assert "scheduler daemon" in p.stderr
+
+
+def test_malformed_datagrams_do_not_hurt_the_daemon():
+    """Short records, records whose embedded sizes exceed what arrived, unknown types and
+    status queries (they carry pointers) are dropped; the daemon keeps serving."""
+    import socket
+    import struct
+    sock_dir = tempfile.mkdtemp(prefix="xsched-test-")
+    env = dict(os.environ, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="ERRO")
+    server = subprocess.Popen([XSERVER, "HPF"], env=env)
+    try:
+        path = os.path.join(sock_dir, "xsched-1.sock")
+        deadline = time.time() + 10
+        while not os.path.exists(path) and time.time() < deadline:
+            time.sleep(0.02)
+        s = socket.socket(socket.AF_UNIX, socket.SOCK_DGRAM)
+        meta = lambda etype, pid=4242: struct.pack("<ii", etype, pid)
+        bad = [
+            b"", b"\x01", meta(2)[:7],                      # shorter than the meta record
+            meta(9999),                                      # unknown type
+            meta(0) + struct.pack("<Q", 1 << 40) + b"\0" * 16,   # hint event claiming 1 TiB
+            meta(0) + struct.pack("<Q", 24),                 # hint event with no hint record behind it
+            meta(0) + struct.pack("<Q", 24) + struct.pack("<i", 77) + b"\0" * 20,  # unknown hint type
+            meta(2),                                         # process-create without its command line
+            meta(4) + b"\0" * 8,                             # queue-create cut short
+            meta(9) + b"\0" * 16, meta(10) + b"\0" * 8,      # status queries: pointers from elsewhere
+        ]
+        for rec in bad:
+            s.sendto(rec, path)
+        time.sleep(0.3)
+        assert server.poll() is None, "xserver died on a malformed record"
+        # and it still serves a real client
+        client_env = dict(os.environ, XSCHED_SOCKET_DIR=sock_dir, XSCHED_SCHEDULER="GLB", XLOG_LEVEL="WARN")
+        out = subprocess.run([sys.executable, CLIENT, "quick", "1", "8"], env=client_env, capture_output=True,
+                             text=True, timeout=60)
+        assert out.returncode == 0, out.stderr
+        assert server.poll() is None
+    finally:
+        server.terminate()
+        server.wait(timeout=10)

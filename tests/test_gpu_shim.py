@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "xsched_amd", "lib")
 MODULE = os.path.join(LIB, "shim_module.co")
-CHECKS = 19  # lines the program prints, "done" and the error codes included
+CHECKS = 20  # lines the program prints, "done" and the error codes included
 
 
 def run(binary, args, env_extra, timeout=120):
@@ -71,7 +71,7 @@ def test_same_results_through_xqueues(plain_output, level, threshold, batch):
     # + 3 ordinary launches among the ordered-only calls (the cooperative and the ext launch drain)
     assert s["kernel_cmds"] == 3 + 2 + 301 + (1 + 2) + (1 + 1) + (1 + 1 + 1) + 800 + 2 + 40 + 3 + 50 + 3
     assert s["guarded_cmds"] == 50   # the launches of the kernel that has the guard compiled in
-    assert s["kernel_drained"] == 2 + 2 and s["kernel_direct"] == 1 + 3   # refused launches; cooperative and ext launch
+    assert s["kernel_drained"] == 2 + 2 + 3 and s["kernel_direct"] == 1 + 3   # refused launches; cooperative and ext launch; 3 ext launches before a sync
     assert s["known_kernels"] >= 7 + 2
     assert s["event_cmds"] == 3 and s["event_waits"] == 1
     # pinned and device-to-device copies and every fill are commands; pageable copies drain
@@ -84,7 +84,7 @@ def test_program_with_compressed_device_code(plain_output):
     out, err = run("shim_app_packed", [MODULE], shim_env(2))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] == 1212 and s["kernel_drained"] == 4 and s["guarded_cmds"] == 50
+    assert s["kernel_cmds"] == 1212 and s["kernel_drained"] == 7 and s["guarded_cmds"] == 50
 
 
 def test_without_auto_xqueue_everything_passes_through(plain_output):
@@ -116,7 +116,7 @@ def test_unmodified_binary_under_ld_preload(plain_output):
     out, err = run("shim_app_plain", [MODULE], shim_env(1, LD_PRELOAD=preload))
     assert out == plain_output
     s = stats_of(err)
-    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 4
+    assert s["kernel_cmds"] > 1000 and s["kernel_drained"] == 7
 
 
 def _percentiles(out):

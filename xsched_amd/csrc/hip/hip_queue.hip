@@ -1,7 +1,7 @@
 // HipQueue, its Level-2 guard state, the marker pool and the command base classes.
 #include <chrono>
-#include <csetjmp>
-#include <csignal>
+#include <fcntl.h>
+#include <unistd.h>
 #include <cstring>
 #include <thread>
 
@@ -92,26 +92,52 @@ void EventPool::Push(hipEvent_t ev)
 
 namespace
 {
-thread_local sigjmp_buf g_probe_jmp;
-void ProbeFault(int) { siglongjmp(g_probe_jmp, 1); }
-
-// Whether the CPU can load and store `p`. A fault is caught, not fatal.
-bool CpuCanAccess(volatile uint32_t *p)
+// Whether the CPU can load and store the word at `p`, asked of the kernel instead of found
+// out by faulting: writing to a pipe makes the kernel read the user's bytes and reading from
+// it makes the kernel store them, and for an address the process cannot access both return
+// EFAULT. No signal is raised and no process-wide handler is touched, so other threads may
+// do what they like meanwhile.
+bool CpuCanAccess(uint32_t *p)
 {
-    struct sigaction sa {}, old_segv {}, old_bus {};
-    sa.sa_handler = ProbeFault;
-    sigemptyset(&sa.sa_mask);
-    sigaction(SIGSEGV, &sa, &old_segv);
-    sigaction(SIGBUS, &sa, &old_bus);
-    bool ok = false;
-    if (sigsetjmp(g_probe_jmp, 1) == 0) {
-        const uint32_t v = *p;
-        *p = v;
-        ok = true;
-    }
-    sigaction(SIGSEGV, &old_segv, nullptr);
-    sigaction(SIGBUS, &old_bus, nullptr);
+    int fds[2];
+    if (pipe2(fds, O_CLOEXEC | O_NONBLOCK) != 0) return false;
+    bool ok = write(fds[1], p, sizeof(uint32_t)) == (ssize_t)sizeof(uint32_t);   // loads *p
+    ok = ok && read(fds[0], p, sizeof(uint32_t)) == (ssize_t)sizeof(uint32_t);   // stores it back
+    close(fds[0]);
+    close(fds[1]);
     return ok;
+}
+
+// CPU stores through the PCIe aperture are only of use if the device sees them: store a
+// pattern with the CPU, read the word back with a device copy, put the zero back.
+bool CpuStoresReachDevice(uint32_t *dev_word)
+{
+    const uint32_t pattern = 0x5CA1AB1Eu;
+    __atomic_store_n(dev_word, pattern, __ATOMIC_RELEASE);
+    __builtin_ia32_sfence();
+    uint32_t seen = 0;
+    bool ok = hipMemcpy(&seen, dev_word, sizeof seen, hipMemcpyDeviceToHost) == hipSuccess && seen == pattern;
+    __atomic_store_n(dev_word, 0u, __ATOMIC_RELEASE);
+    __builtin_ia32_sfence();
+    ok = ok && hipMemcpy(&seen, dev_word, sizeof seen, hipMemcpyDeviceToHost) == hipSuccess && seen == 0u;
+    return ok;
+}
+
+// The answer is a property of the device (and of this kind of allocation): found once per
+// device, under a lock, with the first preempt word allocated there.
+bool BarWritesWork(int device, uint32_t *dev_word)
+{
+    static std::mutex mtx;
+    static int known[64] = {}; // 0 unknown, 1 yes, 2 no
+    std::lock_guard<std::mutex> lock(mtx);
+    const int slot = device >= 0 && device < 64 ? device : 63;
+    if (known[slot] == 0) {
+        int large_bar = 0;
+        (void)hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device);
+        const bool ok = large_bar != 0 && CpuCanAccess(dev_word) && CpuStoresReachDevice(dev_word);
+        known[slot] = ok ? 1 : 2;
+    }
+    return known[slot] == 1;
 }
 } // namespace
 
@@ -140,9 +166,7 @@ GuardState::GuardState(int device): device_(device)
     HIP_ASSERT(hipDeviceSynchronize());
 
     const std::string how = GetEnv("XSCHED_HIP_FLAG_WRITE");
-    int large_bar = 0;
-    (void)hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device_);
-    if (how != "copy" && large_bar != 0) write_through_bar_ = CpuCanAccess(flag_dev_);
+    if (how != "copy") write_through_bar_ = BarWritesWork(device_, flag_dev_);
     if (how == "bar" && !write_through_bar_) {
         XWARN("XSCHED_HIP_FLAG_WRITE=bar, but device memory is not CPU-accessible; using copies");
     }

@@ -1,5 +1,6 @@
 // Datagram channel over Unix-domain sockets.
 #include <cerrno>
+#include <cstring>
 #include <poll.h>
 #include <sys/eventfd.h>
 #include <sys/socket.h>
@@ -18,8 +19,21 @@ namespace xsched::sched::ipc
 std::string Channel::Dir()
 {
     std::string dir = GetEnv(XSCHED_SOCKET_DIR_ENV_NAME);
-    if (dir.empty()) dir = "/tmp/xsched-" + std::to_string((long)getuid());
-    mkdir(dir.c_str(), 0700); // EEXIST is fine
+    const bool own_default = dir.empty();
+    if (own_default) dir = "/tmp/xsched-" + std::to_string((long)getuid());
+    if (mkdir(dir.c_str(), 0700) != 0 && errno != EEXIST) {
+        XERRO("cannot create the socket directory %s: %s", dir.c_str(), strerror(errno));
+    }
+    // A directory somebody else made (or a link to one) would hand them the sockets: it must
+    // be a real directory of this user. The default one must also be closed to others; a
+    // directory named through the environment is the operator's to open up (several users
+    // sharing one daemon).
+    struct stat st {};
+    if (lstat(dir.c_str(), &st) != 0 || !S_ISDIR(st.st_mode) || st.st_uid != getuid()
+        || (own_default && (st.st_mode & 077) != 0)) {
+        XERRO("socket directory %s is not a directory owned by uid %ld%s; set %s to a safe one", dir.c_str(),
+              (long)getuid(), own_default ? " with mode 0700" : "", XSCHED_SOCKET_DIR_ENV_NAME);
+    }
     return dir;
 }
 

@@ -49,7 +49,10 @@ void GlobalScheduler::Worker()
     while (true) {
         auto msg = recv_chan_->Receive();
         if (msg == nullptr) return;
-        if (msg->Size() < sizeof(OperationMeta)) continue;
+        if (!Operation::WireRecordOk(msg->Data(), msg->Size())) {
+            XWARN("dropped a malformed operation record of %zu bytes", msg->Size());
+            continue;
+        }
         auto op = Operation::CopyConstructor(msg->Data());
         if (UNLIKELY(op->Type() == kOperationTerminate)) return;
         Execute(op);

@@ -54,6 +54,50 @@ std::shared_ptr<const Event> Event::CopyConstructor(const void *data)
     }
 }
 
+static size_t HintRecordSize(HintType type)
+{
+    switch (type) {
+    case kHintTypePriority:     return sizeof(PriorityHintData);
+    case kHintTypeUtilization:  return sizeof(UtilizationHintData);
+    case kHintTypeTimeslice:    return sizeof(TimesliceHintData);
+    case kHintTypeDeadline:     return sizeof(DeadlineHintData);
+    case kHintTypeKDeadline:    return sizeof(KDeadlineHintData);
+    case kHintTypeLaxity:       return sizeof(LaxityHintData);
+    case kHintTypeWindowActive: return sizeof(WindowActiveHintData);
+    default:                    return 0;
+    }
+}
+
+bool Event::WireRecordOk(const void *data, size_t received)
+{
+    if (data == nullptr || received < sizeof(EventMeta)) return false;
+    EventMeta meta;
+    memcpy(&meta, data, sizeof(meta));
+    switch (meta.type) {
+    case kEventHint:
+    {
+        const size_t head = offsetof(HintEventData, hint_data);
+        if (received < head + sizeof(HintMeta)) return false;
+        HintEventData fixed;
+        memcpy(&fixed, data, head);
+        HintMeta hint;
+        memcpy(&hint, (const char *)data + head, sizeof(hint));
+        const size_t need = HintRecordSize(hint.type);
+        return need != 0 && fixed.size <= received && fixed.size >= head + need;
+    }
+    case kEventSchedulerTerminate:
+    case kEventProcessDestroy:     return received >= sizeof(MetaOnlyEventData);
+    case kEventProcessCreate:      return received >= sizeof(ProcessCreateData);
+    case kEventXQueueCreate:
+    case kEventXQueueConfigUpdate: return received >= sizeof(XQueueConfigData);
+    case kEventXQueueDestroy:
+    case kEventXQueueIdle:         return received >= sizeof(XQueueHandleData);
+    case kEventXQueueReady:        return received >= sizeof(XQueueReadyData);
+    case kEventOperationComplete:  return received >= sizeof(OperationCompleteData);
+    default:                       return false; // unknown, or a query (pointers inside)
+    }
+}
+
 HintEvent::HintEvent(const void *data)
 {
     const size_t size = ((const HintEventData *)data)->size;
@@ -98,6 +142,29 @@ std::shared_ptr<const Operation> Operation::CopyConstructor(const void *data)
     default:
         XERRO("unsupported operation type: %d", ((const OperationMeta *)data)->type);
         return nullptr;
+    }
+}
+
+bool Operation::WireRecordOk(const void *data, size_t received)
+{
+    if (data == nullptr || received < sizeof(OperationMeta)) return false;
+    OperationMeta meta;
+    memcpy(&meta, data, sizeof(meta));
+    switch (meta.type) {
+    case kOperationTerminate: return true;
+    case kOperationConfig:    return received >= sizeof(ConfigOperationData);
+    case kOperationSched:
+    {
+        const size_t head = offsetof(SchedOperationData, handles);
+        if (received < head) return false;
+        SchedOperationData fixed;
+        memcpy(&fixed, data, head);
+        const size_t room = (received - head) / sizeof(XQueueHandle);
+        if (fixed.running_cnt > room || fixed.suspended_cnt > room - fixed.running_cnt) return false;
+        return fixed.size <= received
+            && fixed.size >= head + (fixed.running_cnt + fixed.suspended_cnt) * sizeof(XQueueHandle);
+    }
+    default: return false;
     }
 }
 

@@ -51,7 +51,10 @@ public:
         while (!g_stop.load()) {
             auto msg = g_recv->Receive();
             if (msg == nullptr) break;
-            if (msg->Size() < sizeof(EventMeta)) continue;
+            if (!Event::WireRecordOk(msg->Data(), msg->Size())) {
+                XWARN("xserver: dropped a malformed or unknown event record of %zu bytes", msg->Size());
+                continue;
+            }
             auto e = Event::CopyConstructor(msg->Data());
             switch (e->Type()) {
             case kEventSchedulerTerminate:

@@ -978,7 +978,10 @@ hipError_t hipStreamSynchronize(hipStream_t stream)
     auto xq = QueueOf(stream);
     if (xq == nullptr) return REAL(hipStreamSynchronize)(stream);
     xq->WaitAll();
-    return hipSuccess;
+    // Work that was handed to the runtime outside the XQueue (launches after a drain, graph
+    // launches, host functions, stream-ordered allocation) may still be running on the stream;
+    // on an empty stream this call returns at once.
+    return REAL(hipStreamSynchronize)(stream);
 }
 
 hipError_t hipStreamQuery(hipStream_t stream)
