@@ -270,4 +270,4 @@ def test_reader_under_address_and_ub_sanitizers(tmp_path):
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-4000:]
     lines = proc.stdout.strip().splitlines()
     assert len(lines) == 3 and all("refused" in line for line in lines), proc.stdout
-    assert lines[0].split(":")[1].strip().startswith("10 kernels") and lines[2].split(":")[1].strip().startswith("2 kernels")
+    assert lines[0].split(":")[1].strip().startswith("11 kernels") and lines[2].split(":")[1].strip().startswith("2 kernels")
