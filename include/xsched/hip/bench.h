@@ -76,6 +76,29 @@ XResult XBenchRunBackgroundAlone(XBench *b, int commands, XBenchPhaseResult *res
 /* Foreground every period while all background queues stream back to back. */
 XResult XBenchRunContended(XBench *b, int samples, double *latency_us, XBenchPhaseResult *res);
 
+/* Where the latency of one foreground command goes. One command per period, `samples` of
+ * them, alone or (contended != 0) beside the background queues; a timing event is recorded
+ * in stream order right before and right after the kernel. out holds 4 values per sample,
+ * microseconds:
+ *   [0] submit   host time until everything is handed over: through an XQueue the three
+ *                XQueueSubmit calls (the launch itself runs inside them when the launch
+ *                thread sleeps), otherwise the event records and the launch call
+ *   [1] device   time between the two events on the device (hipEventElapsedTime): from the
+ *                point the stream reaches the command to the kernel's end
+ *   [2] wait     from there until the host knows the command is done (XQueueWaitAll returns;
+ *                HwQueueSynchronize returns; hipStreamQuery polling succeeds)
+ *   [3] total    [0] + [2]
+ * mode 0: through the foreground XQueue (same path as XBenchRunForegroundAlone / Contended,
+ *         plus the two event-record commands);
+ * mode 1: the adapter without the XQueue core: HwQueueLaunch + HwQueueSynchronize on a
+ *         stream of its own;
+ * mode 2: plain HIP: a stand-in kernel of the same traffic launched with <<<>>> on a stream
+ *         of its own and awaited by polling hipStreamQuery (AXPY foreground only): the floor
+ *         the device and runtime set, with nothing of this library on the path.
+ * The foreground output buffer is updated in every mode (applied counts them all). */
+XResult XBenchRunForegroundBreakdown(XBench *b, int samples, int mode, int contended, double *out,
+                                     XBenchPhaseResult *res);
+
 /* Level-2 / level-1 preemption latency of background queue 0 while it streams:
  * `samples` rounds of XQueueSuspend(kQueueSuspendFlagSyncHwQueue) and
  * XQueueResume, each timed on the host (microseconds). */

@@ -41,8 +41,7 @@ PREEMPT_SRCS = [
     "protocol/log.cpp", "protocol/names.cpp",
     "sched/protocol.cpp", "sched/policy.cpp", "sched/policy_extra.cpp", "sched/local.cpp", "sched/global.cpp",
     "sched/channel.cpp",
-    "preempt/xcommand.cpp", "preempt/command_buffer.cpp", "preempt/launch_worker.cpp",
-    "preempt/async_xqueue.cpp", "preempt/xqueue.cpp", "preempt/agent.cpp",
+    "preempt/xcommand.cpp", "preempt/ring_queue.cpp", "preempt/xqueue.cpp", "preempt/agent.cpp",
 ]
 HOST_SRCS = ["host/host_queue.cpp"]
 SERVER_SRCS = ["service/xserver.cpp"]

@@ -46,6 +46,20 @@ __global__ void FillZipf(int32_t *dst, uint64_t n, uint64_t key, const uint32_t 
          i += (uint64_t)gridDim.x * blockDim.x) dst[i] = (int32_t)synth_zipf_key(table, n_bins, key, i);
 }
 
+// y = 0.5 * x + y with 128-bit accesses, one work-group per 1024 elements: the plain-HIP
+// stand-in of the foreground AXPY for the latency floor (n a multiple of 4).
+__global__ void FloorAxpy(const float4 *x, float4 *y, uint64_t n4)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n4) {
+        const float4 a = x[i];
+        float4 b = y[i];
+        b.x = fmaf(0.5f, a.x, b.x); b.y = fmaf(0.5f, a.y, b.y);
+        b.z = fmaf(0.5f, a.z, b.z); b.w = fmaf(0.5f, a.w, b.w);
+        y[i] = b;
+    }
+}
+
 constexpr uint32_t kHistBins = 65536;
 constexpr double kZipfS = 1.1;
 
@@ -397,6 +411,106 @@ EXPORT_C_FUNC XResult XBenchRunContended(XBench *b, int samples, double *latency
     }
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult XBenchRunForegroundBreakdown(XBench *b, int samples, int mode, int contended, double *out,
+                                                   XBenchPhaseResult *res)
+{
+    if (b == nullptr || b->fg == nullptr || samples <= 0 || out == nullptr || mode < 0 || mode > 2) {
+        return kXSchedErrorInvalidValue;
+    }
+    if (contended && b->bg.empty()) return kXSchedErrorInvalidValue;
+    Lane &fg = *b->fg;
+    if (mode == 2 && (fg.spec.kind != kXBenchAxpy || fg.spec.n % 4 != 0)) return kXSchedErrorNotSupported;
+    hipEvent_t ev_a, ev_b;
+    BENCH_HIP(hipEventCreate(&ev_a));
+    BENCH_HIP(hipEventCreate(&ev_b));
+    // modes 1 and 2 use a stream of their own, with no XQueue on it
+    hipStream_t raw = nullptr;
+    HwQueueHandle raw_hwq = 0;
+    if (mode != 0) {
+        BENCH_X(XQueueWaitAll(fg.xq));
+        BENCH_HIP(hipStreamCreateWithFlags(&raw, hipStreamNonBlocking));
+        if (mode == 1) BENCH_X(HipQueueCreate(&raw_hwq, raw));
+    }
+
+    std::atomic<bool> stop { false };
+    std::vector<std::unique_ptr<BgDriver>> drivers;
+    if (contended) {
+        for (auto &lane : b->bg) {
+            auto d = std::make_unique<BgDriver>();
+            d->lane = lane.get();
+            d->burst = b->cfg.bg_burst > 0 ? b->cfg.bg_burst : 64;
+            d->stop = &stop;
+            drivers.emplace_back(std::move(d));
+        }
+        for (auto &d : drivers) d->Start();
+        std::this_thread::sleep_for(std::chrono::milliseconds(50));
+    }
+
+    const auto t_begin = Clock::now();
+    auto next = t_begin;
+    auto us = [](Clock::duration d) { return std::chrono::duration<double, std::micro>(d).count(); };
+    for (int i = 0; i < samples; ++i) {
+        SleepUntil(next);
+        Clock::time_point t0, t1, t2;
+        if (mode == 0) {
+            HwCommandHandle rec_a = 0, rec_b = 0;
+            BENCH_X(HipEventRecordCommandCreate(&rec_a, ev_a));
+            BENCH_X(HipEventRecordCommandCreate(&rec_b, ev_b));
+            const HwCommandHandle cmd = fg.MakeCommand();
+            t0 = Clock::now();
+            BENCH_X(XQueueSubmit(fg.xq, rec_a));
+            BENCH_X(XQueueSubmit(fg.xq, cmd));
+            BENCH_X(XQueueSubmit(fg.xq, rec_b));
+            t1 = Clock::now();
+            BENCH_X(XQueueWaitAll(fg.xq));
+            t2 = Clock::now();
+            fg.applied.fetch_add(1, std::memory_order_relaxed);
+        } else if (mode == 1) {
+            const HwCommandHandle cmd = fg.MakeCommand();
+            t0 = Clock::now();
+            BENCH_HIP(hipEventRecord(ev_a, raw));
+            BENCH_X(HwQueueLaunch(raw_hwq, cmd));
+            BENCH_HIP(hipEventRecord(ev_b, raw));
+            t1 = Clock::now();
+            BENCH_X(HwQueueSynchronize(raw_hwq));
+            t2 = Clock::now();
+            fg.applied.fetch_add(1, std::memory_order_relaxed);
+        } else {
+            const uint64_t n4 = fg.spec.n / 4;
+            t0 = Clock::now();
+            BENCH_HIP(hipEventRecord(ev_a, raw));
+            hipLaunchKernelGGL(FloorAxpy, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, raw,
+                               (const float4 *)fg.in0, (float4 *)fg.out, n4);
+            BENCH_HIP(hipEventRecord(ev_b, raw));
+            t1 = Clock::now();
+            while (hipStreamQuery(raw) == hipErrorNotReady) __builtin_ia32_pause();
+            t2 = Clock::now();
+            fg.applied.fetch_add(1, std::memory_order_relaxed);
+        }
+        float ms = 0;
+        BENCH_HIP(hipEventSynchronize(ev_b));
+        BENCH_HIP(hipEventElapsedTime(&ms, ev_a, ev_b));
+        out[(size_t)i * 4 + 0] = us(t1 - t0);
+        out[(size_t)i * 4 + 1] = (double)ms * 1e3;
+        out[(size_t)i * 4 + 2] = us(t2 - t1);
+        out[(size_t)i * 4 + 3] = us(t2 - t0);
+        next += std::chrono::microseconds(fg.spec.period_us);
+    }
+    stop.store(true, std::memory_order_release);
+    for (auto &d : drivers) d->Join();
+    if (res) {
+        *res = XBenchPhaseResult {};
+        res->elapsed_s = std::chrono::duration<double>(Clock::now() - t_begin).count();
+        res->fg_samples = (uint64_t)samples;
+        FillStats(b, res);
+    }
+    if (raw_hwq) BENCH_X(HwQueueDestroy(raw_hwq));
+    if (raw) { (void)hipStreamSynchronize(raw); (void)hipStreamDestroy(raw); }
+    (void)hipEventDestroy(ev_a);
+    (void)hipEventDestroy(ev_b);
     return kXSchedSuccess;
 }
 

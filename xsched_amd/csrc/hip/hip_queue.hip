@@ -443,21 +443,29 @@ void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
     n_launch.fetch_add(1, std::memory_order_relaxed);
 }
 
-// Polls first, like a marker wait: the blocking call costs a sleep and a wake-up
-// through the driver, which is longer than most foreground kernels run.
+// A marker recorded behind whatever the stream holds, then polled like any marker. Asking
+// the runtime about the stream itself (hipStreamQuery / hipStreamSynchronize) is several
+// times slower when the newest operation on it is a kernel: the runtime then has to put a
+// marker of its own behind the kernel first and hears of its completion through its signal
+// thread. Recorded here, the marker is on its way while the kernel still runs.
 void HipQueue::Synchronize()
 {
     DeviceScope scope(device_);
     RelaxedCaptureScope relaxed;
+    hipEvent_t marker = EventPool::Instance().Pop();
+    hipError_t err = hipEventRecord(marker, stream_);
+    XASSERT(err == hipSuccess, "hipEventRecord failed: %d (%s)", (int)err, hipGetErrorString(err));
     const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(SyncSpinMicros());
-    while (true) {
-        const hipError_t err = hipStreamQuery(stream_);
-        if (err == hipSuccess) return;
-        XASSERT(err == hipErrorNotReady, "hipStreamQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
-        if (std::chrono::steady_clock::now() >= give_up) break;
+    bool done = false;
+    for (int probes = 1; !done; ++probes) {
+        err = hipEventQuery(marker);
+        if (err == hipSuccess) { done = true; break; }
+        XASSERT(err == hipErrorNotReady, "hipEventQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
+        if ((probes & 7) == 0 && std::chrono::steady_clock::now() >= give_up) break;
         __builtin_ia32_pause();
     }
-    HIP_ASSERT(hipStreamSynchronize(stream_));
+    if (!done) HIP_ASSERT(hipEventSynchronize(marker));
+    EventPool::Instance().Push(marker);
 }
 
 void HipQueue::Deactivate()

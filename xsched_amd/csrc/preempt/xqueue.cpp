@@ -7,7 +7,7 @@
 #include "xsched/utils/env.h"
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/def.h"
-#include "xsched/preempt/xqueue/async_xqueue.h"
+#include "ring_queue.h"
 #include "xsched/preempt/xqueue/xqueue.h"
 
 namespace xsched::preempt
@@ -42,7 +42,7 @@ XResult XQueueManager::Add(XQueueHandle *xq_hp, HwQueueHandle hwq_h, int64_t lev
         return kXSchedSuccess;
     }
 
-    auto xq = std::make_shared<AsyncXQueue>(hwq, (XPreemptLevel)level);
+    auto xq = std::make_shared<RingXQueue>(hwq, (XPreemptLevel)level);
     hwq->SetXQueue(xq); // cycle, broken in Del()
     g_xqs[xq->GetHandle()] = xq;
     *xq_hp = xq->GetHandle();

@@ -49,6 +49,8 @@ def lib():
         h.XBenchRunForegroundAlone.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
         h.XBenchRunBackgroundAlone.argtypes = [c_void_p, c_int, POINTER(PhaseResult)]
         h.XBenchRunContended.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
+        h.XBenchRunForegroundBreakdown.argtypes = [c_void_p, c_int, c_int, c_int, POINTER(c_double),
+                                                   POINTER(PhaseResult)]
         h.XBenchRunPreempt.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(c_double),
                                        POINTER(PhaseResult)]
         h.XBenchRunPreemptDeviceTimed.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
@@ -103,6 +105,13 @@ class Bench:
         lat, res = (c_double * samples)(), PhaseResult()
         xsched_amd.check(lib().XBenchRunContended(self.h, samples, lat, byref(res)))
         return list(lat), res
+
+    def fg_breakdown(self, samples, mode, contended):
+        """Columns submit / device / wait / total (lists, microseconds); see bench.h."""
+        out, res = (c_double * (samples * 4))(), PhaseResult()
+        xsched_amd.check(lib().XBenchRunForegroundBreakdown(self.h, samples, mode, 1 if contended else 0, out, byref(res)))
+        return {name: [out[i * 4 + k] for i in range(samples)]
+                for k, name in enumerate(("submit", "device", "wait", "total"))}
 
     def preempt(self, samples):
         sus, resume, res = (c_double * samples)(), (c_double * samples)(), PhaseResult()
