@@ -10,8 +10,9 @@
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/def.h"
 #include "xsched/protocol/names.h"
-#include "xsched/preempt/sched/agent.h"
+#include "agent.h"
 #include "xsched/preempt/xqueue/xqueue.h"
+#include "xsched/sched/policy/policy.h"
 #include "xsched/sched/scheduler/local.h"
 
 using namespace xsched::sched;

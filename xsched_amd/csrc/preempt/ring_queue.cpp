@@ -6,7 +6,7 @@
 #include "ring_queue.h"
 #include "xsched/utils/env.h"
 #include "xsched/utils/xassert.h"
-#include "xsched/preempt/sched/agent.h"
+#include "agent.h"
 
 using namespace xsched::sched;
 

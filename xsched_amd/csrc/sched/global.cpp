@@ -1,7 +1,7 @@
 // Daemon client. reference sched/src/scheduler/global.cpp:17-69
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/def.h"
-#include "xsched/sched/scheduler/global.h"
+#include "global.h"
 
 namespace xsched::sched
 {

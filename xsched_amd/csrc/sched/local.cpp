@@ -1,18 +1,36 @@
-// In-process scheduler. reference sched/src/scheduler/{local,scheduler}.cpp
+// The in-process scheduler: an inbox, a ledger of operations, a mirror of the XQueues, a
+// heap of alarms and one thread that turns them over in rounds.
+//
+//   round = take everything in the inbox (or an alarm that has come due)
+//           -> fold each event into the mirror (hints go to the policy)
+//           -> policy.Sched(mirror): it answers by marking XQueues suspended / running
+//           -> one scheduling operation per process that has XQueues
+//
+// What a round decides and emits (operation ids included) is that of reference
+// sched/src/scheduler/local.cpp:42-446; tests replay recorded event scripts through both.
 #include <algorithm>
+#include <array>
+#include <condition_variable>
+#include <map>
+#include <mutex>
+#include <queue>
+#include <thread>
+#include <vector>
 
+#include "global.h"
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/names.h"
-#include "xsched/sched/scheduler/global.h"
+#include "xsched/sched/policy/policy.h"
+#include "xsched/sched/protocol/status.h"
 #include "xsched/sched/scheduler/local.h"
-#include "xsched/sched/scheduler/scheduler.h"
 
-using namespace std::chrono;
 using namespace xsched::protocol;
 
 namespace xsched::sched
 {
 
+// A valid policy selects the local scheduler whatever the type says; otherwise the daemon
+// client or the scheduler that does nothing (reference sched/src/scheduler/scheduler.cpp:19-34).
 std::shared_ptr<Scheduler> CreateScheduler(XSchedulerType scheduler, XPolicyType policy)
 {
     if (policy > kPolicyUnknown && policy < kPolicyMax) {
@@ -27,331 +45,368 @@ std::shared_ptr<Scheduler> CreateScheduler(XSchedulerType scheduler, XPolicyType
     return std::make_shared<AppManagedScheduler>();
 }
 
-LocalScheduler::LocalScheduler(XPolicyType type): Scheduler(kSchedulerLocal), policy_type_(type)
+namespace
 {
-    InstallPolicy(type);
-}
 
-LocalScheduler::~LocalScheduler() { this->Stop(); }
+using EventPtr = std::shared_ptr<const Event>;
+using Clock = std::chrono::system_clock;
 
-void LocalScheduler::InstallPolicy(XPolicyType type)
+/// Events waiting for the next round, and the alarms policies have set.
+class Inbox
 {
-    policy_type_ = type;
-    policy_ = CreatePolicy(type);
-    policy_->SetSuspendFunc([this](XQueueHandle h) { this->Suspend(h); });
-    policy_->SetResumeFunc([this](XQueueHandle h) { this->Resume(h); });
-    policy_->SetAddTimerFunc([this](TimePoint tp) { this->AddTimer(tp); });
-}
-
-void LocalScheduler::Run()
-{
-    thread_ = std::make_unique<std::thread>(&LocalScheduler::Worker, this);
-}
-
-void LocalScheduler::Stop()
-{
-    if (thread_) {
-        this->RecvEvent(std::make_shared<SchedulerTerminateEvent>());
-        thread_->join();
-        thread_ = nullptr;
-    }
-    timers_.clear();
-}
-
-// Operation bookkeeping is updated right here on the caller's thread, because the
-// worker thread itself may sit in WaitAllOperations() (local.cpp:42-96).
-void LocalScheduler::RecvEvent(std::shared_ptr<const Event> event)
-{
-    switch (event->Type()) {
-    case kEventProcessCreate:
+public:
+    void Put(EventPtr event)
     {
-        { std::lock_guard<std::mutex> lock(op_mtx_); ops_.try_emplace(event->Pid()); }
-        op_cv_.notify_all();
-        break;
+        { std::lock_guard<std::mutex> g(mu_); waiting_.push_back(std::move(event)); }
+        cv_.notify_one();
     }
-    case kEventProcessDestroy:
+
+    void SetAlarm(TimePoint at)
     {
-        { std::lock_guard<std::mutex> lock(op_mtx_); ops_.erase(event->Pid()); }
-        op_cv_.notify_all();
-        break;
+        std::lock_guard<std::mutex> g(mu_);
+        alarms_.push(at);
     }
-    case kEventOperationComplete:
+
+    void ClearAlarms()
     {
-        auto done = static_cast<const OperationCompleteEvent *>(event.get());
+        std::lock_guard<std::mutex> g(mu_);
+        while (!alarms_.empty()) alarms_.pop();
+    }
+
+    /// Blocks until there are events or an alarm is due; `batch` receives the events (none
+    /// when an alarm ended the wait). Every alarm that is due is struck off together.
+    void Take(std::vector<EventPtr> *batch)
+    {
+        batch->clear();
+        std::unique_lock<std::mutex> g(mu_);
+        while (waiting_.empty()) {
+            if (alarms_.empty()) { cv_.wait(g); continue; }
+            const TimePoint first = alarms_.top();
+            const TimePoint now = Clock::now();
+            if (now < first) { cv_.wait_until(g, first); continue; }
+            while (!alarms_.empty() && !(now < alarms_.top())) alarms_.pop();
+            return;
+        }
+        batch->swap(waiting_);
+    }
+
+private:
+    std::mutex mu_;
+    std::condition_variable cv_;
+    std::vector<EventPtr> waiting_;
+    std::priority_queue<TimePoint, std::vector<TimePoint>, std::greater<TimePoint>> alarms_;
+};
+
+/// Per process: the id of the newest operation sent and of the newest one reported done.
+/// Kept outside the round thread's data: completions arrive on the callers' threads.
+class Ledger
+{
+public:
+    void Open(PID pid)  { { std::lock_guard<std::mutex> g(mu_); book_.try_emplace(pid); } cv_.notify_all(); }
+    void Close(PID pid) { { std::lock_guard<std::mutex> g(mu_); book_.erase(pid); } cv_.notify_all(); }
+
+    /// 0 for a process that never announced itself.
+    OperationId Issue(PID pid)
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        auto it = book_.find(pid);
+        return it == book_.end() ? 0 : ++it->second.sent;
+    }
+
+    void Done(PID pid, OperationId id)
+    {
         {
-            std::lock_guard<std::mutex> lock(op_mtx_);
-            auto it = ops_.find(done->Pid());
-            if (it == ops_.end()) {
-                XWARN("operation " FMT_64U " completed by unknown process " FMT_PID,
-                      done->OpId(), done->Pid());
+            std::lock_guard<std::mutex> g(mu_);
+            auto it = book_.find(pid);
+            if (it == book_.end()) {
+                XWARN("operation " FMT_64U " completed by unknown process " FMT_PID, id, pid);
                 return;
             }
-            XASSERT(done->OpId() <= it->second.issued_id,
-                    "unknown operation " FMT_64U " completed", done->OpId());
-            it->second.completed_id = std::max(it->second.completed_id, done->OpId());
+            XASSERT(id <= it->second.sent, "unknown operation " FMT_64U " completed", id);
+            it->second.done = std::max(it->second.done, id);
         }
-        op_cv_.notify_all();
-        return; // not queued
-    }
-    default:
-        break;
+        cv_.notify_all();
     }
 
-    { std::lock_guard<std::mutex> lock(event_mtx_); event_queue_.emplace_back(std::move(event)); }
-    event_cv_.notify_one();
-}
+private:
+    struct Line { OperationId sent = 0, done = 0; };
+    std::mutex mu_;
+    std::condition_variable cv_;
+    std::map<PID, Line> book_;
+};
 
-void LocalScheduler::SetPolicy(XPolicyType type)
+/// The Status a policy reads, and the only code that edits it.
+class Mirror
 {
-    if (type == policy_type_) return;
-    const std::string old = GetPolicyTypeName(policy_type_);
-    this->Stop();
-    InstallPolicy(type);
-    // Start the new policy from "everything runs".
-    for (auto &status : status_.xqueue_status) Resume(status.first);
-    this->Run();
-    XINFO("policy changed from %s to %s", old.c_str(), GetPolicyTypeName(type).c_str());
-}
+public:
+    const Status &View() const { return status_; }
 
-void LocalScheduler::WaitAllOperations()
-{
-    std::unique_lock<std::mutex> lock(op_mtx_);
-    op_cv_.wait(lock, [this]() {
-        for (auto &p : ops_) if (p.second.completed_id < p.second.issued_id) return false;
-        return true;
-    });
-}
-
-void LocalScheduler::WaitOperations(PID pid)
-{
-    std::unique_lock<std::mutex> lock(op_mtx_);
-    op_cv_.wait(lock, [this, pid]() {
-        auto it = ops_.find(pid);
-        return it == ops_.end() || it->second.completed_id >= it->second.issued_id;
-    });
-}
-
-OperationId LocalScheduler::NextOperationId(PID pid)
-{
-    std::lock_guard<std::mutex> lock(op_mtx_);
-    auto it = ops_.find(pid);
-    return it == ops_.end() ? 0 : ++(it->second.issued_id);
-}
-
-// One round = take every queued event, fold it into Status, run the policy once,
-// send one SchedOperation per process. Rounds are triggered by events or by the
-// earliest timer a policy asked for (local.cpp:142-196).
-void LocalScheduler::Worker()
-{
-    std::vector<std::shared_ptr<const Event>> batch;
-    std::unique_lock<std::mutex> lock(event_mtx_);
-
-    while (true) {
-        while (event_queue_.empty()) {
-            if (timers_.empty()) { event_cv_.wait(lock); continue; }
-            const auto first = timers_.front();
-            const auto now = system_clock::now();
-            if (now < first) { event_cv_.wait_until(lock, first); continue; }
-            while (!timers_.empty() && !(now < timers_.front())) timers_.pop_front();
-            break;
+    ProcessStatus &Process(PID pid)
+    {
+        auto &slot = status_.process_status[pid];
+        if (slot == nullptr) {
+            slot = std::make_unique<ProcessStatus>();
+            slot->info.pid = pid;
         }
-        batch.clear();
-        batch.swap(event_queue_);
-        lock.unlock();
+        return *slot;
+    }
 
-        bool terminate = false;
-        for (auto &event : batch) {
-            if (UNLIKELY(event->Type() == kEventSchedulerTerminate)) { terminate = true; continue; }
-            this->UpdateStatus(*event);
-        }
+    XQueueStatus *Find(XQueueHandle handle)
+    {
+        auto it = status_.xqueue_status.find(handle);
+        return it == status_.xqueue_status.end() ? nullptr : it->second.get();
+    }
 
-        policy_->Sched(status_);
-        this->ExecuteOperations();
-        std::sort(timers_.begin(), timers_.end());
-        if (terminate) return;
-        lock.lock();
+    /// A queue heard of for the first time; it starts out running.
+    XQueueStatus &Adopt(PID pid, XQueueHandle handle)
+    {
+        auto fresh = std::make_unique<XQueueStatus>();
+        fresh->handle = handle;
+        fresh->device = kDeviceTypeUnknown;
+        fresh->level = kPreemptLevelUnknown;
+        fresh->pid = pid;
+        fresh->threshold = 0;
+        fresh->batch_size = 0;
+        fresh->ready = false;
+        fresh->suspended = false;
+        fresh->ready_time = Clock::now();
+        XQueueStatus &ref = *fresh;
+        status_.xqueue_status[handle] = std::move(fresh);
+        Process(pid).running_xqueues.insert(handle);
+        return ref;
     }
-}
 
-void LocalScheduler::ExecuteOperations()
-{
-    for (auto &entry : status_.process_status) {
-        ProcessStatus &ps = *entry.second;
-        if (ps.running_xqueues.empty() && ps.suspended_xqueues.empty()) continue;
-        Execute(std::make_shared<SchedOperation>(NextOperationId(ps.info.pid), ps));
+    void ForgetQueue(XQueueHandle handle, PID claimed_owner)
+    {
+        auto it = status_.xqueue_status.find(handle);
+        if (it == status_.xqueue_status.end()) return;
+        XASSERT(claimed_owner == it->second->pid, "XQueue destroyed by a process that does not own it");
+        auto owner = status_.process_status.find(it->second->pid);
+        if (owner == status_.process_status.end()) return;
+        owner->second->running_xqueues.erase(handle);
+        owner->second->suspended_xqueues.erase(handle);
+        status_.xqueue_status.erase(it);
     }
-}
 
-void LocalScheduler::CreateXQueueStatus(PID pid, XQueueHandle handle, XDevice device,
-                                        XPreemptLevel level, int64_t threshold,
-                                        int64_t batch_size, bool ready,
-                                        system_clock::time_point ready_time)
-{
-    auto xq = std::make_unique<XQueueStatus>();
-    xq->handle = handle;
-    xq->device = device;
-    xq->level = level;
-    xq->pid = pid;
-    xq->threshold = threshold;
-    xq->batch_size = batch_size;
-    xq->ready = ready;
-    xq->suspended = false;
-    xq->ready_time = ready_time;
-    status_.xqueue_status[handle] = std::move(xq);
+    void ForgetProcess(PID pid)
+    {
+        auto it = status_.process_status.find(pid);
+        if (it == status_.process_status.end()) return;
+        for (XQueueHandle h : it->second->running_xqueues) status_.xqueue_status.erase(h);
+        for (XQueueHandle h : it->second->suspended_xqueues) status_.xqueue_status.erase(h);
+        status_.process_status.erase(it);
+    }
 
-    auto &ps = status_.process_status[pid];
-    if (ps == nullptr) {
-        ps = std::make_unique<ProcessStatus>();
-        ps->info.pid = pid;
+    /// The policy's verdict on one queue; a verdict that changes nothing is not recorded.
+    void Mark(XQueueHandle handle, bool suspended)
+    {
+        XQueueStatus *xq = Find(handle);
+        if (xq == nullptr || xq->suspended == suspended) return;
+        xq->suspended = suspended;
+        auto owner = status_.process_status.find(xq->pid);
+        if (owner == status_.process_status.end()) return;
+        ProcessStatus &ps = *owner->second;
+        auto &from = suspended ? ps.running_xqueues : ps.suspended_xqueues;
+        auto &to = suspended ? ps.suspended_xqueues : ps.running_xqueues;
+        from.erase(handle);
+        to.insert(handle);
+        (suspended ? ps.xqueues_to_suspend : ps.xqueues_to_resume).insert(handle);
     }
-    ps->running_xqueues.insert(handle);
-}
 
-void LocalScheduler::UpdateStatus(const Event &event)
-{
-    switch (event.Type()) {
-    case kEventHint:
-        policy_->RecvHint(static_cast<const HintEvent &>(event).GetHint());
-        break;
-    case kEventProcessCreate:
+    void Answer(StatusQuery *query, const XQueueStatus *only)
     {
-        auto &e = static_cast<const ProcessCreateEvent &>(event);
-        auto &ps = status_.process_status[e.Pid()];
-        if (ps == nullptr) {
-            ps = std::make_unique<ProcessStatus>();
-            ps->info.pid = e.Pid();
-        }
-        ps->info.cmdline = e.Cmdline();
-        break;
-    }
-    case kEventProcessDestroy:
-    {
-        auto pit = status_.process_status.find(event.Pid());
-        if (pit == status_.process_status.end()) break;
-        for (XQueueHandle h : pit->second->running_xqueues)   status_.xqueue_status.erase(h);
-        for (XQueueHandle h : pit->second->suspended_xqueues) status_.xqueue_status.erase(h);
-        status_.process_status.erase(pit);
-        break;
-    }
-    case kEventXQueueCreate:
-    case kEventXQueueConfigUpdate:
-    {
-        // Both carry the same record (XQueueConfigData).
-        auto *d = (const XQueueConfigData *)event.Data();
-        auto it = status_.xqueue_status.find(d->handle);
-        if (it == status_.xqueue_status.end()) {
-            CreateXQueueStatus(event.Pid(), d->handle, d->device, d->level,
-                               d->threshold, d->batch_size, false, system_clock::now());
-        } else {
-            it->second->device = d->device;
-            it->second->level = d->level;
-            it->second->threshold = d->threshold;
-            it->second->batch_size = d->batch_size;
-        }
-        break;
-    }
-    case kEventXQueueDestroy:
-    {
-        auto &e = static_cast<const XQueueDestroyEvent &>(event);
-        auto qit = status_.xqueue_status.find(e.Handle());
-        if (qit == status_.xqueue_status.end()) break;
-        const PID pid = qit->second->pid;
-        XASSERT(e.Pid() == pid, "XQueue destroyed by a process that does not own it");
-        auto pit = status_.process_status.find(pid);
-        if (pit == status_.process_status.end()) break;
-        pit->second->running_xqueues.erase(e.Handle());
-        pit->second->suspended_xqueues.erase(e.Handle());
-        status_.xqueue_status.erase(qit);
-        break;
-    }
-    case kEventXQueueReady:
-    {
-        auto &e = static_cast<const XQueueReadyEvent &>(event);
-        auto it = status_.xqueue_status.find(e.Handle());
-        if (it == status_.xqueue_status.end()) {
-            CreateXQueueStatus(e.Pid(), e.Handle(), kDeviceTypeUnknown, kPreemptLevelUnknown,
-                               0, 0, true, e.ReadyTime());
-        } else {
-            it->second->ready = true;
-            it->second->ready_time = e.ReadyTime();
-        }
-        break;
-    }
-    case kEventXQueueIdle:
-    {
-        auto &e = static_cast<const XQueueIdleEvent &>(event);
-        auto it = status_.xqueue_status.find(e.Handle());
-        if (it == status_.xqueue_status.end()) {
-            CreateXQueueStatus(e.Pid(), e.Handle(), kDeviceTypeUnknown, kPreemptLevelUnknown,
-                               0, 0, false, system_clock::now());
-        } else {
-            it->second->ready = false;
-        }
-        break;
-    }
-    case kEventXQueueQuery:
-    {
-        auto &e = static_cast<const XQueueQueryEvent &>(event);
-        StatusQuery *query = e.QueryData();
-        auto it = status_.xqueue_status.find(e.Handle());
-        if (it != status_.xqueue_status.end()) {
-            query->status_.emplace_back(std::make_unique<XQueueStatus>(*it->second));
-            if (query->QueryProcess()) {
-                auto pit = status_.process_status.find(it->second->pid);
-                if (pit != status_.process_status.end()) {
-                    query->processes_.emplace_back(std::make_unique<ProcessInfo>(pit->second->info));
-                }
-            }
-        }
-        query->Notify();
-        break;
-    }
-    case kEventXQueueQueryAll:
-    {
-        auto &e = static_cast<const XQueueQueryAllEvent &>(event);
-        StatusQuery *query = e.QueryData();
-        for (auto &s : status_.xqueue_status) {
-            query->status_.emplace_back(std::make_unique<XQueueStatus>(*s.second));
+        for (auto &entry : status_.xqueue_status) {
+            if (only != nullptr && entry.second.get() != only) continue;
+            query->status_.emplace_back(std::make_unique<XQueueStatus>(*entry.second));
         }
         if (query->QueryProcess()) {
-            for (auto &p : status_.process_status) {
-                query->processes_.emplace_back(std::make_unique<ProcessInfo>(p.second->info));
+            for (auto &entry : status_.process_status) {
+                if (only != nullptr && entry.first != only->pid) continue;
+                query->processes_.emplace_back(std::make_unique<ProcessInfo>(entry.second->info));
             }
         }
+    }
+
+private:
+    Status status_;
+};
+
+} // namespace
+
+class LocalScheduler::Rounds
+{
+public:
+    Rounds(LocalScheduler *owner, XPolicyType type): owner_(owner) { Install(type); }
+
+    void Install(XPolicyType type)
+    {
+        type_ = type;
+        policy_ = CreatePolicy(type);
+        policy_->SetSuspendFunc([this](XQueueHandle h) { mirror_.Mark(h, true); });
+        policy_->SetResumeFunc([this](XQueueHandle h) { mirror_.Mark(h, false); });
+        policy_->SetAddTimerFunc([this](TimePoint at) { inbox_.SetAlarm(at); });
+    }
+
+    void Start() { thread_ = std::thread([this]() { Turn(); }); }
+
+    void Halt()
+    {
+        if (thread_.joinable()) {
+            inbox_.Put(std::make_shared<SchedulerTerminateEvent>());
+            thread_.join();
+        }
+        inbox_.ClearAlarms();
+    }
+
+    /// Ledger entries change on the caller's thread: the round thread may be the one that
+    /// waits for them. A completion is never queued (reference local.cpp:42-96).
+    void Accept(EventPtr event)
+    {
+        switch (event->Type()) {
+        case kEventProcessCreate:  ledger_.Open(event->Pid()); break;
+        case kEventProcessDestroy: ledger_.Close(event->Pid()); break;
+        case kEventOperationComplete:
+            ledger_.Done(event->Pid(), static_cast<const OperationCompleteEvent *>(event.get())->OpId());
+            return;
+        default: break;
+        }
+        inbox_.Put(std::move(event));
+    }
+
+    void SwitchTo(XPolicyType type)
+    {
+        if (type == type_) return;
+        const std::string before = GetPolicyTypeName(type_);
+        Halt();
+        Install(type);
+        // the new policy starts from "everything runs"
+        std::vector<XQueueHandle> all;
+        for (auto &entry : mirror_.View().xqueue_status) all.push_back(entry.first);
+        for (XQueueHandle h : all) mirror_.Mark(h, false);
+        Start();
+        XINFO("policy changed from %s to %s", before.c_str(), GetPolicyTypeName(type).c_str());
+    }
+
+    XPolicyType Type() const { return type_; }
+
+private:
+    void Turn()
+    {
+        std::vector<EventPtr> batch;
+        while (true) {
+            inbox_.Take(&batch);
+            bool last_round = false;
+            for (auto &event : batch) {
+                if (UNLIKELY(event->Type() == kEventSchedulerTerminate)) last_round = true;
+                else Fold(*event);
+            }
+            policy_->Sched(mirror_.View());
+            // one operation per process that has XQueues, whether or not anything changed
+            for (auto &entry : mirror_.View().process_status) {
+                const ProcessStatus &ps = *entry.second;
+                if (ps.running_xqueues.empty() && ps.suspended_xqueues.empty()) continue;
+                owner_->Execute(std::make_shared<SchedOperation>(ledger_.Issue(ps.info.pid), ps));
+            }
+            if (last_round) return;
+        }
+    }
+
+    // ---- folding one event into the mirror, one function per event type ----------------
+
+    void FoldHint(const Event &e) { policy_->RecvHint(static_cast<const HintEvent &>(e).GetHint()); }
+
+    void FoldProcessCreate(const Event &e)
+    {
+        mirror_.Process(e.Pid()).info.cmdline = static_cast<const ProcessCreateEvent &>(e).Cmdline();
+    }
+
+    void FoldProcessDestroy(const Event &e) { mirror_.ForgetProcess(e.Pid()); }
+
+    void FoldQueueConfig(const Event &e) // creation and configuration updates carry the same record
+    {
+        const auto *rec = (const XQueueConfigData *)e.Data();
+        XQueueStatus *xq = mirror_.Find(rec->handle);
+        if (xq == nullptr) xq = &mirror_.Adopt(e.Pid(), rec->handle);
+        xq->device = rec->device;
+        xq->level = rec->level;
+        xq->threshold = rec->threshold;
+        xq->batch_size = rec->batch_size;
+    }
+
+    void FoldQueueDestroy(const Event &e)
+    {
+        mirror_.ForgetQueue(static_cast<const XQueueDestroyEvent &>(e).Handle(), e.Pid());
+    }
+
+    void FoldQueueReady(const Event &e)
+    {
+        auto &ready = static_cast<const XQueueReadyEvent &>(e);
+        XQueueStatus *xq = mirror_.Find(ready.Handle());
+        if (xq == nullptr) xq = &mirror_.Adopt(e.Pid(), ready.Handle()); // ready before its creation was heard of
+        xq->ready = true;
+        xq->ready_time = ready.ReadyTime();
+    }
+
+    void FoldQueueIdle(const Event &e)
+    {
+        const XQueueHandle handle = static_cast<const XQueueIdleEvent &>(e).Handle();
+        XQueueStatus *xq = mirror_.Find(handle);
+        if (xq == nullptr) xq = &mirror_.Adopt(e.Pid(), handle);
+        xq->ready = false;
+    }
+
+    void FoldQueryOne(const Event &e)
+    {
+        auto &ask = static_cast<const XQueueQueryEvent &>(e);
+        StatusQuery *query = ask.QueryData();
+        if (const XQueueStatus *xq = mirror_.Find(ask.Handle())) mirror_.Answer(query, xq);
         query->Notify();
-        break;
     }
-    default:
-        break;
+
+    void FoldQueryAll(const Event &e)
+    {
+        StatusQuery *query = static_cast<const XQueueQueryAllEvent &>(e).QueryData();
+        mirror_.Answer(query, nullptr);
+        query->Notify();
     }
-}
 
-void LocalScheduler::Suspend(XQueueHandle handle)
-{
-    auto qit = status_.xqueue_status.find(handle);
-    if (qit == status_.xqueue_status.end() || qit->second->suspended) return;
-    qit->second->suspended = true;
+    void Fold(const Event &e)
+    {
+        using Folder = void (Rounds::*)(const Event &);
+        static const std::map<EventType, Folder> folders = {
+            { kEventHint, &Rounds::FoldHint },
+            { kEventProcessCreate, &Rounds::FoldProcessCreate },
+            { kEventProcessDestroy, &Rounds::FoldProcessDestroy },
+            { kEventXQueueCreate, &Rounds::FoldQueueConfig },
+            { kEventXQueueConfigUpdate, &Rounds::FoldQueueConfig },
+            { kEventXQueueDestroy, &Rounds::FoldQueueDestroy },
+            { kEventXQueueReady, &Rounds::FoldQueueReady },
+            { kEventXQueueIdle, &Rounds::FoldQueueIdle },
+            { kEventXQueueQuery, &Rounds::FoldQueryOne },
+            { kEventXQueueQueryAll, &Rounds::FoldQueryAll },
+        };
+        auto it = folders.find(e.Type());
+        if (it != folders.end()) (this->*(it->second))(e);
+    }
 
-    auto pit = status_.process_status.find(qit->second->pid);
-    if (pit == status_.process_status.end()) return;
-    pit->second->running_xqueues.erase(handle);
-    pit->second->suspended_xqueues.insert(handle);
-    pit->second->xqueues_to_suspend.insert(handle);
-}
+    LocalScheduler *const owner_;
+    XPolicyType type_ = kPolicyUnknown;
+    std::unique_ptr<Policy> policy_;
+    Inbox inbox_;
+    Ledger ledger_;
+    Mirror mirror_;
+    std::thread thread_;
+};
 
-void LocalScheduler::Resume(XQueueHandle handle)
-{
-    auto qit = status_.xqueue_status.find(handle);
-    if (qit == status_.xqueue_status.end() || !qit->second->suspended) return;
-    qit->second->suspended = false;
+LocalScheduler::LocalScheduler(XPolicyType type)
+    : Scheduler(kSchedulerLocal), rounds_(std::make_unique<Rounds>(this, type)) {}
 
-    auto pit = status_.process_status.find(qit->second->pid);
-    if (pit == status_.process_status.end()) return;
-    pit->second->running_xqueues.insert(handle);
-    pit->second->suspended_xqueues.erase(handle);
-    pit->second->xqueues_to_resume.insert(handle);
-}
+LocalScheduler::~LocalScheduler() { rounds_->Halt(); }
 
-void LocalScheduler::AddTimer(const system_clock::time_point tp) { timers_.push_back(tp); }
+void LocalScheduler::Run() { rounds_->Start(); }
+void LocalScheduler::Stop() { rounds_->Halt(); }
+void LocalScheduler::RecvEvent(std::shared_ptr<const Event> event) { rounds_->Accept(std::move(event)); }
+void LocalScheduler::SetPolicy(XPolicyType type) { rounds_->SwitchTo(type); }
+XPolicyType LocalScheduler::GetPolicy() const { return rounds_->Type(); }
 
 } // namespace xsched::sched

@@ -2,15 +2,17 @@
 // the other policies live in policy_extra.cpp.
 // reference sched/src/policy/{policy,hpf,lax}.cpp
 #include <map>
+#include <unordered_map>
 
 #include "xsched/utils/xassert.h"
-#include "xsched/sched/policy/extra.h"
-#include "xsched/sched/policy/hpf.h"
-#include "xsched/sched/policy/lax.h"
+#include "policy_extra.h"
 #include "xsched/sched/policy/policy.h"
 
 namespace xsched::sched
 {
+
+std::unique_ptr<Policy> MakePriorityBarPolicy();
+std::unique_ptr<Policy> MakeLaxityBarPolicy();
 
 bool PolicyAvailable(XPolicyType type)
 {
@@ -20,8 +22,8 @@ bool PolicyAvailable(XPolicyType type)
 std::unique_ptr<Policy> CreatePolicy(XPolicyType type)
 {
     switch (type) {
-    case kPolicyHighestPriorityFirst: return std::make_unique<HighestPriorityFirstPolicy>();
-    case kPolicyLaxity:               return std::make_unique<LaxityPolicy>();
+    case kPolicyHighestPriorityFirst: return MakePriorityBarPolicy();
+    case kPolicyLaxity:               return MakeLaxityBarPolicy();
     case kPolicyHeterogeneousHighestPriorityFirst: return std::make_unique<GlobalPriorityPolicy>();
     case kPolicyCPUHighestPriorityFirst:           return std::make_unique<ProcessPriorityPolicy>();
     case kPolicyUtilizationPartition:              return std::make_unique<QueueSharePolicy>();
@@ -38,113 +40,127 @@ std::unique_ptr<Policy> CreatePolicy(XPolicyType type)
     }
 }
 
-// ---- Highest Priority First (reference hpf.cpp:8-68) ------------------------
-// Pass 1: per device, the highest priority among READY queues.
-// Pass 2: every queue (ready or not) strictly below its device's maximum is
-// suspended, all others resumed. A device without a ready queue has maximum
-// PRIORITY_MIN, so nothing on it is suspended.
+// ---- the two policies of the preemptible-queue path -----------------------------------------
+// Both are "bar" policies: every XQueue has an effective priority, the bar is the highest one
+// among READY queues of a scope, and a queue below its scope's bar is suspended while every
+// other queue runs. They differ in what the effective priority is and in the scope:
+//
+//   HPF  the hinted priority (default PRIORITY_DEFAULT, clamped to the valid range);
+//        one bar per device (reference sched/src/policy/hpf.cpp:8-68)
+//   LAX  lax_prio until `laxity` us after the queue became ready (and while it is not
+//        ready), crit_prio from then on, PRIORITY_DEFAULT without a hint; ONE bar for all
+//        devices; the earliest expiry still ahead among ready hinted queues is asked for as
+//        a timer (reference sched/src/policy/lax.cpp:8-72)
 
-void HighestPriorityFirstPolicy::Sched(const Status &status)
+namespace
 {
-    std::map<XDevice, Priority> top;
-    for (auto &entry : status.xqueue_status) {
-        const XQueueStatus &xq = *entry.second;
-        if (!xq.ready) continue;
-        const Priority prio = PriorityOf(xq.handle);
-        auto it = top.find(xq.device);
-        if (it == top.end()) top.emplace(xq.device, prio);
-        else if (prio > it->second) it->second = prio;
+
+/// Highest effective priority among ready queues, per scope key; a scope without a ready
+/// queue has no entry and its bar is PRIORITY_MIN (nothing below it).
+class Bars
+{
+public:
+    void Raise(uint64_t scope, Priority prio)
+    {
+        auto [it, fresh] = top_.emplace(scope, prio);
+        if (!fresh && prio > it->second) it->second = prio;
     }
-
-    for (auto &entry : status.xqueue_status) {
-        const XQueueStatus &xq = *entry.second;
-        auto it = top.find(xq.device);
-        const Priority bar = it == top.end() ? (Priority)PRIORITY_MIN : it->second;
-        if (PriorityOf(xq.handle) < bar) this->Suspend(xq.handle);
-        else this->Resume(xq.handle);
+    Priority Of(uint64_t scope) const
+    {
+        auto it = top_.find(scope);
+        return it == top_.end() ? (Priority)PRIORITY_MIN : it->second;
     }
-}
+private:
+    std::map<uint64_t, Priority> top_;
+};
 
-void HighestPriorityFirstPolicy::RecvHint(std::shared_ptr<const Hint> hint)
+class PriorityBarPolicy final : public Policy
 {
-    if (hint->Type() != kHintTypePriority) return;
-    auto h = std::dynamic_pointer_cast<const PriorityHint>(hint);
-    XASSERT(h != nullptr, "hint type mismatch");
+public:
+    PriorityBarPolicy(): Policy(kPolicyHighestPriorityFirst) {}
 
-    Priority prio = h->Prio();
-    if (prio < PRIORITY_MIN) prio = PRIORITY_MIN;
-    if (prio > PRIORITY_MAX) prio = PRIORITY_MAX;
-    if (prio != h->Prio()) {
-        XWARN("priority %d of XQueue 0x" FMT_64X " clamped to %d", h->Prio(), h->Handle(), prio);
-    }
-    priorities_[h->Handle()] = prio;
-}
-
-Priority HighestPriorityFirstPolicy::PriorityOf(XQueueHandle handle) const
-{
-    auto it = priorities_.find(handle);
-    return it == priorities_.end() ? (Priority)PRIORITY_DEFAULT : it->second;
-}
-
-// ---- Laxity (reference lax.cpp:8-72) ----------------------------------------
-// expiry(q)    = ready_time(q) + laxity(q)
-// effective(q) = lax_prio while q is not ready or now < expiry(q), else crit_prio;
-//                PRIORITY_DEFAULT for queues without a hint
-// bar          = max effective priority over READY queues (PRIORITY_MIN if none)
-// Queues below the bar are suspended. The earliest expiry still in the future
-// among ready hinted queues becomes a timer so the decision is re-evaluated then.
-
-void LaxityPolicy::Sched(const Status &status)
-{
-    const TimePoint now = test_now_us_ != 0
-        ? TimePoint(std::chrono::microseconds(test_now_us_))
-        : std::chrono::system_clock::now();
-
-    Priority bar = PRIORITY_MIN;
-    bool have_timer = false;
-    TimePoint next_expiry = (TimePoint::max)();
-
-    for (auto &entry : status.xqueue_status) {
-        const XQueueStatus &xq = *entry.second;
-        if (!xq.ready) continue;
-
-        auto it = laxity_infos_.find(xq.handle);
-        if (it == laxity_infos_.end()) {
-            if (PRIORITY_DEFAULT > bar) bar = PRIORITY_DEFAULT;
-            continue;
+    void Sched(const Status &status) override
+    {
+        Bars bars;
+        for (auto &entry : status.xqueue_status) {
+            if (entry.second->ready) bars.Raise(entry.second->device, Hinted(entry.first));
         }
-        const TimePoint expiry = xq.ready_time + std::chrono::microseconds(it->second.lax);
-        const Priority prio = now < expiry ? it->second.lax_prio : it->second.crit_prio;
-        if (prio > bar) bar = prio;
-        if (now < expiry && expiry < next_expiry) {
-            next_expiry = expiry;
-            have_timer = true;
+        for (auto &entry : status.xqueue_status) {
+            if (Hinted(entry.first) < bars.Of(entry.second->device)) Suspend(entry.first);
+            else Resume(entry.first);
         }
     }
 
-    for (auto &entry : status.xqueue_status) {
-        const XQueueStatus &xq = *entry.second;
-        Priority prio = PRIORITY_DEFAULT;
-        auto it = laxity_infos_.find(xq.handle);
-        if (it != laxity_infos_.end()) {
+    void RecvHint(std::shared_ptr<const Hint> hint) override
+    {
+        if (hint->Type() != kHintTypePriority) return;
+        auto *h = static_cast<const PriorityHint *>(hint.get());
+        const Priority asked = h->Prio();
+        const Priority kept = asked < PRIORITY_MIN ? (Priority)PRIORITY_MIN
+                            : asked > PRIORITY_MAX ? (Priority)PRIORITY_MAX : asked;
+        if (kept != asked) XWARN("priority %d of XQueue 0x" FMT_64X " clamped to %d", asked, h->Handle(), kept);
+        hinted_[h->Handle()] = kept;
+    }
+
+private:
+    Priority Hinted(XQueueHandle handle) const
+    {
+        auto it = hinted_.find(handle);
+        return it == hinted_.end() ? (Priority)PRIORITY_DEFAULT : it->second;
+    }
+    std::unordered_map<XQueueHandle, Priority> hinted_;
+};
+
+class LaxityBarPolicy final : public Policy
+{
+public:
+    LaxityBarPolicy(): Policy(kPolicyLaxity) {}
+
+    void Sched(const Status &status) override
+    {
+        const TimePoint now = std::chrono::system_clock::now();
+        Bars bars; // one scope
+        bool alarm = false;
+        TimePoint earliest = (TimePoint::max)();
+        for (auto &entry : status.xqueue_status) {
+            const XQueueStatus &xq = *entry.second;
+            if (!xq.ready) continue;
+            bars.Raise(0, Effective(xq, now));
+            auto it = terms_.find(xq.handle);
+            if (it == terms_.end()) continue;
             const TimePoint expiry = xq.ready_time + std::chrono::microseconds(it->second.lax);
-            prio = (!xq.ready || now < expiry) ? it->second.lax_prio : it->second.crit_prio;
+            if (now < expiry && expiry < earliest) { earliest = expiry; alarm = true; }
         }
-        if (prio < bar) this->Suspend(xq.handle);
-        else this->Resume(xq.handle);
+        for (auto &entry : status.xqueue_status) {
+            if (Effective(*entry.second, now) < bars.Of(0)) Suspend(entry.first);
+            else Resume(entry.first);
+        }
+        if (alarm) AddTimer(earliest);
     }
 
-    if (have_timer) this->AddTimer(next_expiry);
-}
+    void RecvHint(std::shared_ptr<const Hint> hint) override
+    {
+        if (hint->Type() != kHintTypeLaxity) return;
+        auto *h = static_cast<const LaxityHint *>(hint.get());
+        terms_[h->Handle()] = Terms { h->Lax() < 0 ? (Laxity)NO_LAXITY : h->Lax(), h->LaxPrio(), h->CritPrio() };
+    }
 
-void LaxityPolicy::RecvHint(std::shared_ptr<const Hint> hint)
-{
-    if (hint->Type() != kHintTypeLaxity) return;
-    auto h = std::dynamic_pointer_cast<const LaxityHint>(hint);
-    XASSERT(h != nullptr, "hint type mismatch");
-    laxity_infos_[h->Handle()] = LaxityInfo {
-        h->Lax() < 0 ? (Laxity)NO_LAXITY : h->Lax(), h->LaxPrio(), h->CritPrio()
-    };
-}
+private:
+    struct Terms { Laxity lax; Priority relaxed; Priority critical; };
+
+    Priority Effective(const XQueueStatus &xq, TimePoint now) const
+    {
+        auto it = terms_.find(xq.handle);
+        if (it == terms_.end()) return PRIORITY_DEFAULT;
+        const TimePoint expiry = xq.ready_time + std::chrono::microseconds(it->second.lax);
+        return (!xq.ready || now < expiry) ? it->second.relaxed : it->second.critical;
+    }
+    std::unordered_map<XQueueHandle, Terms> terms_;
+};
+
+} // namespace
+
+std::unique_ptr<Policy> MakePriorityBarPolicy() { return std::make_unique<PriorityBarPolicy>(); }
+std::unique_ptr<Policy> MakeLaxityBarPolicy() { return std::make_unique<LaxityBarPolicy>(); }
 
 } // namespace xsched::sched

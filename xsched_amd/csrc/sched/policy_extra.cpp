@@ -11,7 +11,7 @@
 
 #include "xsched/utils/log.h"
 #include "xsched/utils/xassert.h"
-#include "xsched/sched/policy/extra.h"
+#include "policy_extra.h"
 
 using namespace std::chrono;
 

@@ -23,6 +23,7 @@
 #include "xsched/protocol/def.h"
 #include "xsched/protocol/names.h"
 #include "xsched/sched/ipc/channel.h"
+#include "xsched/sched/policy/policy.h"
 #include "xsched/sched/scheduler/local.h"
 
 using namespace xsched::sched;
