@@ -1,18 +1,24 @@
 #!/usr/bin/env python3
 """Headline benchmark: foreground latency under a saturating background on one MI355X.
 
-Default workload (`--config 2`): a background XQueue streams fp32
-AXPY y = 0.5*x + y over 2^28 elements back to back (Level-1, HPF policy, priority 1); a
-foreground XQueue submits the same kernel over 2^22 elements every 20 ms (priority 2). One
-"step" is one foreground command under contention (submit -> XQueueWaitAll returns).
+Default workload (`--config 2`): a background XQueue streams fp32 AXPY y = 0.5*x + y over
+2^28 elements back to back (Level-1, HPF policy, priority 1); a foreground XQueue submits the
+same kernel over 2^22 elements every 20 ms (priority 2). One "step" is one foreground command
+under contention (submit -> XQueueWaitAll returns); `--warmup` untimed steps, then exactly
+`--steps` timed ones give `ms_per_step`.
 
-Prints ONE JSON line. `value` is the foreground p99 latency under contention in
-microseconds (percentile rule sorted[floor(p*n)], as XSched's own DataProcessor). The same
-line carries the background kernel's achieved rate against the MI355X peak (`roofline`),
-the guard overhead, the Level-2 preemption latency, and a CPU baseline of the same workload
-(`cpu_baseline`).
+Prints ONE JSON line. `value` is the foreground p99 latency under contention in microseconds
+(percentile rule sorted[floor(p*n)], as XSched's own DataProcessor) over a block of FIXED size
+(400 samples, whatever --steps says: the p99 of 20 samples would be their maximum). The line
+also carries: the background kernel's achieved rate against the MI355X peak (`roofline`), where
+a foreground command's latency goes and the plain-HIP floor beside it (`fg_latency_us`), a
+bit-exact check of the buffers the timed phases produced (`bit_exact`), guard overhead and
+Level-2 preemption latency, compact blocks for the other four configurations (`others`), and a
+CPU baseline of the same workload (`cpu_baseline`).
 
-The other single-GPU configurations print a line of the same shape:
+Each configuration also prints a full line of its own:
+    --config 1   CPU only, host adapter: two XQueues, L1, HPF, window 8/4; background streams of
+                 1000 fp32 vector additions over 2^20 elements, foreground 2^16 every 10 ms
     --config 3   Level-2 guarded bf16 GEMM 8192^3 back to back, foreground GEMM 1024^3
                  every 5 ms (MFMA roofline, guard on/off, preemption latency)
     --config 4   laxity policy: 4 background XQueues histogramming 2^26 Zipf keys,
@@ -20,7 +26,7 @@ The other single-GPU configurations print a line of the same shape:
     --config 5   16 XQueues, priorities 0-15, cycling AXPY 2^24 / GEMM 2048^3 / histogram
                  2^24, exponential arrivals (mean 5 ms, seed 7), HPF, Level-2
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1|2|3|4|5] [--quick]
 """
 import argparse
 import json
@@ -99,24 +105,37 @@ def preempt_block(H, kind, n, quick):
             "level2_stats": st2}
 
 
-def contended_run(H, cfg, steps, warmup, bg_warm=8, bg_cmds=40):
-    """fg alone -> bg alone -> contended (warm-up, then exactly `steps` timed steps)."""
+LATENCY_BLOCK = 400   # foreground samples per phase of the fixed-size latency block
+BREAKDOWN_SAMPLES = 200
+
+
+def contended_run(H, cfg, steps, warmup, bg_warm=8, bg_cmds=40, block=0, keep=None):
+    """fg alone -> bg alone -> contended. With `block` > 0 the latencies come from phases of
+    that many samples (after `warmup` untimed ones) and the `steps` timed steps are a phase of
+    their own; otherwise (the per-configuration lines) the timed steps are the samples.
+    `keep`, when given, is called with the live harness before it is torn down."""
     with H.Bench(cfg) as b:
-        alone, _ = b.fg_alone(steps + warmup)
+        n_alone = (block or steps) + warmup
+        alone, _ = b.fg_alone(n_alone)
         b.bg_alone(bg_warm)
         alone_res = b.bg_alone(bg_cmds)
         bg_alone_ms = alone_res.bg_stream_ms / alone_res.bg_stream_cmds
         if warmup:
             b.contended(warmup)
         t0 = time.perf_counter()
-        cont, res = b.contended(steps)
+        timed, timed_res = b.contended(steps)
         wall = time.perf_counter() - t0
-        return {"fg_alone": alone[warmup:], "fg_contended": cont, "wall_s": wall,
-                "bg_alone_ms": bg_alone_ms,
-                "bg_alone_cmds": int(alone_res.bg_commands), "bg_alone_elapsed": alone_res.elapsed_s,
-                "bg_cont_ms": (res.bg_stream_ms / res.bg_stream_cmds) if res.bg_stream_cmds else None,
-                "bg_cont_cmds": int(res.bg_commands), "bg_cont_elapsed": res.elapsed_s,
-                "deadline_miss": int(res.fg_deadline_miss), "stats": list(res.stats)}
+        cont, res = (b.contended(block) if block else (timed, timed_res))
+        out = {"fg_alone": alone[warmup:], "fg_contended": cont, "fg_timed_steps": timed, "wall_s": wall,
+               "bg_alone_ms": bg_alone_ms,
+               "bg_alone_cmds": int(alone_res.bg_commands), "bg_alone_elapsed": alone_res.elapsed_s,
+               "bg_cont_ms": (res.bg_stream_ms / res.bg_stream_cmds) if res.bg_stream_cmds else None,
+               "bg_cont_launches": int(res.bg_stream_cmds),
+               "bg_cont_cmds": int(res.bg_commands), "bg_cont_elapsed": res.elapsed_s,
+               "deadline_miss": int(res.fg_deadline_miss), "stats": list(res.stats)}
+        if keep is not None:
+            out["kept"] = keep(b)
+        return out
 
 
 def recorded_traffic(summary, applies=True):
@@ -132,14 +151,14 @@ def recorded_traffic(summary, applies=True):
     return None
 
 
-def cpu_baseline(seconds_budget=15.0):
-    """The same workload on host cores: XSched's own host loop where its build is present
-    (kind "reference"), else the compact port; bounded sample."""
+def cpu_baseline(config=2):
+    """The same workload on host cores, on XSched's own host loop compiled from the reference
+    sources (oracle/_ref, kind "reference"); bounded sample."""
     try:
         from oracle import cpu_baseline as cb
-        return cb.run_config2_sample(seconds_budget, samples=300)
+        return cb.run_config1_sample(150) if config == 1 else cb.run_config2_sample(15.0, samples=300)
     except Exception as e:  # checker libraries not built
-        return {"value": None, "unit": "us", "cores": 0, "kind": "port", "sample": f"unavailable: {e}"}
+        return {"value": None, "unit": "us", "cores": 0, "kind": "reference", "sample": f"unavailable: {e}"}
 
 
 def base_line(a, value, wall_s, workload, extra_cfg):
@@ -151,29 +170,168 @@ def base_line(a, value, wall_s, workload, extra_cfg):
             "config": cfg}
 
 
+# ---- bit-exact checks against the CPU oracle (the checker; nothing timed runs through it) ----
+
+def axpy_slices(n, pieces=8, length=1 << 12):
+    """Slices spread over [0, n): the head, the tail and evenly spaced ones in between."""
+    length = min(length, n)
+    starts = sorted({0, n - length} | {((n - length) * k // (pieces - 1)) // 4 * 4 for k in range(pieces)})
+    return [(s0, length) for s0 in starts]
+
+
+def check_axpy_buffer(b, which, q, lane_id, n, seed=0, full=False):
+    """Compares a result buffer of the harness, bit for bit, with `applied` oracle
+    applications of y = fma(0.5, x, y) to the seeded inputs: the whole buffer when `full`,
+    else slices (an application count in the thousands makes the whole buffer a matter of
+    minutes on the host)."""
+    import numpy as np
+    import oracle
+    s_x, s_y = lane_id * 4, lane_id * 4 + 1
+    checked = 0
+    applied = None
+    for first, count in ([(0, n)] if full else axpy_slices(n)):
+        got, applied = b.read(which, q, first, count, np.float32)
+        want = oracle.axpy(0.5, oracle.fill_uniform(seed, s_x, first, count),
+                           oracle.fill_uniform(seed, s_y, first, count), times=applied)
+        if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+            return {"ok": False, "applied": applied, "first_bad_slice": first}
+        checked += count
+    return {"ok": True, "applied": applied, "elements_checked": checked}
+
+
+def full_buffer_check(H, bg_n, fg_n):
+    """Fresh queues at the full sizes. Level 1, plain kernels: two background and three
+    foreground commands, then EVERY element of both buffers against the oracle. Level 2,
+    guarded kernels: the background streams through three suspend / resume rounds (a hundred
+    or more commands, flushed and replayed), then slices of its buffer against as many oracle
+    applications as commands were applied."""
+    cfg = H.Config(H.HPF, 1, H.spec(H.AXPY, bg_n, 0, 1, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(H.AXPY, fg_n, 0, 1, 8, 4, 2, period_us=2000), 2, 0)
+    with H.Bench(cfg) as b:
+        b.bg_alone(2)
+        b.fg_alone(3)
+        out = {"level1_plain_every_element": {"bg": check_axpy_buffer(b, 0, 0, 1, bg_n, full=True),
+                                              "fg": check_axpy_buffer(b, 1, 0, 0, fg_n, full=True)}}
+    cfg = H.Config(H.HPF, 1, H.spec(H.AXPY, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 1),
+                   H.spec(H.AXPY, fg_n, 1, 2, 8, 4, 2, period_us=2000), 8, 0)
+    with H.Bench(cfg) as b:
+        _, _, res = b.preempt(3)
+        out["level2_guarded_preempted_slices"] = {"bg": dict(check_axpy_buffer(b, 0, 0, 1, bg_n),
+                                                             replayed_launches=int(res.stats[1]))}
+    return out
+
+
+def breakdown_block(b, H, samples):
+    """Where a foreground command's latency goes (see bench.h), alone and contended, through the
+    XQueue, through the adapter alone, and for plain HIP launches (the floor)."""
+    out = {}
+    for name, mode in (("xqueue", 0), ("adapter_only", 1), ("plain_hip_floor", 2)):
+        for cont in (False, True):
+            r = b.fg_breakdown(samples, mode, cont)
+            out[name + ("_contended" if cont else "_alone")] = {
+                k: {"p50": H.pct(v[5:], 0.5), "p99": H.pct(v[5:], 0.99)} for k, v in r.items()}
+    out["samples"] = samples - 5
+    out["note"] = ("submit = host time to hand over (two timing-event records + the kernel), device = between "
+                   "the two events, wait = until the host knows, total = submit + wait; the XQueue rows carry "
+                   "two extra event-record commands per sample, the fixed-size block above does not")
+    return out
+
+
 # ---- configurations ------------------------------------------------------------------
+
+def config1(a):
+    """CPU only: the host adapter (libhalhost.so), no GPU and no torch."""
+    import ctypes
+    import numpy as np
+    import oracle
+    import xsched_amd as xs
+    h = xs.halhost()
+    n_bg, n_fg, samples = 1 << 20, 1 << 16, (100 if a.quick else LATENCY_BLOCK)
+
+    class Cfg(ctypes.Structure):
+        _fields_ = [("bg_n", ctypes.c_uint64), ("fg_n", ctypes.c_uint64), ("bg_burst", ctypes.c_int32),
+                    ("threshold", ctypes.c_int32), ("batch", ctypes.c_int32), ("samples", ctypes.c_int32),
+                    ("period_us", ctypes.c_int64)]
+
+    class Res(ctypes.Structure):
+        _fields_ = [("alone_s", ctypes.c_double), ("contended_s", ctypes.c_double),
+                    ("bg_commands", ctypes.c_uint64), ("fg_commands", ctypes.c_uint64)]
+
+    def filled(n, stream):
+        arr = np.empty(n, np.float32)
+        h.HostBenchFillUniform(arr.ctypes.data, 0, n, 0, stream)
+        return arr
+    bg_a, bg_b, fg_a, fg_b = filled(n_bg, 4), filled(n_bg, 5), filled(n_fg, 0), filled(n_fg, 1)
+    bg_c, fg_c = np.zeros(n_bg, np.float32), np.zeros(n_fg, np.float32)
+    cfg, res = Cfg(n_bg, n_fg, 1000, 8, 4, samples, 10000), Res()
+    alone, cont = (ctypes.c_double * samples)(), (ctypes.c_double * samples)()
+    t0 = time.perf_counter()
+    xs.check(h.HostBenchRunVecAdd(ctypes.byref(cfg), bg_a.ctypes.data, bg_b.ctypes.data, bg_c.ctypes.data,
+                                  fg_a.ctypes.data, fg_b.ctypes.data, fg_c.ctypes.data, alone, cont,
+                                  ctypes.byref(res)))
+    wall = time.perf_counter() - t0
+    alone, cont = list(alone)[5:], list(cont)[5:]
+    # the checker: seeded inputs and sums recomputed by the oracle
+    exact = (np.array_equal(bg_a, oracle.fill_uniform(0, 4, 0, n_bg)) and np.array_equal(fg_b, oracle.fill_uniform(0, 1, 0, n_fg))
+             and np.array_equal(bg_c.view(np.uint32), oracle.vecadd(bg_a, bg_b).view(np.uint32))
+             and np.array_equal(fg_c.view(np.uint32), oracle.vecadd(fg_a, fg_b).view(np.uint32)))
+    pct = lambda v, p: sorted(v)[min(int(p * len(v)), len(v) - 1)]
+    line = {"metric": "fg_p99_latency_us_under_contention", "value": pct(cont, 0.99), "unit": "us", "n_gpus": 0,
+            "steps": len(cont), "warmup": 5, "ms_per_step": res.contended_s * 1e3 / samples,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "data": "synthetic", "dtype": "f32",
+            "config": {"workload": "cfg1: host adapter, 2 XQueues, L1 HPF, window 8/4, bg streams of 1000 fp32 vector "
+                                   "additions 2^20, fg 2^16 every 10 ms", "percentile_rule": "sorted[floor(p*n)]"},
+            "fg_latency_us": {"alone_p50": pct(alone, 0.5), "alone_p99": pct(alone, 0.99),
+                              "contended_p50": pct(cont, 0.5), "contended_p99": pct(cont, 0.99),
+                              "p99_ratio": pct(cont, 0.99) / pct(alone, 0.99), "samples": len(cont)},
+            "bg": {"commands_while_contended": int(res.bg_commands),
+                   "host_GBs": 12.0 * n_bg * res.bg_commands / res.contended_s / 1e9},
+            "bit_exact": bool(exact), "wall_s": wall,
+            "roofline": {"bound": "hbm", "achieved": 12.0 * n_bg * res.bg_commands / res.contended_s / 1e9, "peak": None,
+                         "unit": "GB/s", "frac": None, "traffic": None,
+                         "note": "host DRAM, one executor thread: informational, no device kernel in this configuration"}}
+    return line
+
 
 def config2(H, a):
     bg_n, fg_n = 1 << a.bg_log2, 1 << a.fg_log2
     cfg = H.Config(H.HPF, 1, H.spec(H.AXPY, bg_n, 1, 1, BG_THRESHOLD, BG_BATCH, 1),
                    H.spec(H.AXPY, fg_n, 0, 1, 8, 4, 2, period_us=20000), 64, 0)
-    r = contended_run(H, cfg, a.steps, a.warmup)
+    block = 100 if a.quick else LATENCY_BLOCK
+
+    def after(b):
+        kept = {"breakdown": None if a.quick else breakdown_block(b, H, BREAKDOWN_SAMPLES)}
+        kept["bit_exact_slices"] = {"bg": check_axpy_buffer(b, 0, 0, 1, bg_n), "fg": check_axpy_buffer(b, 1, 0, 0, fg_n)}
+        return kept
+    r = contended_run(H, cfg, a.steps, a.warmup, block=block, keep=after)
     fg = fg_summary(H, r["fg_alone"], r["fg_contended"])
+    fg["samples_per_phase"] = block
+    fg["timed_steps"] = {"n": a.steps, "p50": H.pct(r["fg_timed_steps"], 0.5), "max": max(r["fg_timed_steps"])}
     per_launch_ms = r["bg_cont_ms"] or r["bg_alone_ms"]
     achieved = axpy_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
     line = base_line(a, fg["contended_p99"], r["wall_s"],
                      "cfg2: L1 HPF, bg AXPY 2^%d back-to-back, fg AXPY 2^%d every 20 ms" % (a.bg_log2, a.fg_log2),
-                     {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
+                     {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4,
+                      "value_from": "p99 of %d contended foreground samples (fixed-size block, not the --steps region)" % block})
     line["dtype"] = "f32"
     line["fg_latency_us"] = fg
+    if r["kept"]["breakdown"]:
+        line["fg_latency_us"]["breakdown"] = r["kept"]["breakdown"]
     line["bg"] = {"alone_GBs": axpy_bytes(bg_n) / r["bg_alone_ms"] / 1e6,
                   "contended_GBs": axpy_bytes(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e9,
-                  "commands_in_timed_region": r["bg_cont_cmds"]}
+                  "commands_in_latency_block": r["bg_cont_cmds"]}
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("axpy_2p28_hbm_traffic.md", bg_n == 1 << 28),
                         "kernel": "AxpyPersistentKernel<3, false>" if bg_n >= 1 << 23 else "AxpyVec4Kernel<false, 4>",
                         "algorithmic_bytes_per_launch": axpy_bytes(bg_n),
-                        "avg_launch_ms": per_launch_ms}
+                        "avg_launch_ms": per_launch_ms, "launches_timed": r["bg_cont_launches"],
+                        "timed_with": "HIP events on the background stream around the contended latency block"}
+    slices = r["kept"]["bit_exact_slices"]
+    line["bit_exact"] = {"after_timed_phases_slices": slices}
+    if not a.quick:
+        line["bit_exact"]["fresh_run_every_element"] = full_buffer_check(H, bg_n, fg_n)
+    line["bit_exact"]["all_ok"] = all(
+        v["ok"] for grp in ([slices] + list(line["bit_exact"].get("fresh_run_every_element", {}).values())) for v in grp.values())
     if not a.quick:
         ms_plain = bg_ms_per_launch(H, H.AXPY, bg_n, 1, 0)
         ms_guard = bg_ms_per_launch(H, H.AXPY, bg_n, 1, 2)
@@ -184,24 +342,11 @@ def config2(H, a):
                          "guard_overhead_frac": 1.0 - ms_plain / ms_guard,
                          "level2_overhead_frac": 1.0 - ms_plain / ms_l2}
         line["preempt_us"] = preempt_block(H, H.AXPY, bg_n, False)
-        # For comparison: guarded launches on the plain kernel's grid (one wave per chunk,
-        # guard at work-group entry) instead of the two long-lived waves per CU.
-        os.environ["XSCHED_HIP_AXPY_GRID"] = "chunk"
-        try:
-            ms_cg = bg_ms_per_launch(H, H.AXPY, bg_n, 2, 1)
-            sus, res, _ = preempt_latency(H, H.AXPY, bg_n, 2, 200)
-            dev = device_drain(H, H.AXPY, bg_n, 2, 200)
-        finally:
-            del os.environ["XSCHED_HIP_AXPY_GRID"]
-        line["chunk_grid_variant"] = {
-            "level2_device_drain_p50": H.pct(dev, 0.5), "level2_device_drain_p99": H.pct(dev, 0.99),
-            "level2_GBs": axpy_bytes(bg_n) / ms_cg / 1e6, "level2_overhead_frac": 1.0 - ms_plain / ms_cg,
-            "level2_suspend_sync_p50": H.pct(sus, 0.5), "level2_suspend_sync_p99": H.pct(sus, 0.99),
-            "level2_resume_p50": H.pct(res, 0.5), "level2_resume_p99": H.pct(res, 0.99)}
     return line
 
 
 def config3(H, a):
+    compact = getattr(a, "compact", False)
     bg_n, fg_n = 8192, 1024
     cfg = H.Config(H.HPF, 1, H.spec(H.GEMM, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 1),
                    H.spec(H.GEMM, fg_n, 0, 1, 8, 4, 2, period_us=5000), 64, 0)
@@ -221,13 +366,14 @@ def config3(H, a):
                         "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": recorded_traffic("gemm_8192_hbm_traffic.md"), "kernel": "GemmBf16Kernel",
                         "algorithmic_flops_per_launch": gemm_flops(bg_n), "avg_launch_ms": per_launch_ms}
     if not a.quick:
-        # Seven alternating rounds of 12 launches per form. The clock under this load moves by a
+        # Seven (five in the compact block) alternating rounds of 12 launches per form. The clock under this load moves by a
         # few percent within seconds, more than the guard costs: the overheads are medians of
         # the per-round ratios (forms measured within a second of each other), the rates are
         # medians of each form.
         rounds = [(bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 12, 4), bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 12, 4),
-                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 12, 4)) for _ in range(7)]
-        ms_plain, ms_guard, ms_l2 = (sorted(r[i] for r in rounds)[3] for i in range(3))
+                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 12, 4)) for _ in range(5 if compact else 7)]
+        mid = len(rounds) // 2
+        ms_plain, ms_guard, ms_l2 = (sorted(r[i] for r in rounds)[mid] for i in range(3))
         guard_frac = sorted(1.0 - r[0] / r[1] for r in rounds)
         l2_frac = sorted(1.0 - r[0] / r[2] for r in rounds)
 
@@ -236,17 +382,18 @@ def config3(H, a):
         line["guard"] = {"plain_TFLOPs": tf(ms_plain), "guarded_TFLOPs": tf(ms_guard), "level2_TFLOPs": tf(ms_l2),
                          "plain_mfma_util": tf(ms_plain) / MFMA_BF16_PEAK_TF,
                          "guarded_mfma_util": tf(ms_guard) / MFMA_BF16_PEAK_TF,
-                         "guard_overhead_frac": guard_frac[3], "level2_overhead_frac": l2_frac[3],
+                         "guard_overhead_frac": guard_frac[mid], "level2_overhead_frac": l2_frac[mid],
                          "guard_overhead_frac_min_max": [guard_frac[0], guard_frac[-1]],
                          "level2_overhead_frac_min_max": [l2_frac[0], l2_frac[-1]],
                          "rounds": len(rounds), "launches_per_round_and_form": 12}
-        line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, False)
+        line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, compact)
     return line
 
 
 def config4(H, a):
+    compact = getattr(a, "compact", False)
     bg_n, fg_n, deadline = 1 << 26, 1 << 20, 1000
-    laxities = [300] if a.quick else [0, 300, 600, 900]
+    laxities = [300] if (a.quick or compact) else [0, 300, 600, 900]
     runs = {}
     for lax in laxities:
         # Background queues run at constant priority 0. The foreground runs beside them at
@@ -262,8 +409,8 @@ def config4(H, a):
     # Five alternating rounds of 120 commands, the median of each form: a single round moves
     # by a microsecond with where the buffers of that round happen to lie.
     rounds = [(bg_ms_per_launch(H, H.HIST, bg_n, 2, 1, 120, 20),
-               None if a.quick else bg_ms_per_launch(H, H.HIST, bg_n, 1, 0, 120, 20)) for _ in range(5)]
-    per_launch_ms = sorted(r[0] for r in rounds)[2]
+               None if a.quick else bg_ms_per_launch(H, H.HIST, bg_n, 1, 0, 120, 20)) for _ in range(3 if compact else 5)]
+    per_launch_ms = sorted(r[0] for r in rounds)[len(rounds) // 2]
     achieved = hist_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
     line = base_line(a, fg["contended_p99"], head["wall_s"],
                      "cfg4: L2 LAX, 4 bg XQueues histogram 2^26 Zipf(1.1) keys, fg 2^20 keys every 2 ms, "
@@ -288,7 +435,7 @@ def config4(H, a):
                         "note": "one queue streaming guarded histogram commands back to back; a command is the "
                                 "counting kernel followed by the merge kernel, avg_launch_ms covers both"}
     if not a.quick:
-        ms_plain = sorted(r[1] for r in rounds)[2]
+        ms_plain = sorted(r[1] for r in rounds)[len(rounds) // 2]
         line["guard"] = {"plain_GBs": hist_bytes(bg_n) / ms_plain / 1e6, "level2_GBs": achieved,
                          # median of the per-round ratios (the two forms of a round run within a second)
                          "level2_overhead_frac": sorted(1.0 - r[1] / r[0] for r in rounds)[len(rounds) // 2],
@@ -301,7 +448,8 @@ def config4(H, a):
 
 def config5(H, a):
     axpy_n, gemm_n, hist_n, nq = 1 << 24, 2048, 1 << 24, 16
-    duration = min(a.steps / 100.0, 4.0)  # seconds of arrivals, ~200 commands per queue and second
+    # seconds of arrivals, ~200 commands per queue and second
+    duration = 2.0 if getattr(a, "compact", False) else max(min(a.steps / 100.0, 4.0), 1.0)
     cfg = H.StressConfig(H.HPF, nq, 2, 1, 4, 2, axpy_n, gemm_n, hist_n, 5000.0, 7)
     with H.Bench(cfg) as b:
         b.stress(0.2)  # warm-up
@@ -436,12 +584,50 @@ def transparent_preemption():
             "under_xsched_shim_daemon_level2": under}
 
 
+def compact_of(line):
+    """The figures of a configuration's full line that the default line carries."""
+    keep = {"workload": line["config"]["workload"], "fg_p99_contended_us": line["value"],
+            "fg_latency_us": {k: v for k, v in line.get("fg_latency_us", {}).items()
+                              if k in ("alone_p50", "alone_p99", "contended_p50", "contended_p99", "p99_ratio", "samples")},
+            "fg_samples": line["steps"]}
+    roof = line.get("roofline", {})
+    keep["roofline"] = {k: roof.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "avg_launch_ms", "traffic")}
+    if "guard" in line:
+        keep["guard"] = {k: v for k, v in line["guard"].items() if k.endswith("overhead_frac") or k.endswith("_min_max")}
+    if "preempt_us" in line:
+        keep["preempt_us"] = {k: v for k, v in line["preempt_us"].items()
+                              if k.startswith("level2_device_drain") or k.startswith("level2_resume") or k.startswith("level2_suspend")}
+    for k in ("deadline_miss_rate", "bit_exact"):
+        if k in line:
+            keep[k] = line[k]
+    if "per_priority_latency_us" in line:
+        keep["p99_by_priority_us"] = {k: v["p99"] for k, v in line["per_priority_latency_us"].items()}
+        keep["aggregate"] = {k: line["aggregate"][k] for k in ("commands", "hbm_frac_of_peak", "mfma_frac_of_peak")}
+    return keep
+
+
+def other_configurations(H, a):
+    """Compact blocks of configurations 1, 3, 4 and 5 for the default line (about 45 s in all:
+    200 foreground samples each, fewer overhead rounds than their own full lines)."""
+    sub = argparse.Namespace(steps=200, warmup=10, quick=False, compact=True, bg_log2=28, fg_log2=22)
+    out = {}
+    for name, run in (("cfg1", lambda: config1(argparse.Namespace(quick=True))), ("cfg3", lambda: config3(H, sub)),
+                      ("cfg4", lambda: config4(H, sub)), ("cfg5", lambda: config5(H, sub))):
+        t0 = time.perf_counter()
+        try:
+            out[name] = compact_of(run())
+        except Exception as e:  # one configuration failing must not take the headline line with it
+            out[name] = {"error": repr(e)}
+        out[name]["seconds"] = round(time.perf_counter() - t0, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--bg-log2", type=int, default=28)
     ap.add_argument("--fg-log2", type=int, default=22)
     ap.add_argument("--skip-cpu", action="store_true")
@@ -451,6 +637,16 @@ def main():
         print("bench.py measures one GPU: XQueues are per-device and this path has no "
               "cross-GPU exchange; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if a.steps < 1:
+        print("--steps must be at least 1", file=sys.stderr)
+        sys.exit(2)
+
+    if a.config == 1:
+        line = config1(a)
+        line["cpu_baseline"] = ({"value": None, "unit": "us", "cores": 0, "kind": "reference", "sample": "skipped"}
+                                if a.skip_cpu else cpu_baseline(1))
+        print(json.dumps(line))
+        return
 
     import torch  # device presence check only; the harness allocates through HIP itself
     if not torch.cuda.is_available():
@@ -460,13 +656,14 @@ def main():
 
     line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
     if a.config == 2 and not a.quick:
+        line["others"] = other_configurations(H, a)
         line["shim_launch_cost"] = shim_launch_cost()
         line["transparent_preemption"] = transparent_preemption()
     if a.config == 2 and not a.skip_cpu:
-        line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline"] = cpu_baseline(2)
     else:
-        line["cpu_baseline"] = {"value": None, "unit": "us", "cores": 0, "kind": "port",
-                                "sample": "skipped" if a.config == 2 else "measured for the headline workload only"}
+        line["cpu_baseline"] = {"value": None, "unit": "us", "cores": 0, "kind": "reference",
+                                "sample": "skipped" if a.config == 2 else "measured for the headline workload and for --config 1"}
     print(json.dumps(line))
 
 

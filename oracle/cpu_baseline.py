@@ -83,6 +83,41 @@ def run_config2_sample(seconds_budget=15.0, scale_log2=4, samples=100, which="au
     }
 
 
+def run_config1_sample(samples=150, which="reference"):
+    """The CPU-only configuration at its full size on the reference's own host loop: background
+    streams of 1000 fp32 vector additions over 2^20 elements, a 2^16-element addition every
+    10 ms in the foreground, window 8 / 4, level 1, HPF."""
+    ref_path = os.path.join(_DIR, "_ref", "libxqueue_ref.so")
+    path = ref_path if which == "reference" else os.path.join(_DIR, "libhostbench.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} missing")
+    os.environ.setdefault("XLOG_LEVEL", "ERRO")
+    fn = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL).hostbench_run_fg_bg_vecadd
+    fn.restype = c_int
+    fn.argtypes = [c_uint64, c_uint64, c_int64, c_int, c_int, c_int, c_int, POINTER(c_double), POINTER(c_double),
+                   POINTER(c_uint64), POINTER(c_double), POINTER(c_uint64)]
+    alone, cont = (c_double * samples)(), (c_double * samples)()
+    bg_cmds, secs, chk = c_uint64(), c_double(), c_uint64()
+    rc = fn(1 << 20, 1 << 16, 10000, samples, 8, 4, 1000, alone, cont, byref(bg_cmds), byref(secs), byref(chk))
+    if rc != 0:
+        raise RuntimeError(f"CPU baseline run failed with XResult {rc}")
+    alone, cont = list(alone)[5:], list(cont)[5:]
+    model, logical, usable = host_cpu()
+    return {
+        "value": _pct(cont, 0.99), "unit": "us", "cores": 7,
+        "host_cpu_model": model, "host_logical_cores": logical, "host_usable_cores": usable,
+        "kind": "reference" if which == "reference" else "shipped-host",
+        "sample": ("XSched's own XQueue core, local scheduler and HPF policy (oracle/_ref/libxqueue_ref.so) over this "
+                   "repository's host adapter: bg fp32 vector additions 2^20 in streams of 1000, fg 2^16 every 10 ms, "
+                   "window 8/4, %d fg samples; scalar single-threaded kernels; threads: 2 executors + 2 launch workers "
+                   "+ 1 scheduler + 2 submitters" % len(cont)),
+        "fg_alone_p50_us": _pct(alone, 0.5), "fg_alone_p99_us": _pct(alone, 0.99),
+        "fg_contended_p50_us": _pct(cont, 0.5), "fg_contended_p99_us": _pct(cont, 0.99),
+        "bg_GBs": 12.0 * (1 << 20) * bg_cmds.value / secs.value / 1e9 if secs.value else 0.0,
+        "fg_checksum": chk.value,
+    }
+
+
 if __name__ == "__main__":
     import json
     import sys

@@ -38,12 +38,20 @@ using Clock = std::chrono::steady_clock;
 // background window is bg_threshold / bg_batch (foreground 8 / 4). Outputs: the two latency
 // arrays (microseconds), background commands completed and seconds of the contended phase,
 // and a checksum over every 97th element of the foreground result.
-extern "C" __attribute__((visibility("default")))
-int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, int samples,
-                             int bg_threshold, int bg_batch, double *alone_us, double *contended_us,
-                             uint64_t *bg_commands, double *contended_seconds, uint64_t *checksum)
+namespace
+{
+enum class Op { kAxpy, kVecAdd };
+
+// kAxpy: y = fma(0.5, x, y) in place (the GPU headline workload scaled down);
+// kVecAdd: c = a + b into a third array (the CPU-only configuration: 1000 x 2^20 additions
+// in the background, 2^16 every 10 ms in the foreground, window 8 / 4 on both queues).
+int Run(Op op, uint64_t bg_n, uint64_t fg_n, int64_t period_us, int samples,
+        int bg_threshold, int bg_batch, int fg_threshold, int fg_batch, int bg_burst,
+        double *alone_us, double *contended_us,
+        uint64_t *bg_commands, double *contended_seconds, uint64_t *checksum)
 {
     std::vector<float> bx(bg_n), by(bg_n), fx(fg_n), fy(fg_n);
+    std::vector<float> bc(op == Op::kVecAdd ? bg_n : 0), fc(op == Op::kVecAdd ? fg_n : 0);
     oracle_fill_uniform(bx.data(), 0, bg_n, oracle_stream_key(0, 4));
     oracle_fill_uniform(by.data(), 0, bg_n, oracle_stream_key(0, 5));
     oracle_fill_uniform(fx.data(), 0, fg_n, oracle_stream_key(0, 0));
@@ -57,14 +65,16 @@ int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, in
     HB_CHECK(XQueueCreate(&bg_xq, bg_hwq, kPreemptLevelBlock, kQueueCreateFlagNone));
     HB_CHECK(XQueueCreate(&fg_xq, fg_hwq, kPreemptLevelBlock, kQueueCreateFlagNone));
     HB_CHECK(XQueueSetLaunchConfig(bg_xq, bg_threshold, bg_batch));
-    HB_CHECK(XQueueSetLaunchConfig(fg_xq, 8, 4));
+    HB_CHECK(XQueueSetLaunchConfig(fg_xq, fg_threshold, fg_batch));
     HB_CHECK(XHintPriority(bg_xq, 1));
     HB_CHECK(XHintPriority(fg_xq, 2));
 
     auto fg_once = [&]() -> double {
         HwCommandHandle cmd = 0;
         const auto t0 = Clock::now();
-        if (HostAxpyCommandCreate(&cmd, 0.5f, fx.data(), fy.data(), fg_n, 0) != kXSchedSuccess) return -1;
+        const XResult made = op == Op::kAxpy ? HostAxpyCommandCreate(&cmd, 0.5f, fx.data(), fy.data(), fg_n, 0)
+                                             : HostVecAddCommandCreate(&cmd, fx.data(), fy.data(), fc.data(), fg_n, 0);
+        if (made != kXSchedSuccess) return -1;
         if (XQueueSubmit(fg_xq, cmd) != kXSchedSuccess) return -1;
         if (XQueueWaitAll(fg_xq) != kXSchedSuccess) return -1;
         return std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
@@ -83,9 +93,11 @@ int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, in
     std::atomic<bool> stop { false };
     std::thread bg_thread([&] {
         while (!stop.load()) {
-            for (int n = 0; n < 8 && !stop.load(); ++n) {
+            for (int n = 0; n < bg_burst && !stop.load(); ++n) {
                 HwCommandHandle cmd = 0;
-                if (HostAxpyCommandCreate(&cmd, 0.5f, bx.data(), by.data(), bg_n, 0) != kXSchedSuccess) return;
+                const XResult made = op == Op::kAxpy ? HostAxpyCommandCreate(&cmd, 0.5f, bx.data(), by.data(), bg_n, 0)
+                                                     : HostVecAddCommandCreate(&cmd, bx.data(), by.data(), bc.data(), bg_n, 0);
+                if (made != kXSchedSuccess) return;
                 if (XQueueSubmit(bg_xq, cmd) != kXSchedSuccess) return;
             }
             XQueueWaitAll(bg_xq);
@@ -105,7 +117,8 @@ int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, in
     bg_thread.join();
 
     uint64_t sum = 0;
-    for (uint64_t i = 0; i < fg_n; i += 97) { uint32_t u; memcpy(&u, &fy[i], 4); sum += u; }
+    const std::vector<float> &result = op == Op::kAxpy ? fy : fc;
+    for (uint64_t i = 0; i < fg_n; i += 97) { uint32_t u; memcpy(&u, &result[i], 4); sum += u; }
     *checksum = sum;
 
     HB_CHECK(XQueueDestroy(bg_xq));
@@ -113,4 +126,26 @@ int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, in
     HB_CHECK(HwQueueDestroy(bg_hwq));
     HB_CHECK(HwQueueDestroy(fg_hwq));
     return 0;
+}
+} // namespace
+
+extern "C" __attribute__((visibility("default")))
+int hostbench_run_fg_bg_axpy(uint64_t bg_n, uint64_t fg_n, int64_t period_us, int samples,
+                             int bg_threshold, int bg_batch, double *alone_us, double *contended_us,
+                             uint64_t *bg_commands, double *contended_seconds, uint64_t *checksum)
+{
+    return Run(Op::kAxpy, bg_n, fg_n, period_us, samples, bg_threshold, bg_batch, 8, 4, 8, alone_us, contended_us,
+               bg_commands, contended_seconds, checksum);
+}
+
+// The CPU-only configuration: both queues with the window `threshold` / `batch`, the
+// background in streams of `bg_burst` commands. The checksum covers every 97th element of
+// the foreground sum a + b.
+extern "C" __attribute__((visibility("default")))
+int hostbench_run_fg_bg_vecadd(uint64_t bg_n, uint64_t fg_n, int64_t period_us, int samples,
+                               int threshold, int batch, int bg_burst, double *alone_us, double *contended_us,
+                               uint64_t *bg_commands, double *contended_seconds, uint64_t *checksum)
+{
+    return Run(Op::kVecAdd, bg_n, fg_n, period_us, samples, threshold, batch, threshold, batch, bg_burst, alone_us,
+               contended_us, bg_commands, contended_seconds, checksum);
 }

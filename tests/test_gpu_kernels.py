@@ -125,6 +125,53 @@ def test_axpy_long_arrays(xs, gpu, monkeypatch, steps, n, level, guard):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_axpy_at_the_full_size_of_the_headline_configuration(xs, gpu):
+    """2^28 elements, where the grid sits exactly on the progress map's limit of 2^18
+    work-groups, and 2^28 + 5 (the chunk doubles, the end is ragged): a plain launch at level 1,
+    then guarded launches at level 2 with a suspend / resume while they are in flight; every
+    element against the oracle."""
+    torch = gpu
+    p = xs.preempt()
+    n_big = (1 << 28) + 5
+    x_h = oracle.fill_uniform(0, 4, 0, n_big)
+    y_h = oracle.fill_uniform(0, 5, 0, n_big)
+    x = torch.from_numpy(x_h).cuda()
+
+    n = 1 << 28
+    print(f"case axpy-full n={n} plain level 1", flush=True)
+    y = torch.from_numpy(y_h[:n].copy()).cuda()
+    q = Queue(xs, torch, 1, threshold=2, batch=1)
+    q.submit(axpy_cmd(xs, 0.5, x, y, n, 0))
+    q.wait()
+    want = oracle.axpy(0.5, x_h[:n], y_h[:n], 1)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    q.close()
+
+    print(f"case axpy-full n={n} guarded level 2, suspended in flight", flush=True)
+    q = Queue(xs, torch, 2, threshold=2, batch=1)
+    q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    xs.check(p.XQueueSuspend(q.xq, xs.kQueueSuspendFlagSyncHwQueue))
+    xs.check(p.XQueueResume(q.xq, xs.kQueueResumeFlagNone))
+    q.wait()
+    want = oracle.axpy(0.5, x_h[:n], want, 2)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    stats = (ctypes.c_uint64 * 8)()
+    xs.check(xs.halhip().HipQueueGetStats(q.hwq, stats))
+    assert stats[2] == 1 and stats[3] == 1   # one deactivation, one reactivation
+    q.close()
+    del y, want
+
+    print(f"case axpy-full n={n_big} guarded level 2", flush=True)
+    y = torch.from_numpy(y_h.copy()).cuda()
+    q = Queue(xs, torch, 2, threshold=2, batch=1)
+    q.submit(axpy_cmd(xs, 0.5, x, y, n_big, 1))
+    q.wait()
+    want = oracle.axpy(0.5, x_h, y_h, 1)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    q.close()
+
+
 def test_axpy_general_alpha_and_unaligned(xs, gpu):
     """alpha whose product is inexact (one rounding: fma) and a pointer that is only
     4-byte aligned (scalar fallback kernel)."""

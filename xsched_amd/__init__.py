@@ -91,6 +91,9 @@ HALHOST_API = {
     "HostKernelCommandCreate": (XResult, [POINTER(c_uint64), HostKernelFn, c_void_p, c_uint32, c_int]),
     "HostVecAddCommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_void_p, c_void_p, c_size_t, c_int]),
     "HostAxpyCommandCreate": (XResult, [POINTER(c_uint64), c_float, c_void_p, c_void_p, c_size_t, c_int]),
+    "HostBenchFillUniform": (None, [c_void_p, c_uint64, c_uint64, c_uint64, c_uint64]),
+    "HostBenchRunVecAdd": (XResult, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     POINTER(c_double), POINTER(c_double), c_void_p]),
     "HostQueueGetStats": (XResult, [c_uint64, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
 }
 

@@ -17,6 +17,8 @@ namespace
 {
 constexpr size_t kInitialRingSlots = 256;
 constexpr int64_t kSpinMicros = 150; // a waiter polls this long before it sleeps
+constexpr int64_t kStandByMicros = 500;      // how long the launcher leaves the device to callers that launch themselves
+constexpr int64_t kStandBySliceMicros = 100; // how often it looks whether their commands have retired
 
 size_t PowerOfTwoAtLeast(size_t n)
 {
@@ -106,12 +108,15 @@ void RingXQueue::Submit(std::shared_ptr<HwCommand> hw_cmd)
             reported_ = kQueueStateReady;
             SchedAgent::SendEvent(std::make_shared<XQueueReadyEvent>(kHandle, std::chrono::system_clock::now()));
         }
+        const bool launcher_owed_nothing = owed_ == Owed::kNothing;
         owed_ = Owed::kBatchThenDrain;
         // The launcher is parked and nothing waits in the ring: launching here keeps
         // submission order, and the ring lock keeps it so against other submitters.
         const bool launched = caller_may_launch_ && parked_ && ring_count_ == 0 && TryLaunchOnCaller(hw_cmd);
         if (!launched) PushLocked(Slot::kCommand, wait_for_launch ? hw_cmd : std::move(hw_cmd));
-        wake = parked_;
+        // A launcher that already stands by for callers (see NextStep) needs no wake-up for a
+        // command that is on the device already; it looks again by itself.
+        wake = parked_ && (!launched || launcher_owed_nothing);
     }
     if (wake) ring_cv_.notify_one();
     if (wait_for_launch) hw_cmd->WaitUntil(kCommandStateInFlight);
@@ -137,6 +142,22 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
             }
         }
         out->cmd = nullptr;
+        if (owed_ != Owed::kNothing && caller_may_launch_ && stood_by_for_ != handed_over_.load(std::memory_order_acquire)) {
+            // Callers launch and wait for themselves: the launcher stands by, still parked as
+            // far as submitters are concerned, until what they launched has retired (then the
+            // waits it owes return at once), something is queued for it, or the stand-by has
+            // lasted long enough that nobody seems to be waiting. It does not ask the device
+            // meanwhile: a second thread polling the runtime slows the callers' launches.
+            const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(kStandByMicros);
+            parked_ = true;
+            while (ring_count_ == 0 && retired_.load(std::memory_order_acquire) < handed_over_.load(std::memory_order_acquire) &&
+                   std::chrono::steady_clock::now() < until) {
+                ring_cv_.wait_for(g, std::chrono::microseconds(kStandBySliceMicros));
+            }
+            parked_ = false;
+            stood_by_for_ = handed_over_.load(std::memory_order_acquire);
+            if (ring_count_ != 0) continue;
+        }
         if (owed_ == Owed::kBatchThenDrain) { owed_ = Owed::kDrain; return Step::kBatch; }
         if (owed_ == Owed::kDrain) { owed_ = Owed::kNothing; return Step::kDrain; }
         if (reported_ == kQueueStateReady) {
@@ -185,10 +206,15 @@ int64_t RingXQueue::RequestDrain(std::shared_ptr<XCommand> marker)
         Guard g(ring_mu_);
         if (reported_ == kQueueStateIdle) return -1;
         ticket = next_idx_.load(std::memory_order_acquire) - 1;
+        // With everything launched already and a caller that may wait for the device itself,
+        // nothing is queued and nobody is woken: the launcher's own drain (owed since the
+        // last submission) reports Idle afterwards.
+        const bool caller_drains = marker == nullptr && caller_may_launch_ && ring_count_ == 0 &&
+                                   handed_over_.load(std::memory_order_acquire) >= ticket;
         // A drain that already closes the ring (queued, or the launcher's own) covers
         // everything submitted so far (command_buffer.cpp:127-155); a marker object always
         // gets a slot of its own, it has to be completed by somebody.
-        if (marker != nullptr || owed_ != Owed::kNothing) {
+        if (!caller_drains && (marker != nullptr || owed_ != Owed::kNothing)) {
             PushLocked(Slot::kDrain, std::move(marker));
             owed_ = Owed::kNothing;
             wake = parked_;
