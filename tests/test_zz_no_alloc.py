@@ -32,9 +32,9 @@ def test_no_alloc_histogram_matches_the_command_and_the_oracle(xs, gpu):
     torch = gpu
     h = xs.halhip()
     stream = torch.cuda.Stream()
-    # first call: the largest input the entry point takes with ragged end (2^25 - 5 keys, Zipf);
+    # first call: the largest input the entry point takes with ragged end (2^26 - 5 keys, Zipf);
     # second call: a smaller one with uniform keys over fewer bins, on the same stream
-    cases = [((1 << 25) - 5, N_BINS, "zipf"), ((1 << 20) + 3, 1000, "uniform")]
+    cases = [((1 << 26) - 5, N_BINS, "zipf"), ((1 << 20) + 3, 1000, "uniform")]
     inputs = []
     for n, n_bins, kind in cases:
         if kind == "zipf":
@@ -71,7 +71,7 @@ def test_no_alloc_histogram_refuses_what_its_array_cannot_hold(xs, gpu):
     keys = torch.zeros(16, dtype=torch.int32, device="cuda")
     bins = torch.zeros(16, dtype=torch.int32, device="cuda")
     s = torch.cuda.current_stream().cuda_stream
-    assert h.HipHistogramLaunchNoAlloc(s, keys.data_ptr(), (1 << 25) + 1, bins.data_ptr(), 16) == xs.kXSchedErrorInvalidValue
+    assert h.HipHistogramLaunchNoAlloc(s, keys.data_ptr(), (1 << 26) + 1, bins.data_ptr(), 16) == xs.kXSchedErrorInvalidValue
     assert h.HipHistogramLaunchNoAlloc(s, keys.data_ptr(), 16, bins.data_ptr(), 65537) == xs.kXSchedErrorInvalidValue
     assert h.HipHistogramLaunchNoAlloc(s, None, 16, bins.data_ptr(), 16) == xs.kXSchedErrorInvalidValue
     assert h.HipHistogramLaunchNoAlloc(s, keys.data_ptr(), 0, bins.data_ptr(), 16) == xs.kXSchedSuccess

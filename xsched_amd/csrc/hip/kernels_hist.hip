@@ -15,21 +15,26 @@
 // all keys and would otherwise serialise the LDS atomics of a wave on one address.
 // The other keys go to LDS counters, in one of two layouts:
 //
-// Two kernels (kMerge; the layout in use up to 2^28 keys). 32768 LDS words hold all
-// 65536 bins as 16-bit halves: word w counts bin w in its low half and bin w + 32768 in its high half (a
-// hot low bin shares its word with a cold high one), one ds_add of 1 or 65536 per key
-// (without a branch: one vote per iteration tells whether every key of the wave is
-// below n_bins, and lanes that hold a ballot key add to a dummy word of their own).
-// The group then stores its words (128 KiB, plain coalesced stores) as one partial
-// histogram into a scratch buffer, and a second kernel sums the partials
-// (each of its groups reads a 512-byte column of every partial) and adds the totals to
-// the result with one 64-bit atomic per pair of bins. A half overflows only when one
-// bin outside the ballot bins takes 65536 keys of a chunk (at least a quarter of it).
-// Every overflow lowers the sum of all halves by at least 65534 and nothing raises it,
-// so "sum of halves == keys that must be in the words" (all keys of the chunk minus the
-// ballot keys and the invalid ones) proves there was none; a group that fails the
-// test stores an all-zero partial and recounts its chunk the slow way (32-bit
-// counters, two passes over its keys, atomic sweep into the result).
+// Two kernels (kMerge; the layout in use up to 2^28 keys). The group's 128 KiB of LDS
+// counters are split in two. Bins below 256 (two thirds of all Zipf(1.1) keys, a fifth of
+// them in bins 0 and 1) have one 32-bit counter PER LANE: 256 bins x 64 lanes, so the lanes of
+// a wave never add to the same address for them, no vote and no popcount is needed, and they
+// cannot overflow. Every other bin is a BYTE: 16384 words shared by the group, word w counts
+// bins w, w + 16384, w + 32768, w + 49152 in its bytes 0..3, one ds_add of
+// 1 << 8 * (key >> 14) per key. One vote per iteration tells whether every key of the wave is
+// below n_bins, so the add needs no branch. The group then stores a partial histogram of
+// 68 KiB (the byte words as they are, the per-lane counters summed) into a scratch buffer,
+// and a second kernel sums the partials column by column and adds the totals to the result
+// with one 64-bit atomic per pair of bins. A byte overflows only when one bin outside the
+// first 256 takes 256 keys of a chunk (0.1 % of it; the hottest such bin of a Zipf(1.1)
+// chunk takes 80). Every overflow lowers the sum of all counters by at least 255 and nothing
+// raises it, so "sum of counters == keys that must be in them" (all key slots of the chunk
+// minus the invalid ones) proves there was none; a group that fails the test stores an
+// all-zero partial and recounts its chunk the slow way (32-bit counters, two passes over its
+// keys, atomic sweep into the result). The first version of this layout kept 16-bit halves
+// for every bin and ballot counters for bins 0 and 1: partials of 128 KiB (32 MiB written
+// and read back per 2^26 keys, now 17 MiB), 14 vector instructions per key (now 10), and
+// LDS adds that serialised on the hot bins.
 //
 // One kernel (above 2^28 keys, where the partials would need more than 128 MiB of
 // scratch, when the scratch buffer cannot be allocated, or on request through
@@ -93,10 +98,19 @@ constexpr uint32_t kTargetGroups = 256;       // compute units of an MI355X
 constexpr uint32_t kSegBins = 256;            // bins one wave sweeps per step
 constexpr uint32_t kSegs = kLdsBins / kSegBins;
 // merge layout
-constexpr uint32_t kPartialWords = kLdsBins + 64;   // packed words, then the ballot bins' counts
-constexpr uint32_t kMergeGroups = 256;              // groups of the merge kernel
-constexpr uint32_t kMergeWords = kLdsBins / kMergeGroups;  // packed words per merge group (128)
+constexpr uint32_t kColdWords = 1u << 14;           // byte counters: word w, byte b = bin w + b * 16384
+constexpr uint32_t kWarmBins = 256;                 // bins below this have 32-bit counters of their own
+constexpr uint32_t kCountWords = kColdWords + kWarmBins * 64;   // LDS words in use: byte words, then a counter per warm bin and lane
+static_assert(kCountWords <= kLdsBins, "the merge layout's counters fit the group's LDS array");
+// A partial histogram in memory is kMergeGroups columns, one per merge group: 64 byte words,
+// then one 32-bit word with the count of bin <column> (the sum of its per-lane counters),
+// then padding to a multiple of 16 bytes.
+constexpr uint32_t kMergeGroups = 256;
+constexpr uint32_t kMergeWords = kColdWords / kMergeGroups;          // byte words per column (64)
+constexpr uint32_t kColumnWords = kMergeWords + 4;
+constexpr uint32_t kPartialWords = kMergeGroups * kColumnWords;      // 68 KiB
 constexpr uint32_t kMaxPartials = 1024;
+static_assert(kWarmBins == kMergeGroups && kHotBins <= kWarmBins, "column j carries the outside count of bin j");
 constexpr uint64_t kMergeMinKeys = 1;             // the two-kernel layout wins at every size measured
 constexpr uint32_t kMergeMinChunk = 16384;        // fewer, fuller partials for small inputs
 
@@ -122,10 +136,8 @@ struct Shared
     uint32_t tail_count;
     uint32_t bailed;
     uint32_t guard_word;
-    uint32_t hot[kHotBins]; // merge layout: ballot counts of the whole group
     uint32_t invalid;       // merge layout: keys outside [0, n_bins), absent ones included
-    uint32_t sum;           // merge layout: sum of all 16-bit halves
-    uint32_t dummy[64];     // merge layout: where the lanes that hold a ballot key add
+    uint32_t sum;           // merge layout: sum of all packed counters
 };
 
 __device__ __forceinline__ void LdsAdd(uint32_t *p, uint32_t v)
@@ -205,9 +217,28 @@ __device__ __forceinline__ void SweepOut(Shared &sh, uint32_t *dst, uint32_t cou
     }
 }
 
-__device__ __forceinline__ void ClearBins(Shared &sh)
+__device__ __forceinline__ void ClearBins(Shared &sh, uint32_t words = kLdsBins)
 {
-    for (uint32_t i = threadIdx.x * 4; i < kLdsBins; i += kThreads * 4) *(u32x4 *)&sh.bins[i] = u32x4 { 0, 0, 0, 0 };
+    for (uint32_t i = threadIdx.x * 4; i < words; i += kThreads * 4) *(u32x4 *)&sh.bins[i] = u32x4 { 0, 0, 0, 0 };
+}
+
+/// Merge layout: where a valid key is counted, and by how much. Bins below kWarmBins (two
+/// thirds of all Zipf(1.1) keys) have one 32-bit counter PER LANE, so the lanes of a wave never
+/// add to the same address for them; every other bin is a byte of a word shared by the group.
+__device__ __forceinline__ void PackedSlot(uint32_t key, uint32_t lane, uint32_t &word, uint32_t &inc)
+{
+    const bool warm = key < kWarmBins;
+    word = warm ? kColdWords + key * 64 + lane : key & (kColdWords - 1);
+    inc = warm ? 1u : 1u << ((key >> 11) & 24u);
+}
+
+/// Sum of the four byte counters of each of four packed words.
+__device__ __forceinline__ uint32_t ByteSum(const u32x4 &w)
+{
+    const uint32_t even = (w.x & 0x00FF00FFu) + (w.y & 0x00FF00FFu) + (w.z & 0x00FF00FFu) + (w.w & 0x00FF00FFu);
+    const uint32_t odd = ((w.x >> 8) & 0x00FF00FFu) + ((w.y >> 8) & 0x00FF00FFu) + ((w.z >> 8) & 0x00FF00FFu) +
+                         ((w.w >> 8) & 0x00FF00FFu);
+    return (even & 0xFFFFu) + (even >> 16) + (odd & 0xFFFFu) + (odd >> 16);
 }
 
 /// kMerge: the group stores a packed partial histogram at partials + blockIdx.x *
@@ -229,9 +260,8 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     const uint32_t tail_range = !kMerge && n_bins > kLdsBins ? n_bins - kLdsBins : 0;
     XGuardBlock guard(g, blockIdx.x, &sh.guard_word);
 
-    ClearBins(sh);
+    ClearBins(sh, kMerge ? kCountWords : kLdsBins);   // the same number today; the layouts differ
     if (tid == 0) { sh.tail_count = 0; sh.bailed = 0; sh.invalid = 0; sh.sum = 0; }
-    if (tid < kHotBins) sh.hot[tid] = 0;
 
     const uint64_t begin = (uint64_t)blockIdx.x * chunk;
     const uint64_t end = begin + chunk < n ? begin + chunk : n;
@@ -307,29 +337,29 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             k[u * 4 + 2] = (uint32_t)v[u].z; k[u * 4 + 3] = (uint32_t)v[u].w;
         }
         if (kMerge) {
-#pragma unroll
-            for (uint32_t j = 0; j < kN; ++j) {
-#pragma unroll
-                for (uint32_t b = 0; b < kHotBins; ++b) AddPopcount(hot[b], __ballot(k[j] == b));
-            }
-            // Are all keys of the wave below n_bins (the usual case)? One max per key pair
-            // and one vote per iteration decide it; then every key is either a ballot key
-            // or counted, nothing has to be tallied per key, and the LDS add needs no
-            // branch: ballot keys add to a lane-private dummy word instead.
+            // Are all keys of the wave below n_bins (the usual case)? One max per key and one
+            // vote per iteration decide it; then nothing has to be tallied per key and the
+            // LDS add needs no branch.
             uint32_t largest = k[0];
 #pragma unroll
             for (uint32_t j = 1; j < kN; ++j) largest = largest > k[j] ? largest : k[j];
             if (__ballot(largest >= n_bins) == 0) {
 #pragma unroll
                 for (uint32_t j = 0; j < kN; ++j) {
-                    uint32_t *word = k[j] >= kHotBins ? &sh.bins[k[j] & (kLdsBins - 1)] : &sh.dummy[lane];
-                    LdsAdd(word, 1u + (k[j] >> 15) * 65535u);
+                    uint32_t word, inc;
+                    PackedSlot(k[j], lane, word, inc);
+                    LdsAdd(&sh.bins[word], inc);
                 }
             } else {
 #pragma unroll
                 for (uint32_t j = 0; j < kN; ++j) {
-                    if (k[j] >= n_bins) invalid += 1;
-                    if (k[j] - kHotBins < main_range) LdsAdd(&sh.bins[k[j] & (kLdsBins - 1)], 1u + (k[j] >> 15) * 65535u);
+                    if (k[j] >= n_bins) {
+                        invalid += 1;
+                    } else {
+                        uint32_t word, inc;
+                        PackedSlot(k[j], lane, word, inc);
+                        LdsAdd(&sh.bins[word], inc);
+                    }
                 }
             }
         } else {
@@ -448,12 +478,10 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     if (!count_chunk() && lane == 0) sh.bailed = 1;
 
     // Ballot counters are per wave: lane 0 of each wave folds them into the group's.
-    if (lane == 0) {
+    if (!kMerge && lane == 0) {
 #pragma unroll
         for (uint32_t b = 0; b < kHotBins; ++b) {
-            if (hot[b] == 0 || b >= lds_used) continue;
-            if (kMerge) LdsAdd(&sh.hot[b], hot[b]);
-            else        LdsAdd(&sh.bins[b], hot[b]);
+            if (hot[b] != 0 && b < lds_used) LdsAdd(&sh.bins[b], hot[b]);
         }
     }
     if (kMerge && invalid != 0) LdsAdd(&sh.invalid, invalid);
@@ -471,28 +499,37 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     const uint32_t rot = (blockIdx.x * 37u) & (kSegs - 1);
     if (kMerge) {
         uint32_t *part = partials + (size_t)blockIdx.x * kPartialWords;
-        uint32_t halves = 0;
-        for (uint32_t i = tid * 4; i < kLdsBins; i += kThreads * 4) {
+        uint32_t counted = 0;
+        for (uint32_t i = tid * 4; i < kColdWords; i += kThreads * 4) {
             const u32x4 w = *(const u32x4 *)&sh.bins[i];
-            *(u32x4 *)&part[i] = w;
-            halves += (w.x & 0xFFFFu) + (w.x >> 16) + (w.y & 0xFFFFu) + (w.y >> 16)
-                    + (w.z & 0xFFFFu) + (w.z >> 16) + (w.w & 0xFFFFu) + (w.w >> 16);
+            *(u32x4 *)&part[(i / kMergeWords) * kColumnWords + i % kMergeWords] = w;
+            counted += ByteSum(w);
         }
-        if (tid < 64) part[kLdsBins + tid] = tid < kHotBins ? sh.hot[tid] : 0u;
-        LdsAdd(&sh.sum, halves);
+        {
+            // the 64 per-lane counters of warm bin tid / 4: four threads sum 16 each
+            const uint32_t *mine = &sh.bins[kColdWords + (tid / 4) * 64 + (tid % 4) * 16];
+            uint32_t warm = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < 4; ++q) {
+                const u32x4 w = *(const u32x4 *)&mine[q * 4];
+                warm += w.x + w.y + w.z + w.w;
+            }
+            counted += warm;
+            warm += __shfl_xor(warm, 1);
+            warm += __shfl_xor(warm, 2);
+            if (tid % 4 == 0) *(u32x4 *)&part[(tid / 4) * kColumnWords + kMergeWords] = u32x4 { warm, 0, 0, 0 };
+        }
+        LdsAdd(&sh.sum, counted);
         __syncthreads();
         // every key slot the group went through (absent keys of the ragged end included) is
-        // a ballot key, an invalid one, or in the words
-        uint32_t expected = (uint32_t)(full_end - begin)
-                          + (uint32_t)((end - full_end + kUnitKeys - 1) / kUnitKeys) * kUnitKeys - sh.invalid;
-#pragma unroll
-        for (uint32_t b = 0; b < kHotBins; ++b) expected -= sh.hot[b];
+        // an invalid key or in the counters
+        const uint32_t expected = (uint32_t)(full_end - begin)
+                                + (uint32_t)((end - full_end + kUnitKeys - 1) / kUnitKeys) * kUnitKeys - sh.invalid;
         if (__builtin_amdgcn_readfirstlane(sh.sum) != __builtin_amdgcn_readfirstlane(expected)) {
-            // A 16-bit half overflowed: this group's partial counts nothing, and the chunk
+            // A byte counter overflowed: this group's partial counts nothing, and the chunk
             // is counted again with 32-bit counters, one half of the bins at a time.
             __syncthreads();
-            for (uint32_t i = tid * 4; i < kLdsBins; i += kThreads * 4) *(u32x4 *)&part[i] = u32x4 { 0, 0, 0, 0 };
-            if (tid < 64) part[kLdsBins + tid] = 0u;
+            for (uint32_t i = tid * 4; i < kPartialWords; i += kThreads * 4) *(u32x4 *)&part[i] = u32x4 { 0, 0, 0, 0 };
             for (uint32_t first = 0; first < n_bins; first += kLdsBins) {
                 const uint32_t count = n_bins - first < kLdsBins ? n_bins - first : kLdsBins;
                 ClearBins(sh);
@@ -531,38 +568,52 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
     if (kGuard) guard.Commit();
 }
 
-/// Sums the packed partial histograms of the counting groups and adds the totals to
-/// bins. Group j owns packed words [j * kMergeWords, (j + 1) * kMergeWords): thread
-/// (row, col) reads four of them from partials row, row + 32, ...; its progress byte is
-/// first_wg + j.
+/// Sums the partial histograms of the counting groups and adds the totals to bins. Group j
+/// owns column j of every partial: 64 words of byte counters (word w, byte b = bin
+/// w + b * 16384) and the count of bin j, which is kept outside the bytes. Thread (row, col)
+/// reads four byte words of its column from partials row, row + 64, ...; the threads of
+/// col 0 also read the outside count. The group's progress byte is first_wg + j.
 template <bool kGuard>
 __global__ __launch_bounds__(kThreads)
 void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part, uint32_t *__restrict__ bins,
                           uint32_t n_bins, uint32_t first_wg, XGuardArgs g)
 {
-    constexpr uint32_t kCols = kMergeWords / 4, kRows = kThreads / kCols; // 32 x 32
-    __shared__ uint32_t red[kRows][8][kCols];
-    __shared__ uint32_t total[2][kMergeWords];
-    __shared__ uint32_t hot_total[kHotBins];
+    constexpr uint32_t kCols = kMergeWords / 4, kRows = kThreads / kCols; // 16 x 64
+    constexpr uint32_t kAhead = 4;                                       // rows requested before the guard's reads
+    __shared__ uint32_t red[kRows][16][kCols];   // per row: the 16 byte counters of each of the 16 word quads
+    __shared__ uint32_t total[16][kCols];
+    __shared__ uint32_t outside_total;
     __shared__ uint32_t guard_word;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t col = tid % kCols, row = tid / kCols;
-    const uint32_t word0 = blockIdx.x * kMergeWords + col * 4;
+    const uint32_t column = blockIdx.x;
+    const uint32_t word0 = column * kColumnWords + col * 4;
     auto load_words = [&](uint32_t p) {
         return p < n_part ? *(const u32x4 *)(partials + (size_t)p * kPartialWords + word0) : u32x4 { 0, 0, 0, 0 };
     };
-    uint32_t acc[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
-    auto add_words = [&](const u32x4 &w) {
-        acc[0] += w.x & 0xFFFFu; acc[1] += w.y & 0xFFFFu; acc[2] += w.z & 0xFFFFu; acc[3] += w.w & 0xFFFFu;
-        acc[4] += w.x >> 16;     acc[5] += w.y >> 16;     acc[6] += w.z >> 16;     acc[7] += w.w >> 16;
+    auto load_outside = [&](uint32_t p) {
+        return col == 0 && p < n_part ? partials[(size_t)p * kPartialWords + column * kColumnWords + kMergeWords] : 0u;
     };
-    // The first eight rows are requested before the guard's reads: the kernel is short, and
-    // the round trips overlap. Reading has no side effect (after a flushed counting launch
-    // the words are stale, and nothing is done with them).
-    u32x4 first[8];
+    // even[i] holds bytes 0 and 2 of word i in its halves, odd[i] bytes 1 and 3; a thread adds
+    // at most kMaxPartials / kRows = 16 values of 255 into a half.
+    uint32_t even[4] = { 0, 0, 0, 0 }, odd[4] = { 0, 0, 0, 0 }, outside = 0;
+    auto add_words = [&](const u32x4 &w) {
+        const uint32_t v[4] = { w.x, w.y, w.z, w.w };
 #pragma unroll
-    for (uint32_t i = 0; i < 8; ++i) first[i] = load_words(row + i * kRows);
+        for (uint32_t i = 0; i < 4; ++i) { even[i] += v[i] & 0x00FF00FFu; odd[i] += (v[i] >> 8) & 0x00FF00FFu; }
+    };
+    // The first rows are requested before the guard's reads: the kernel is short, and the
+    // round trips overlap. Reading has no side effect (after a flushed counting launch the
+    // words are stale, and nothing is done with them).
+    u32x4 first[kAhead];
+    uint32_t first_outside[kAhead];
+#pragma unroll
+    for (uint32_t i = 0; i < kAhead; ++i) {
+        first[i] = load_words(row + i * kRows);
+        first_outside[i] = load_outside(row + i * kRows);
+    }
+    if (tid == 0) outside_total = 0;
 
     if (kGuard) {
         // A flushed counting launch leaves partials missing: every counting group must have
@@ -585,41 +636,42 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
         int all = 1;
 #pragma unroll
         for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) all &= tag[i] == (uint8_t)g.gen;
-        const int complete = __syncthreads_and(all);   // also publishes guard_word
+        const int complete = __syncthreads_and(all);   // also publishes guard_word (and outside_total = 0)
         if (!complete || guard_word == 0) return;
+    } else {
+        __syncthreads();
     }
-    if (tid < kHotBins) hot_total[tid] = 0;
 
 #pragma unroll
-    for (uint32_t i = 0; i < 8; ++i) add_words(first[i]);
-#pragma unroll 8
-    for (uint32_t p = row + 8 * kRows; p < n_part; p += kRows) add_words(load_words(p));
+    for (uint32_t i = 0; i < kAhead; ++i) { add_words(first[i]); outside += first_outside[i]; }
+#pragma unroll 4
+    for (uint32_t p = row + kAhead * kRows; p < n_part; p += kRows) { add_words(load_words(p)); outside += load_outside(p); }
+    // counter b * 4 + i of a thread: byte b of its word i
 #pragma unroll
-    for (uint32_t v = 0; v < 8; ++v) red[row][v][col] = acc[v];
-    __syncthreads();
-    if (blockIdx.x == 0) {
-        // the ballot bins' counts ride behind the packed words of every partial
-        for (uint32_t p = tid; p < n_part * kHotBins; p += kThreads) {
-            const uint32_t v = partials[(size_t)(p / kHotBins) * kPartialWords + kLdsBins + p % kHotBins];
-            if (v != 0) LdsAdd(&hot_total[p % kHotBins], v);
-        }
+    for (uint32_t i = 0; i < 4; ++i) {
+        red[row][0 + i][col] = even[i] & 0xFFFFu;
+        red[row][4 + i][col] = odd[i] & 0xFFFFu;
+        red[row][8 + i][col] = even[i] >> 16;
+        red[row][12 + i][col] = odd[i] >> 16;
     }
-    if (tid < 8 * kCols) {
+    if (outside != 0) LdsAdd(&outside_total, outside);
+    __syncthreads();
+    if (tid < 16 * kCols) {
         const uint32_t v = tid / kCols, c = tid % kCols;
         uint32_t t = 0;
-#pragma unroll
+#pragma unroll 16
         for (uint32_t r = 0; r < kRows; ++r) t += red[r][v][c];
-        total[v >> 2][c * 4 + (v & 3)] = t;
+        total[v][c] = t;
     }
     __syncthreads();
 
+    // 256 counters, 128 pairs of neighbouring bins: counter (b, i) of quad c is bin
+    // column * 64 + c * 4 + i + b * 16384.
     const bool pair_ok = (((uintptr_t)bins) & 7) == 0;
-    if (tid < kMergeWords) {
-        const uint32_t half = tid / (kMergeWords / 2), q = tid % (kMergeWords / 2);
-        const uint32_t bin = half * kLdsBins + blockIdx.x * kMergeWords + q * 2;
-        uint32_t lo = total[half][q * 2], hi = total[half][q * 2 + 1];
-        if (bin < kHotBins) lo += hot_total[bin];
-        if (bin + 1 < kHotBins) hi += hot_total[bin + 1];
+    if (tid < 128) {
+        const uint32_t b = tid / 32, c = (tid % 32) / 2, i = (tid % 2) * 2;
+        const uint32_t lo = total[b * 4 + i][c], hi = total[b * 4 + i + 1][c];
+        const uint32_t bin = column * kMergeWords + c * 4 + i + b * kColdWords;
         if ((lo | hi) != 0) {
             if (pair_ok && bin + 1 < n_bins) {
                 PairFix(bins + bin, PairAdd(bins + bin, lo, hi), lo);
@@ -628,6 +680,9 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
                 if (hi != 0 && bin + 1 < n_bins) GlobalAdd(bins + bin + 1, hi);
             }
         }
+    } else if (tid == 128) {
+        // bin <column>, counted outside the bytes (which hold nothing for bins below 256)
+        if (outside_total != 0 && column < n_bins) GlobalAdd(bins + column, outside_total);
     }
     if (kGuard) {
         XGuardBlock guard(g, first_wg + blockIdx.x, &guard_word);
@@ -714,11 +769,11 @@ using namespace xsched::hip;
 // hipGetSymbolAddress(), never a device pointer.
 namespace
 {
-constexpr uint32_t kNoAllocMaxGroups = 128;                       // counting work-groups
-constexpr uint64_t kNoAllocMaxKeys = (uint64_t)kNoAllocMaxGroups * hist::kMaxChunk; // 2^25
+constexpr uint32_t kNoAllocMaxGroups = 256;                       // counting work-groups
+constexpr uint64_t kNoAllocMaxKeys = (uint64_t)kNoAllocMaxGroups * hist::kMaxChunk; // 2^26
 constexpr size_t kNoAllocScratchWords = (size_t)kNoAllocMaxGroups * hist::kPartialWords;
 
-static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];          // 16.03 MiB
+static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];          // 17 MiB
 
 constexpr int kNoAllocMaxDevices = 64;
 std::mutex g_scratch_mtx;
