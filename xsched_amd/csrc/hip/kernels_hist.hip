@@ -79,7 +79,7 @@ constexpr uint32_t kHotBins = XSCHED_HIST_HOT_BINS;
 constexpr uint32_t kLdsBins = 1u << 15;       // 128 KiB of counters
 constexpr uint32_t kTailCap = 14336;          // 16-bit entries, 28 KiB
 #ifndef XSCHED_HIST_UNITS
-#define XSCHED_HIST_UNITS 2
+#define XSCHED_HIST_UNITS 1
 #endif
 constexpr uint32_t kUnits = XSCHED_HIST_UNITS;  // 128-bit loads per thread and iteration
 #ifndef XSCHED_HIST_DEPTH
