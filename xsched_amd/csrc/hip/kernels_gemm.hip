@@ -19,9 +19,10 @@
 //
 // Guard: the tile is computed in registers and written once at the end, so a
 // work-group may give up at any K step without side effects. The preempt word is
-// checked at entry and then every kPollSteps K steps (piggy-backed on a barrier the
-// loop has anyway); a flushed tile leaves its progress bit clear and is redone by
-// the replay. Work-group ids are remapped so that the 32 CUs of one XCD (ids equal
+// checked at entry and then every kPollSteps K steps: wave 0 requests it with a vector load
+// at the top of the step and looks at it in front of the barrier the loop has anyway, so
+// nobody waits for it; a flushed tile leaves its progress byte untagged and is redone by
+// the replay. The tile is written out through LDS, whole rows of 128 bytes per eight lanes. Work-group ids are remapped so that the 32 CUs of one XCD (ids equal
 // modulo 8 land on one XCD) work on neighbouring tiles and share A/B panels in that
 // XCD's L2.
 #include "hip_hal.h"
@@ -222,6 +223,14 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     for (int t = 0; t < steps; ++t) {
         const int cur = t & 1;
         const int k_next = (t + 2 < steps ? t + 2 : steps - 1) * kStepK;
+        // Every kPollSteps steps wave 0 asks for the preempt word here, with a vector load that
+        // is on its way during the whole step, and looks at it just before the barrier: no
+        // wave ever waits for the word alone (a scalar load at the barrier made wave 0 wait
+        // for the uncached round trip and for all of its LDS reads while the other seven
+        // waves stood at the barrier).
+        const bool poll_step = kGuard && (t % kPollSteps) == kPollSteps - 1;
+        uint32_t polled = 0;
+        if (poll_step && wave == 0) polled = xguard_read_flag_begin(xguard_flag_copy(g, blockIdx.x));
 
         load_frags(cur, 1, fa[1], fb[1]);
         mfma_slice(0);
@@ -234,13 +243,15 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         load_global(k_next);
         mfma_slice(0);
 
-        if (kGuard && (t % kPollSteps) == kPollSteps - 1 && tid == 0) {
-            const bool current = xguard_read_flag(xguard_flag_copy(g, blockIdx.x)) == g.epoch;
-            if (!current) xguard_note_flush(g);
-            guard_word = current ? 1u : 0u;
+        if (poll_step && wave == 0) {
+            const bool current = xguard_read_flag_end(polled) == g.epoch;
+            if (lane == 0) {
+                if (!current) xguard_note_flush(g);
+                guard_word = current ? 1u : 0u;
+            }
         }
         __syncthreads(); // buffer cur^1 is complete, buffer cur is free to be overwritten
-        if (kGuard && (t % kPollSteps) == kPollSteps - 1) {
+        if (poll_step) {
             if (guard_word == 0) return; // whole group leaves together; nothing was written
         }
 
@@ -248,16 +259,32 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         mfma_slice(1);
     }
 
+    // Write-out. A lane holds one column of sixteen rows of each 32x32 block, so storing from
+    // the accumulators means 2-byte stores to sixteen different rows. Instead every wave turns
+    // its strips of 32 rows x 64 columns over in LDS (an area of its own in the A buffers,
+    // rows padded by 8 bf16), and stores them as whole rows: 16 bytes per lane, eight lanes to
+    // a row of 128 bytes.
+    constexpr int kStripStride = 64 + 8;
+    static_assert(sizeof(As) >= (size_t)kWavesM * kWavesN * 32 * kStripStride * 2, "the A buffers hold one strip per wave");
+    __syncthreads(); // every wave has read its last fragments
+    uint16_t *strip = &As[0][0] + wave * (32 * kStripStride);
 #pragma unroll
     for (int i = 0; i < kBlocksM; ++i) {
 #pragma unroll
         for (int j = 0; j < kBlocksN; ++j) {
-            const size_t col = n0 + 64 * wn + 32 * j + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const size_t row = m0 + 32 * kBlocksM * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                C[row * (size_t)N + col] = f32_to_bf16_rne(acc[i][j][r]);
+                const uint32_t row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                strip[row * kStripStride + 32 * j + (lane & 31)] = f32_to_bf16_rne(acc[i][j][r]);
             }
+        }
+        const size_t row0 = m0 + 32 * kBlocksM * wm + 32 * i;
+        const size_t col0 = n0 + 64 * wn + 8 * (lane & 7);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t row = 8 * q + (lane >> 3);
+            const u32x4 v = *(const u32x4 *)(strip + row * kStripStride + 8 * (lane & 7));
+            *(u32x4 *)(C + (row0 + row) * (size_t)N + col0) = v;
         }
     }
 
