@@ -152,7 +152,9 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
             parked_ = true;
             while (ring_count_ == 0 && retired_.load(std::memory_order_acquire) < handed_over_.load(std::memory_order_acquire) &&
                    std::chrono::steady_clock::now() < until) {
-                ring_cv_.wait_for(g, std::chrono::microseconds(kStandBySliceMicros));
+                // (a wait on the system clock: the sanitizer build's runtime does not know the
+                // steady-clock wait of newer C libraries and would lose track of the lock)
+                ring_cv_.wait_until(g, std::chrono::system_clock::now() + std::chrono::microseconds(kStandBySliceMicros));
             }
             parked_ = false;
             stood_by_for_ = handed_over_.load(std::memory_order_acquire);
