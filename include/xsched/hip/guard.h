@@ -126,6 +126,18 @@ __device__ __forceinline__ void xguard_note_flush(const XGuardArgs &g)
     if (g.flushed) *g.flushed = g.epoch;
 }
 
+/// The `flushed` word (wave-uniform); a value no launch carries when the queue has none.
+__device__ __forceinline__ uint32_t xguard_read_flushed(const XGuardArgs &g)
+{
+    return g.flushed != nullptr ? (uint32_t)__builtin_amdgcn_readfirstlane((int)*g.flushed) : ~g.epoch;
+}
+
+/// The work-group's byte of the progress map (wave-uniform).
+__device__ __forceinline__ uint32_t xguard_read_tag(const XGuardArgs &g, uint32_t wg)
+{
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)__builtin_nontemporal_load(&g.done[wg]));
+}
+
 /// True when an earlier launch of this epoch has been flushed (wave-uniform).
 __device__ __forceinline__ bool xguard_epoch_flushed(const XGuardArgs &g)
 {
@@ -148,14 +160,13 @@ public:
     __device__ __forceinline__ bool Enter() const
     {
         if (xguard_inert(g_)) return true;
-        const bool earlier_flushed = xguard_epoch_flushed(g_);
-        if (xguard_read_flag(xguard_flag_copy(g_, wg_)) != g_.epoch) {
-            if ((threadIdx.x & 63) == 0) xguard_note_flush(g_);
-            return false;
-        }
-        if (earlier_flushed) return false;
-        if (g_.resume && g_.done && xguard_committed(g_, wg_)) return false;
-        return true;
+        const uint32_t flushed_word = xguard_read_flushed(g_);
+        const uint32_t copy = xguard_read_flag(xguard_flag_copy(g_, wg_));
+        const bool replay_with_map = g_.resume && g_.done;
+        const uint32_t tag = replay_with_map && copy == g_.epoch ? xguard_read_tag(g_, wg_) : 0u;
+        const XGuardVerdict v = xguard_entry_verdict(copy, flushed_word, g_.epoch, g_.resume, g_.done != nullptr, tag, g_.gen);
+        if (v.note_flush && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
+        return v.run != 0;
     }
 
     /// Call after the last store of the work-group.
@@ -181,12 +192,15 @@ public:
     {
         if (xguard_inert(g_)) return true;
         if (threadIdx.x < 64) {
-            const bool earlier_flushed = xguard_epoch_flushed(g_);
-            bool go = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
-            if (!go && threadIdx.x == 0) xguard_note_flush(g_);
-            if (earlier_flushed) go = false;
-            if (go && g_.resume && g_.done && xguard_committed(g_, wg_)) go = false;
-            if (threadIdx.x == 0) *lds_ = go ? 1u : 0u;
+            const uint32_t flushed_word = xguard_read_flushed(g_);
+            const uint32_t copy = xguard_read_flag(xguard_flag_copy(g_, wg_));
+            const bool replay_with_map = g_.resume && g_.done;
+            const uint32_t tag = replay_with_map && copy == g_.epoch ? xguard_read_tag(g_, wg_) : 0u;
+            const XGuardVerdict v = xguard_entry_verdict(copy, flushed_word, g_.epoch, g_.resume, g_.done != nullptr, tag, g_.gen);
+            if (threadIdx.x == 0) {
+                if (v.note_flush) xguard_note_flush(g_);
+                *lds_ = v.run;
+            }
         }
         __syncthreads();
         return *lds_ != 0;
@@ -201,9 +215,9 @@ public:
         if (xguard_inert(g_)) return true;
         __syncthreads();
         if (threadIdx.x == 0) {
-            const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
-            if (!current) xguard_note_flush(g_);
-            *lds_ = current ? 1u : 0u;
+            const XGuardVerdict v = xguard_recheck_verdict(xguard_read_flag(xguard_flag_copy(g_, wg_)), g_.epoch);
+            if (v.note_flush) xguard_note_flush(g_);
+            *lds_ = v.run;
         }
         __syncthreads();
         return *lds_ != 0;
@@ -216,9 +230,9 @@ public:
     __device__ __forceinline__ bool WaveStillCurrent() const
     {
         if (xguard_inert(g_)) return true;
-        const bool current = xguard_read_flag(xguard_flag_copy(g_, wg_)) == g_.epoch;
-        if (!current && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
-        return current;
+        const XGuardVerdict v = xguard_recheck_verdict(xguard_read_flag(xguard_flag_copy(g_, wg_)), g_.epoch);
+        if (v.note_flush && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
+        return v.run != 0;
     }
 
     /// WaveStillCurrent() split in two so that the read of the preempt word overlaps the
@@ -231,9 +245,9 @@ public:
 
     __device__ __forceinline__ bool WavePollEnd(uint32_t pending) const
     {
-        const bool current = xguard_read_flag_end(pending) == g_.epoch;
-        if (!current && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
-        return current;
+        const XGuardVerdict v = xguard_recheck_verdict(xguard_read_flag_end(pending), g_.epoch);
+        if (v.note_flush && (threadIdx.x & 63) == 0) xguard_note_flush(g_);
+        return v.run != 0;
     }
 
     /// Call after the last store of the work-group (all waves; one barrier inside).

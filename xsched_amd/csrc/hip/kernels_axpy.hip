@@ -164,10 +164,9 @@ void AxpyPersistentKernel(float alpha, const float4 *x, float4 *y, uint64_t n4, 
                 // The scalar read of the preempt word waits for itself only: the vector loads
                 // stay in flight across it. A flushed wave drops what it has loaded.
                 if (kGuard) {
-                    if (xguard_read_flag(flag) != g.epoch) {
-                        if (lane == 0) xguard_note_flush(g);
-                        return;
-                    }
+                    const XGuardVerdict v = xguard_recheck_verdict(xguard_read_flag(flag), g.epoch);
+                    if (v.note_flush && lane == 0) xguard_note_flush(g);
+                    if (!v.run) return;
                     skip = g.resume && g.done && xguard_committed(g, c);
                 }
                 if (!skip && !full) {
