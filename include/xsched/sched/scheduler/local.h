@@ -27,6 +27,9 @@ public:
     /// next round tells the processes.
     void SetPolicy(XPolicyType type);
     XPolicyType GetPolicy() const;
+    /// The id for an operation the caller is about to send to process `pid` itself (the
+    /// daemon's configuration requests); 0 for a process that never announced itself.
+    OperationId NextOperationId(PID pid);
 
 private:
     class Rounds;

@@ -1,6 +1,7 @@
 """Helper process for tests/test_daemon.py: one XSched client talking to xserver
 (XSCHED_SCHEDULER=GLB). Roles:
   busy <prio> <seconds>   one host queue at priority <prio> that is busy for <seconds>
+  idle <prio> <seconds>   one host queue at priority <prio> with no work, kept for <seconds>
   quick <prio> <count>    one host queue at priority <prio>; submits <count> quick kernels,
                           reports how many had run after 0.3 s and after everything finished
 Prints one JSON line."""
@@ -36,6 +37,9 @@ def main():
         xs.check(p.XQueueSubmit(xq, cmd.value))
         print(json.dumps({"event": "busy-started", "pid": os.getpid()}), flush=True)
         xs.check(p.XQueueWaitAll(xq))
+    elif role == "idle":
+        print(json.dumps({"event": "busy-started", "pid": os.getpid()}), flush=True)
+        time.sleep(arg)
     else:
         @xs.HostKernelFn
         def quick(a, wg, n):

@@ -44,7 +44,7 @@ PREEMPT_SRCS = [
     "preempt/xcommand.cpp", "preempt/ring_queue.cpp", "preempt/xqueue.cpp", "preempt/agent.cpp",
 ]
 HOST_SRCS = ["host/host_queue.cpp", "host/host_bench.cpp"]
-SERVER_SRCS = ["service/xserver.cpp"]
+SERVER_SRCS = ["service/xserver.cpp", "service/http.cpp"]
 SHIM_SRCS = ["shim/code_object.cpp", "shim/hip_shim.cpp"]
 HIP_SRCS = ["hip/hip_queue.hip", "hip/hip_command.hip", "hip/kernels_axpy.hip",
             "hip/kernels_gemm.hip", "hip/kernels_hist.hip", "bench/harness.hip"]

@@ -288,6 +288,7 @@ public:
     }
 
     XPolicyType Type() const { return type_; }
+    OperationId IssueId(PID pid) { return ledger_.Issue(pid); }
 
 private:
     void Turn()
@@ -408,5 +409,6 @@ void LocalScheduler::Stop() { rounds_->Halt(); }
 void LocalScheduler::RecvEvent(std::shared_ptr<const Event> event) { rounds_->Accept(std::move(event)); }
 void LocalScheduler::SetPolicy(XPolicyType type) { rounds_->SwitchTo(type); }
 XPolicyType LocalScheduler::GetPolicy() const { return rounds_->Type(); }
+OperationId LocalScheduler::NextOperationId(PID pid) { return rounds_->IssueId(pid); }
 
 } // namespace xsched::sched
