@@ -3,12 +3,17 @@
 //
 // MFMA-bound: 2*M*N*K flop. One work-group of 512 threads (8 wavefronts) owns one
 // 256x256 tile of C and walks K in steps of 64 through two LDS buffers:
-//   global -> registers (tile t+2 is requested while tile t is computed), 128-bit loads for
-//                       both operands
-//   registers -> LDS    A tile as [256 rows][64 k], rows padded to 72 bf16 so that the 128-bit
-//                       fragment reads of 32 consecutive rows fall into distinct banks;
-//                       B tile as it sits in memory, [64 k][256 cols], rows padded to 272 bf16;
-//                       written to the buffer that is not being read, one barrier per step
+//   global -> LDS       buffer_load ... lds: every wave-wide load moves 64 x 16 bytes straight
+//                       into 1 KiB of LDS, no registers and no LDS store instructions in
+//                       between. Lane l of a load fills the l-th 16-byte slot of that KiB and
+//                       is free in what it fetches, so the tiles are kept unpadded and
+//                       XOR-swizzled: the slot a piece lands in is its natural slot XOR a few
+//                       bits of its row, chosen so that every fragment read below touches
+//                       each LDS bank once.
+//                       A tile: [256 rows][64 k], two rows to a 256-byte line of sixteen
+//                       slots, slot = ((row & 1) * 8 + k / 8) ^ (line & 15).
+//                       B tile: as it sits in memory, [64 k][256 cols], eight 64-byte granules
+//                       to a row, granule = (col / 32) ^ ((k & 3) | ((k >> 1) & 4)).
 //   LDS -> MFMA         v_mfma_f32_32x32x16_bf16; wave (wm, wn) of the 2x4 wave grid
 //                       accumulates a 128x64 sub-tile = 4x2 blocks of 32x32
 // An MFMA operand wants eight consecutive k per lane. A has them contiguous in memory; for B
@@ -17,14 +22,20 @@
 // There is no split-K: every element of C is summed by one wave in one fixed order, which
 // makes a replayed tile bit-identical.
 //
+// Under this load the device runs against its power limit (the clock settles near 1.85 GHz),
+// so bytes moved cost time even when nothing waits for them: the loop issues one LDS read or
+// one global load next to each MFMA and nothing else.
+//
 // Guard: the tile is computed in registers and written once at the end, so a
 // work-group may give up at any K step without side effects. The preempt word is
 // checked at entry and then every kPollSteps K steps: wave 0 requests it with a vector load
 // at the top of the step and looks at it in front of the barrier the loop has anyway, so
 // nobody waits for it; a flushed tile leaves its progress byte untagged and is redone by
-// the replay. The tile is written out through LDS, whole rows of 128 bytes per eight lanes. Work-group ids are remapped so that the 32 CUs of one XCD (ids equal
-// modulo 8 land on one XCD) work on neighbouring tiles and share A/B panels in that
-// XCD's L2.
+// the replay. The tile is written out through LDS, whole rows of 128 bytes per eight lanes.
+// Work-group ids are remapped so that the 32 CUs of one XCD (ids equal modulo 8 land on one
+// XCD) work on neighbouring tiles and share A/B panels in that XCD's L2.
+#include <type_traits>
+
 #include "hip_hal.h"
 #include "xsched/hip/hal.h"
 
@@ -39,20 +50,21 @@ namespace gemm
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 LdsS16x4;
+typedef __attribute__((address_space(3))) void LdsVoid;
+typedef __attribute__((address_space(3))) volatile uint32_t LdsVolatileWord;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kLargeTile = 256;     // edge of the large tile of C (M and N)
 constexpr int kSmallTile = 128;     // edge of the small one
 constexpr int kStepK = 64;          // K per step
-constexpr int kLdsStride = 72;      // bf16 per row of the A tile in LDS (64 + 8 padding)
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef __attribute__((address_space(3))) s16x4 LdsS16x4;
 constexpr int kPollSteps = 8;       // K steps between two looks at the preempt word
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 4;       // tile rows walked together
-
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+constexpr int kMaxK = 1 << 22;      // 32-bit byte offsets inside a 256-row panel of A
 
 /// Round-to-nearest-even to bf16, NaNs quieted: the conversion instruction of gfx950
 /// (v_cvt_pk_bf16_f32), which gives bit for bit what the integer formula
@@ -84,34 +96,56 @@ __device__ __forceinline__ void TileOf(uint32_t wg, uint32_t tiles_m, uint32_t t
     tn = in_band / rows;
 }
 
-// Two LDS buffers and ONE barrier per K step: while the MFMAs of step t read buffer
-// t % 2, the registers holding tile t + 1 are written to the other buffer and the global
-// loads of tile t + 2 are issued; the fragments of the next 16-wide k slice are read from
-// LDS before the MFMAs of the current slice are issued.
+// The compiler keeps the instructions of one group in the order the groups are listed:
+// mask 0x008 = MFMA, 0x100 = LDS read.
+#define XS_GROUP(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define XS_PIN __builtin_amdgcn_sched_barrier(0)
+#define XS_WAIT_GLOBAL_LOADS __builtin_amdgcn_s_waitcnt(0x0F70) /* vmcnt(0), nothing else */
+
+// Two LDS buffers and ONE barrier per K step. While the MFMAs of step t read buffer t % 2,
+// tile t + 1 is landing in the other buffer (its loads were issued a whole step earlier);
+// after the barrier buffer t % 2 is free and the loads of tile t + 2 go out, one next to
+// each MFMA of the step's last k slice. The fragments of the next 16-wide k slice are read
+// from LDS next to the MFMAs of the current slice, one read per MFMA.
 //
 // kTile x kTile is the tile of C, kWavesM x kWavesN the wave grid over it; a wave owns
 // kBlocksM x kBlocksN blocks of 32x32. Two shapes are built: 256 with 2x4 waves (4x2 blocks
 // per wave), and 128 with 2x2 waves (2x2 blocks) for outputs of too few large tiles to fill
 // the device. Every element is summed in the same order in both.
+//
+// (The body is a device function: the host pass cannot parse the buffer-resource builtins
+// and would silently drop the launch stub of a kernel that uses them directly.)
 template <bool kGuard, int kTile, int kWavesM, int kWavesN>
-__global__ __launch_bounds__(64 * kWavesM * kWavesN)
-void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                             uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
+__device__ __forceinline__
+void GemmBf16Body(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                  uint16_t *__restrict__ C, int M, int N, int K, const XGuardArgs &g)
 {
-    constexpr int kThreads = 64 * kWavesM * kWavesN;
+    constexpr int kWaves = kWavesM * kWavesN;
     constexpr int kBlocksM = kTile / (32 * kWavesM);
     constexpr int kBlocksN = kTile / (32 * kWavesN);
-    constexpr int kBStride = kTile + 16;               // bf16 per row of the B tile in LDS: four consecutive rows start in four different 32-byte bank groups
-    constexpr int kAChunks = kTile * (kStepK / 8) / kThreads; // 16-byte pieces of the A tile per thread
-    constexpr int kBChunks = kStepK * (kTile / 8) / kThreads; // and of the B tile
-    static_assert(kBlocksN == 2, "the transposing B reads below cover two 32-column blocks per wave");
-    __shared__ __attribute__((aligned(16))) uint16_t As[2][kTile * kLdsStride];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kStepK * kBStride];
-    __shared__ uint32_t guard_word;
+    constexpr int kMfmas = kBlocksM * kBlocksN;          // per wave and 16-wide k slice
+    constexpr int kABytes = kTile * kStepK * 2;          // one A tile in LDS
+    constexpr int kBBytes = kStepK * kTile * 2;          // one B tile
+    constexpr int kALoads = kABytes / 1024 / kWaves;     // wave-wide 1 KiB loads per wave and tile
+    constexpr int kBLoads = kBBytes / 1024 / kWaves;
+    constexpr int kLoadsPerMfma = (kALoads + kBLoads) / kMfmas;
+    constexpr int kBRowBytes = kTile * 2;                // one k row of the B tile
+    constexpr int kBSlotsPerRow = kBRowBytes / 16;
+    constexpr int kBRowsPerLoad = 64 / kBSlotsPerRow;
+    constexpr uint32_t kBGranuleMask = kBRowBytes / 64 - 1;
+    static_assert(kBlocksN == 2, "the block index is XORed into the granule number as one bit");
+    static_assert(kMfmas * kLoadsPerMfma == kALoads + kBLoads && kBlocksM + kBlocksN <= kMfmas, "loads and reads pair up with the MFMAs of a slice");
+    // One LDS object for everything, the word the waves agree on a poll through included:
+    // with a second object the compiler attaches alias scopes to the LDS accesses and then
+    // makes every fragment read wait for all global loads that are on their way into LDS.
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * (kABytes + kBBytes) + 16];
+    uint32_t &guard_word = *(uint32_t *)(lds + 2 * (kABytes + kBBytes));
+    uint8_t *const As0 = lds;
+    uint8_t *const Bs0 = lds + 2 * kABytes;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
-    const uint32_t wave = tid >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave / kWavesN;
     const uint32_t wn = wave % kWavesN;
 
@@ -119,65 +153,72 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     TileOf(blockIdx.x, (uint32_t)M / kTile, (uint32_t)N / kTile, tm, tn);
     const size_t m0 = (size_t)tm * kTile, n0 = (size_t)tn * kTile;
 
-    u32x4 a_reg[kAChunks];
-    u32x4 b_vec[kBChunks];
+    // ---- global -> LDS: lane l of wave-wide load q fills LDS slot 64 q + l (16 bytes) ----
+    // Byte offsets of what each lane fetches, relative to the first element of the tile.
+    uint32_t a_off[kALoads], b_off[kBLoads];
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i) {
+        const uint32_t q = wave * kALoads + i;
+        const uint32_t line = 4 * q + (lane >> 4);
+        const uint32_t piece = (lane & 15) ^ (line & 15);   // which piece of the line belongs in this slot
+        const uint32_t row = 2 * line + (piece >> 3), kc = piece & 7;
+        a_off[i] = (row * (uint32_t)K + kc * 8) * 2;
+    }
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i) {
+        const uint32_t q = wave * kBLoads + i;
+        const uint32_t k = kBRowsPerLoad * q + lane / kBSlotsPerRow;
+        const uint32_t slot = lane % kBSlotsPerRow;
+        const uint32_t granule = (slot >> 2) ^ (((k & 3) | ((k >> 1) & 4)) & kBGranuleMask);
+        b_off[i] = (k * (uint32_t)N + granule * 32 + (slot & 3) * 8) * 2;
+    }
+    const uint16_t *const a_tile = A + m0 * (size_t)K;   // + 64 columns per step
+    const uint16_t *const b_tile = B + n0;               // + 64 rows per step
 
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < kAChunks; ++i) {
-            const uint32_t c = tid + kThreads * i;
-            const uint32_t row = c >> 3, kc = c & 7;
-            a_reg[i] = *(const u32x4 *)(A + (m0 + row) * (size_t)K + k0 + kc * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < kBChunks; ++i) {
-            const uint32_t c = tid + kThreads * i;
-            const uint32_t krow = c / (kTile / 8), chunk = c % (kTile / 8);
-            b_vec[i] = *(const u32x4 *)(B + (size_t)(k0 + krow) * N + n0 + chunk * 8);
+    // Load number idx (A first, then B) of the tile of K step `step` into buffer `buf`.
+    auto load_piece = [&](int buf, int step, int idx) {
+        if (idx < kALoads) {
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)(a_tile + (size_t)step * kStepK), 0, 0x7fffffff, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (LdsVoid *)(As0 + buf * kABytes + (wave * kALoads + idx) * 1024), 16, a_off[idx], 0, 0, 0);
+        } else {
+            const int i = idx - kALoads;
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)(b_tile + (size_t)step * kStepK * N), 0, 0x7fffffff, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (LdsVoid *)(Bs0 + buf * kBBytes + (wave * kBLoads + i) * 1024), 16, b_off[i], 0, 0, 0);
         }
     };
-
-    auto store_lds = [&](int buf) {
+    auto load_tile = [&](int buf, int step) {
 #pragma unroll
-        for (int i = 0; i < kAChunks; ++i) {
-            const uint32_t c = tid + kThreads * i;
-            const uint32_t row = c >> 3, kc = c & 7;
-            *(u32x4 *)(As[buf] + row * kLdsStride + kc * 8) = a_reg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < kBChunks; ++i) {
-            const uint32_t c = tid + kThreads * i;
-            const uint32_t krow = c / (kTile / 8), chunk = c % (kTile / 8);
-            *(u32x4 *)(Bs[buf] + krow * kBStride + chunk * 8) = b_vec[i];
-        }
+        for (int idx = 0; idx < kALoads + kBLoads; ++idx) load_piece(buf, step, idx);
     };
 
+    // ---- LDS -> fragments ----
+    // A: lane reads row a_row0 + 32 i, pieces 2 ks + (lane >> 5). 32 rows further is 16 lines
+    // further: the same swizzle bits, so one base address serves all blocks of the wave.
     const uint32_t a_row0 = 32 * kBlocksM * wm + (lane & 31);
-    const uint32_t khalf = 8 * (lane >> 5);
-    auto load_a_frags = [&](int buf, int ks, bf16x8 *fa) {
-        const uint32_t koff = ks * 16 + khalf;
-#pragma unroll
-        for (int i = 0; i < kBlocksM; ++i) fa[i] = *(const bf16x8 *)(As[buf] + (a_row0 + 32 * i) * kLdsStride + koff);
+    const uint32_t a_line = a_row0 >> 1;
+    const uint32_t a_base = a_line * 256 + (((((lane & 1) << 3) | (lane >> 5)) ^ (a_line & 15)) << 4);
+    auto read_a = [&](int buf, int ks, int i) {
+        return *(const bf16x8 *)(As0 + buf * kABytes + (a_base ^ (ks << 5)) + i * 4096);
     };
     // B sits in LDS as it sits in memory, [k][n]. The transposing read hands lane l of every 16
     // lanes the element (l & 3) of what lanes 4 * j + (l >> 2), j = 0..3, of the same 16 point
     // at: with lane r pointing at row (r >> 2), columns 4 * (r & 3) .. + 3, lane l receives
-    // column l of rows 0..3. Two reads give the eight consecutive k of one fragment.
-    const uint32_t b_tr_row = 8 * (lane >> 5) + ((lane & 15) >> 2);
-    const uint32_t b_tr_col = 64 * wn + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    auto load_b_frags = [&](int buf, int ks, bf16x8 *fb) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint16_t *p = Bs[buf] + (ks * 16 + b_tr_row) * kBStride + b_tr_col + 32 * j;
-            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)p);
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)(p + 4 * kBStride));
-            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            fb[j] = __builtin_bit_cast(bf16x8, both);
-        }
+    // column l of rows 0..3. Two reads give the eight consecutive k of one fragment. The rows
+    // a lane points at all have the same swizzle bits (k & 3 and bit 3 of k are fixed per lane).
+    const uint32_t b_row = 8 * (lane >> 5) + ((lane & 15) >> 2);
+    const uint32_t b_swz = (((lane & 15) >> 2) | ((lane >> 5) << 2)) & kBGranuleMask;
+    const uint32_t b_base = b_row * kBRowBytes + (((kBlocksN * wn) ^ b_swz) << 6) + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    auto read_b = [&](int buf, int ks, int j) {
+        const uint8_t *p = Bs0 + buf * kBBytes + ks * 16 * kBRowBytes + (b_base ^ (j << 6));
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)p);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)(p + 4 * kBRowBytes));
+        return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     };
-    auto load_frags = [&](int buf, int ks, bf16x8 *fa, bf16x8 *fb) {
-        load_a_frags(buf, ks, fa);
-        load_b_frags(buf, ks, fb);
+    auto read_frags = [&](int buf, int ks, bf16x8 *fa, bf16x8 *fb) {
+#pragma unroll
+        for (int i = 0; i < kBlocksM; ++i) fa[i] = read_a(buf, ks, i);
+#pragma unroll
+        for (int j = 0; j < kBlocksN; ++j) fb[j] = read_b(buf, ks, j);
     };
 
     f32x16 acc[kBlocksM][kBlocksN];
@@ -188,75 +229,106 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    load_global(0);
+    const int steps = K / kStepK;
+    load_tile(0, 0);
 
     if (kGuard) {
         XGuardBlock guard(g, blockIdx.x, &guard_word);
-        if (!guard.Enter()) return;
+        if (!guard.Enter()) {
+            XS_WAIT_GLOBAL_LOADS; // nothing may still be on its way into LDS when the group is gone
+            return;
+        }
     }
 
-    const int steps = K / kStepK;
-    store_lds(0);
-    load_global(steps > 1 ? kStepK : 0);
+    XS_WAIT_GLOBAL_LOADS;
     __syncthreads();
+    load_tile(1, steps > 1 ? 1 : 0);
 
-    // The loop body is branch-free (loads and LDS stores past the last tile are clamped or
-    // harmless repeats), so that it is one scheduling region. Per step and wave: 32 MFMAs in four k slices of 8; next to them
-    //   slice 0: fragment reads of slice 1
-    //   slice 1: fragment reads of slice 2, registers of tile t+1 -> the other LDS buffer
-    //   slice 2: fragment reads of slice 3, global loads of tile t+2
-    //   barrier  (the other buffer is complete, this one is no longer read)
-    //   slice 3: fragment reads of slice 0 of the NEXT tile from the other buffer
-    // Both fragment sets are double-buffered in registers (40 of them): the reads of slice
-    // s + 1 are issued before the MFMAs of slice s.
     bf16x8 fa[2][kBlocksM], fb[2][kBlocksN];
-    load_frags(0, 0, fa[0], fb[0]);
+    read_frags(0, 0, fa[0], fb[0]);
 
-    auto mfma_slice = [&](int set) {
+    // One k slice: the MFMAs on fragment set `set`, the reads of the next slice into the other
+    // set, one read after each of the first MFMAs (the small tile has fewer MFMAs than reads:
+    // there a B fragment's two reads follow one MFMA).
+    auto slice = [&](int set, int next_buf, int next_ks) {
+        XS_PIN;
+        read_frags(next_buf, next_ks, fa[set ^ 1], fb[set ^ 1]);
 #pragma unroll
         for (int i = 0; i < kBlocksM; ++i)
 #pragma unroll
             for (int j = 0; j < kBlocksN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+        constexpr int kReads = kBlocksM + 2 * kBlocksN;
+        if constexpr (kMfmas >= kReads) {
+#pragma unroll
+            for (int n = 0; n < kReads; ++n) { XS_GROUP(0x008, 1); XS_GROUP(0x100, 1); }
+        } else {
+#pragma unroll
+            for (int n = 0; n < kBlocksM; ++n) { XS_GROUP(0x008, 1); XS_GROUP(0x100, 1); }
+#pragma unroll
+            for (int n = 0; n < kBlocksN; ++n) { XS_GROUP(0x008, 1); XS_GROUP(0x100, 2); }
+        }
+        XS_PIN;
     };
 
-    for (int t = 0; t < steps; ++t) {
+    // One K step. The polling form (every kPollSteps-th step of a guarded launch) is a body of
+    // its own: its branches split the step into several scheduling regions and put the address
+    // arithmetic of the loads behind the barrier, which costs the step about 3 % - paid on one
+    // step in kPollSteps instead of on all of them. False: the work-group has to leave.
+    auto step = [&](int t, auto polling) -> bool {
+        constexpr bool kPoll = decltype(polling)::value;
         const int cur = t & 1;
-        const int k_next = (t + 2 < steps ? t + 2 : steps - 1) * kStepK;
-        // Every kPollSteps steps wave 0 asks for the preempt word here, with a vector load that
-        // is on its way during the whole step, and looks at it just before the barrier: no
-        // wave ever waits for the word alone (a scalar load at the barrier made wave 0 wait
-        // for the uncached round trip and for all of its LDS reads while the other seven
-        // waves stood at the barrier).
-        const bool poll_step = kGuard && (t % kPollSteps) == kPollSteps - 1;
+        const int next_tile = t + 2 < steps ? t + 2 : steps - 1; // past the end: a harmless repeat
+        // Wave 0 asks for the preempt word here, with a vector load that is on its way during
+        // the whole step, and looks at it just before the barrier: no wave ever waits for the
+        // word alone (a scalar load at the barrier made wave 0 wait for the uncached round trip
+        // and for all of its LDS reads while the other seven waves stood at the barrier).
         uint32_t polled = 0;
-        if (poll_step && wave == 0) polled = xguard_read_flag_begin(xguard_flag_copy(g, blockIdx.x));
+        if (kPoll && wave == 0) polled = xguard_read_flag_begin(xguard_flag_copy(g, blockIdx.x));
 
-        load_frags(cur, 1, fa[1], fb[1]);
-        mfma_slice(0);
+        slice(0, cur, 1);
+        slice(1, cur, 2);
+        slice(0, cur, 3);
 
-        load_frags(cur, 2, fa[0], fb[0]);
-        store_lds(cur ^ 1);
-        mfma_slice(1);
-
-        load_frags(cur, 3, fa[1], fb[1]);
-        load_global(k_next);
-        mfma_slice(0);
-
-        if (poll_step && wave == 0) {
+        if (kPoll && wave == 0) {
             const bool current = xguard_read_flag_end(polled) == g.epoch;
             if (lane == 0) {
                 if (!current) xguard_note_flush(g);
                 guard_word = current ? 1u : 0u;
             }
         }
-        __syncthreads(); // buffer cur^1 is complete, buffer cur is free to be overwritten
-        if (poll_step) {
-            if (guard_word == 0) return; // whole group leaves together; nothing was written
+        XS_WAIT_GLOBAL_LOADS; // this wave's part of tile t + 1 has landed
+        __syncthreads();      // tile t + 1 is complete, nobody reads buffer cur any more
+        if (kPoll) {
+            if (*(LdsVolatileWord *)&guard_word == 0) return false; // the whole group leaves together; nothing was written, no load is in flight
         }
 
-        load_frags(cur ^ 1, 0, fa[0], fb[0]);
-        mfma_slice(1);
+        // Last slice of the step: its MFMAs, next to them the first fragments of tile t + 1
+        // and the loads of tile t + 2 into the buffer that has just become free.
+        XS_PIN;
+#pragma unroll
+        for (int i = 0; i < kBlocksM; ++i)
+#pragma unroll
+            for (int j = 0; j < kBlocksN; ++j) {
+                const int n = i * kBlocksN + j;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+                if (n < kBlocksM) fa[0][n] = read_a(cur ^ 1, 0, n);
+                else if (n < kBlocksM + kBlocksN) fb[0][n - kBlocksM] = read_b(cur ^ 1, 0, n - kBlocksM);
+#pragma unroll
+                for (int l = 0; l < kLoadsPerMfma; ++l) load_piece(cur, next_tile, n * kLoadsPerMfma + l);
+                XS_PIN;
+            }
+        return true;
+    };
+
+    if constexpr (!kGuard) {
+        for (int t = 0; t < steps; ++t) step(t, std::false_type {});
+    } else {
+        for (int t0 = 0; t0 < steps; t0 += kPollSteps) {
+            const int last = min(t0 + kPollSteps, steps) - 1;
+            for (int t = t0; t < last; ++t) step(t, std::false_type {});
+            if (!step(last, std::true_type {})) return;
+        }
     }
 
     // Write-out. A lane holds one column of sixteen rows of each 32x32 block, so storing from
@@ -265,9 +337,10 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
     // rows padded by 8 bf16), and stores them as whole rows: 16 bytes per lane, eight lanes to
     // a row of 128 bytes.
     constexpr int kStripStride = 64 + 8;
-    static_assert(sizeof(As) >= (size_t)kWavesM * kWavesN * 32 * kStripStride * 2, "the A buffers hold one strip per wave");
-    __syncthreads(); // every wave has read its last fragments
-    uint16_t *strip = &As[0][0] + wave * (32 * kStripStride);
+    static_assert(2 * kABytes >= kWaves * 32 * kStripStride * 2, "the A buffers hold one strip per wave");
+    XS_WAIT_GLOBAL_LOADS; // the repeats issued by the last step land before the strips are written
+    __syncthreads();      // every wave has read its last fragments
+    uint16_t *strip = (uint16_t *)As0 + wave * (32 * kStripStride);
 #pragma unroll
     for (int i = 0; i < kBlocksM; ++i) {
 #pragma unroll
@@ -292,6 +365,14 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
         XGuardBlock guard(g, blockIdx.x, &guard_word);
         guard.Commit();
     }
+}
+
+template <bool kGuard, int kTile, int kWavesM, int kWavesN>
+__global__ __launch_bounds__(64 * kWavesM * kWavesN)
+void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                    uint16_t *__restrict__ C, int M, int N, int K, XGuardArgs g)
+{
+    GemmBf16Body<kGuard, kTile, kWavesM, kWavesN>(A, B, C, M, N, K, g);
 }
 
 
@@ -357,8 +438,9 @@ EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void 
     if (cmd == nullptr || A == nullptr || B == nullptr || C == nullptr || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
-    if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kSmallTile || N % gemm::kSmallTile || K % gemm::kStepK) {
-        XWARN("HipGemmBf16CommandCreate: M and N must be multiples of 128 and K of 64 (got %d %d %d)", M, N, K);
+    if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kSmallTile || N % gemm::kSmallTile || K % gemm::kStepK ||
+        K > gemm::kMaxK || N > gemm::kMaxK) {
+        XWARN("HipGemmBf16CommandCreate: M and N must be multiples of 128 and K of 64, K and N at most 2^22 (got %d %d %d)", M, N, K);
         return kXSchedErrorInvalidValue;
     }
     const int tile = gemm::TileFor(M, N);
