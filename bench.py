@@ -350,7 +350,7 @@ def config3(H, a):
     bg_n, fg_n = 8192, 1024
     cfg = H.Config(H.HPF, 1, H.spec(H.GEMM, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 1),
                    H.spec(H.GEMM, fg_n, 0, 1, 8, 4, 2, period_us=5000), 64, 0)
-    r = contended_run(H, cfg, a.steps, a.warmup, bg_warm=12, bg_cmds=24)
+    r = contended_run(H, cfg, a.steps, a.warmup, bg_warm=40, bg_cmds=24)
     fg = fg_summary(H, r["fg_alone"], r["fg_contended"])
     per_launch_ms = r["bg_alone_ms"]
     achieved = gemm_flops(bg_n) / (per_launch_ms * 1e-3) / 1e12
@@ -366,13 +366,15 @@ def config3(H, a):
                         "frac": achieved / MFMA_BF16_PEAK_TF, "traffic": recorded_traffic("gemm_8192_hbm_traffic.md"), "kernel": "GemmBf16Kernel",
                         "algorithmic_flops_per_launch": gemm_flops(bg_n), "avg_launch_ms": per_launch_ms}
     if not a.quick:
-        # Seven (five in the compact block) alternating rounds of 16 launches per form, after 12
-        # untimed ones each (the first launches on fresh buffers run 10-30 % long). The clock under this load moves by a
+        # Seven (five in the compact block) alternating rounds of 24 launches per form, after 40
+        # untimed ones each: the device runs this kernel against its power limit, and after an
+        # idle spell the clock first overshoots, then drops by up to 30 %, and needs some 30
+        # launches to settle. The settled clock still moves by a
         # few percent within seconds, more than the guard costs: the overheads are medians of
         # the per-round ratios (forms measured within a second of each other), the rates are
         # medians of each form.
-        rounds = [(bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 16, 12), bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 16, 12),
-                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 16, 12)) for _ in range(5 if compact else 7)]
+        rounds = [(bg_ms_per_launch(H, H.GEMM, bg_n, 1, 0, 24, 40), bg_ms_per_launch(H, H.GEMM, bg_n, 1, 2, 24, 40),
+                   bg_ms_per_launch(H, H.GEMM, bg_n, 2, 1, 24, 40)) for _ in range(5 if compact else 7)]
         mid = len(rounds) // 2
         ms_plain, ms_guard, ms_l2 = (sorted(r[i] for r in rounds)[mid] for i in range(3))
         guard_frac = sorted(1.0 - r[0] / r[1] for r in rounds)
@@ -386,7 +388,7 @@ def config3(H, a):
                          "guard_overhead_frac": guard_frac[mid], "level2_overhead_frac": l2_frac[mid],
                          "guard_overhead_frac_min_max": [guard_frac[0], guard_frac[-1]],
                          "level2_overhead_frac_min_max": [l2_frac[0], l2_frac[-1]],
-                         "rounds": len(rounds), "launches_per_round_and_form": 16}
+                         "rounds": len(rounds), "launches_per_round_and_form": 24, "untimed_launches_before_each": 40}
         line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, compact)
     return line
 
