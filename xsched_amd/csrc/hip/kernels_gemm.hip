@@ -31,7 +31,8 @@
 // checked at entry and then every kPollSteps K steps: wave 0 requests it with a vector load
 // at the top of the step and looks at it in front of the barrier the loop has anyway, so
 // nobody waits for it; a flushed tile leaves its progress byte untagged and is redone by
-// the replay. The tile is written out through LDS, whole rows of 128 bytes per eight lanes.
+// the replay. The tile is written out through LDS (64-bit stores of four rows of a column,
+// transposing reads back), whole rows of 128 bytes per eight lanes.
 // Work-group ids are remapped so that the 32 CUs of one XCD (ids equal modulo 8 land on one
 // XCD) work on neighbouring tiles and share A/B panels in that XCD's L2.
 #include <type_traits>
@@ -50,6 +51,7 @@ namespace gemm
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4 LdsS16x4;
@@ -66,14 +68,15 @@ constexpr int kXcds = 8;
 constexpr int kGroupRows = 4;       // tile rows walked together
 constexpr int kMaxK = 1 << 22;      // 32-bit byte offsets inside a 256-row panel of A
 
-/// Round-to-nearest-even to bf16, NaNs quieted: the conversion instruction of gfx950
-/// (v_cvt_pk_bf16_f32), which gives bit for bit what the integer formula
-/// (u + 0x7FFF + ((u >> 16) & 1)) >> 16, NaN -> (u >> 16) | 0x40 gives (a GPU test compares
-/// the two over products that hit ties, overflow, denormals, infinities and NaNs).
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
+/// Two floats rounded to nearest-even bf16 (NaNs quieted), `lo` in the low half: the
+/// conversion instruction of gfx950 (v_cvt_pk_bf16_f32), which gives bit for bit what the
+/// integer formula (u + 0x7FFF + ((u >> 16) & 1)) >> 16, NaN -> (u >> 16) | 0x40 gives (a GPU
+/// test compares the two over products that hit ties, overflow, denormals, infinities and
+/// NaNs).
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_rne(float lo, float hi)
 {
-    const bf16x2 pair = __builtin_convertvector(f32x2 { f, 0.f }, bf16x2);
-    return (uint16_t)__builtin_bit_cast(uint32_t, pair);
+    const bf16x2 pair = __builtin_convertvector(f32x2 { lo, hi }, bf16x2);
+    return __builtin_bit_cast(uint32_t, pair);
 }
 
 // Work-group id -> tile coordinates. Ids with equal (id % 8) run on one XCD; each
@@ -274,11 +277,15 @@ void GemmBf16Body(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B
     // One K step. The polling form (every kPollSteps-th step of a guarded launch) is a body of
     // its own: its branches split the step into several scheduling regions and put the address
     // arithmetic of the loads behind the barrier, which costs the step about 3 % - paid on one
-    // step in kPollSteps instead of on all of them. False: the work-group has to leave.
-    auto step = [&](int t, auto polling) -> bool {
+    // step in kPollSteps instead of on all of them. The last two steps have nothing left to
+    // load (`loading` false), the last one nothing to read ahead either (`reading_ahead`
+    // false): after its barrier no wave touches the tile buffers any more. False: the
+    // work-group has to leave.
+    auto step = [&](int t, auto polling, auto loading, auto reading_ahead) -> bool {
         constexpr bool kPoll = decltype(polling)::value;
+        constexpr bool kLoad = decltype(loading)::value;
+        constexpr bool kReadAhead = decltype(reading_ahead)::value;
         const int cur = t & 1;
-        const int next_tile = t + 2 < steps ? t + 2 : steps - 1; // past the end: a harmless repeat
         // Wave 0 asks for the preempt word here, with a vector load that is on its way during
         // the whole step, and looks at it just before the barrier: no wave ever waits for the
         // word alone (a scalar load at the barrier made wave 0 wait for the uncached round trip
@@ -312,52 +319,72 @@ void GemmBf16Body(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B
             for (int j = 0; j < kBlocksN; ++j) {
                 const int n = i * kBlocksN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
-                if (n < kBlocksM) fa[0][n] = read_a(cur ^ 1, 0, n);
-                else if (n < kBlocksM + kBlocksN) fb[0][n - kBlocksM] = read_b(cur ^ 1, 0, n - kBlocksM);
+                if (kReadAhead) {
+                    if (n < kBlocksM) fa[0][n] = read_a(cur ^ 1, 0, n);
+                    else if (n < kBlocksM + kBlocksN) fb[0][n - kBlocksM] = read_b(cur ^ 1, 0, n - kBlocksM);
+                }
+                if (kLoad) {
 #pragma unroll
-                for (int l = 0; l < kLoadsPerMfma; ++l) load_piece(cur, next_tile, n * kLoadsPerMfma + l);
+                    for (int l = 0; l < kLoadsPerMfma; ++l) load_piece(cur, t + 2, n * kLoadsPerMfma + l);
+                }
                 XS_PIN;
             }
         return true;
     };
+    constexpr std::true_type yes {};
+    constexpr std::false_type no {};
 
+    const int loading_steps = steps - 2; // steps whose tile t + 2 exists
     if constexpr (!kGuard) {
-        for (int t = 0; t < steps; ++t) step(t, std::false_type {});
+        for (int t = 0; t < loading_steps; ++t) step(t, no, yes, yes);
     } else {
-        for (int t0 = 0; t0 < steps; t0 += kPollSteps) {
-            const int last = min(t0 + kPollSteps, steps) - 1;
-            for (int t = t0; t < last; ++t) step(t, std::false_type {});
-            if (!step(last, std::true_type {})) return;
+        for (int t0 = 0; t0 < loading_steps; t0 += kPollSteps) {
+            const int last = min(t0 + kPollSteps, loading_steps) - 1;
+            for (int t = t0; t < last; ++t) step(t, no, yes, yes);
+            if (!step(last, yes, yes, yes)) return;
         }
     }
+    if (steps >= 2) step(steps - 2, no, no, yes);
+    step(steps - 1, no, no, no);
 
-    // Write-out. A lane holds one column of sixteen rows of each 32x32 block, so storing from
-    // the accumulators means 2-byte stores to sixteen different rows. Instead every wave turns
-    // its strips of 32 rows x 64 columns over in LDS (an area of its own in the A buffers,
-    // rows padded by 8 bf16), and stores them as whole rows: 16 bytes per lane, eight lanes to
-    // a row of 128 bytes.
-    constexpr int kStripStride = 64 + 8;
-    static_assert(2 * kABytes >= kWaves * 32 * kStripStride * 2, "the A buffers hold one strip per wave");
-    XS_WAIT_GLOBAL_LOADS; // the repeats issued by the last step land before the strips are written
-    __syncthreads();      // every wave has read its last fragments
-    uint16_t *strip = (uint16_t *)As0 + wave * (32 * kStripStride);
+    // Write-out. A lane holds one column of sixteen rows of each 32x32 block (four runs of four
+    // consecutive rows), so storing from the accumulators would mean 2-byte stores to sixteen
+    // different rows. Instead every wave turns its strips of 32 rows x 64 columns over in LDS,
+    // in an area of its own inside the tile buffers (nobody reads those any more, and nothing
+    // is on its way into them): a run of four rows of one column goes in as ONE 64-bit store
+    // (the strip is kept column-major, a column padded from 64 to 72 bytes so that the 32
+    // columns of a store fall into 32 different 8-byte bank groups), and the transposing read
+    // brings it back out row-major: pointed at four rows of columns 8 q + j (lane 4 j + q of
+    // every 16), it hands lane l row (l & 3) of columns 8 (l >> 2) + 0..3; a second read four
+    // columns further completes 16 bytes per lane, and 8 rows x 128 bytes leave per store.
+    constexpr int kStripColumnBytes = 64 + 8;
+    constexpr int kStripBytes = 64 * kStripColumnBytes;
+    static_assert(2 * kABytes >= kWaves * kStripBytes, "the A buffers hold one strip per wave");
+    uint8_t *const strip = As0 + wave * kStripBytes;
+    const uint32_t put_at = (lane & 31) * kStripColumnBytes + 4 * (lane >> 5) * 2;
+    const uint32_t l16 = lane & 15, patch = lane >> 4;   // a patch: 4 rows x 32 columns per 16 lanes
+    const uint32_t get_row = 4 * (patch >> 1), get_col = 32 * (patch & 1);
+    const uint32_t get_at = (get_col + 8 * (l16 & 3) + (l16 >> 2)) * kStripColumnBytes + get_row * 2;
 #pragma unroll
     for (int i = 0; i < kBlocksM; ++i) {
 #pragma unroll
         for (int j = 0; j < kBlocksN; ++j) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                strip[row * kStripStride + 32 * j + (lane & 31)] = f32_to_bf16_rne(acc[i][j][r]);
+            for (int run = 0; run < 4; ++run) {
+                const uint32_t lo = f32x2_to_bf16x2_rne(acc[i][j][4 * run], acc[i][j][4 * run + 1]);
+                const uint32_t hi = f32x2_to_bf16x2_rne(acc[i][j][4 * run + 2], acc[i][j][4 * run + 3]);
+                *(u32x2 *)(strip + 32 * j * kStripColumnBytes + put_at + 8 * run * 2) = u32x2 { lo, hi };
             }
         }
         const size_t row0 = m0 + 32 * kBlocksM * wm + 32 * i;
-        const size_t col0 = n0 + 64 * wn + 8 * (lane & 7);
+        const size_t col0 = n0 + 64 * wn + get_col + 8 * (l16 >> 2);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const uint32_t row = 8 * q + (lane >> 3);
-            const u32x4 v = *(const u32x4 *)(strip + row * kStripStride + 8 * (lane & 7));
-            *(u32x4 *)(C + (row0 + row) * (size_t)N + col0) = v;
+            const uint8_t *p = strip + get_at + 8 * q * 2;
+            const s16x4 left = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)p);
+            const s16x4 right = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)(p + 4 * kStripColumnBytes));
+            const s16x8 row = __builtin_shufflevector(left, right, 0, 1, 2, 3, 4, 5, 6, 7);
+            *(s16x8 *)(C + (row0 + 8 * q + get_row + (l16 & 3)) * (size_t)N + col0) = row;
         }
     }
 
