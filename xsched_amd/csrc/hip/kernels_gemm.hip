@@ -384,7 +384,9 @@ void GemmBf16Body(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B
             const s16x4 left = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)p);
             const s16x4 right = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS16x4 *)(p + 4 * kStripColumnBytes));
             const s16x8 row = __builtin_shufflevector(left, right, 0, 1, 2, 3, 4, 5, 6, 7);
-            *(s16x8 *)(C + (row0 + 8 * q + get_row + (l16 & 3)) * (size_t)N + col0) = row;
+            // (non-temporal: C is written once and not read again; left in L2 it pushes out A and B panels
+            // that the XCD's other tiles still need: 1 % of the kernel)
+            __builtin_nontemporal_store(row, (s16x8 *)(C + (row0 + 8 * q + get_row + (l16 & 3)) * (size_t)N + col0));
         }
     }
 
