@@ -195,3 +195,35 @@ def test_priority_hint_over_http_changes_who_runs(daemon_http):
             if p.poll() is None:
                 p.kill()
                 p.wait()
+
+
+def test_malformed_requests_do_not_hurt_the_daemon(daemon_http):
+    """Garbage, an oversized request, a half-sent request and an unknown method are answered
+    with an error or dropped; the daemon keeps serving."""
+    port, _ = daemon_http
+
+    def raw(data, wait=True):
+        s = socket.create_connection(("127.0.0.1", port), timeout=3)
+        try:
+            s.sendall(data)
+            if not wait:
+                return b""
+            s.settimeout(3)
+            try:
+                return s.recv(4096)
+            except OSError:
+                return b""
+        finally:
+            s.close()
+
+    assert raw(b"\x00\xff\x10 not http at all\r\n\r\n").split(b" ")[1] in (b"400", b"404")
+    assert raw(b"BREW /policy HTTP/1.1\r\nHost: x\r\n\r\n").split(b" ")[1] in (b"404", b"405", b"400")
+    assert raw(b"POST /hint HTTP/1.1\r\nContent-Length: 99999999\r\n\r\n{}").split(b" ")[1] in (b"400", b"413")
+    big = b"GET /" + b"a" * 100000 + b" HTTP/1.1\r\n\r\n"
+    try:
+        reply = raw(big)
+    except OSError:
+        reply = b""
+    assert reply == b"" or reply.split(b" ")[1] in (b"400", b"413", b"414")
+    raw(b"GET /xqueues HTT", wait=False)          # hangs up in the middle of the request line
+    assert call(port, "GET", "/policy") == (200, {"policy": 1})
