@@ -559,24 +559,31 @@ def transparent_preemption():
         alone = subprocess.run([os.path.join(lib, "shim_app_plain")] + probe_args, env=base, capture_output=True,
                                text=True, timeout=60)
         native = next_to("shim_app_plain", {}, {})
-        sock_dir = tempfile.mkdtemp(prefix="xsched-bench-")
-        server = subprocess.Popen([os.path.join(lib, "xserver"), "HPF"],
-                                  env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN"))
-        try:
-            deadline = time.time() + 5
-            while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
-                time.sleep(0.01)
-            common = {"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
-                      "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}
-            under = next_to("shim_app", dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
-                                             XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"),
-                            dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
-        finally:
-            server.terminate()
+        def under_daemon(extra):
+            """Both processes under shim + daemon + level 2; `extra` goes into all three environments."""
+            sock_dir = tempfile.mkdtemp(prefix="xsched-bench-")
+            server = subprocess.Popen([os.path.join(lib, "xserver"), "HPF"],
+                                      env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN", **extra))
             try:
-                server.wait(timeout=5)
-            except subprocess.TimeoutExpired:
-                server.kill()
+                deadline = time.time() + 5
+                while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
+                    time.sleep(0.01)
+                common = dict({"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
+                               "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}, **extra)
+                return next_to("shim_app", dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
+                                                XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"),
+                               dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
+            finally:
+                server.terminate()
+                try:
+                    server.wait(timeout=5)
+                except subprocess.TimeoutExpired:
+                    server.kill()
+
+        under = under_daemon({})
+        # The same with the three threads that relay a preemption (daemon receiver, its round
+        # thread, the load's receiver) polling for 5 ms after each message instead of sleeping.
+        under_polling = under_daemon({"XSCHED_SPIN_US": "5000"})
     except (OSError, subprocess.SubprocessError, AttributeError):
         return None
     if native is None or under is None or alone.returncode != 0:
@@ -584,7 +591,8 @@ def transparent_preemption():
     return {"workload": "fg: 256x256-thread kernel every 2 ms, 300 samples; load: 2048x256-thread guarded kernels of "
                         "5 ms back to back; two processes, plain HIP host code, percentile = sorted[floor(p*n)]",
             "fg_alone_us": percentiles(alone.stdout), "hardware_scheduling_only": native,
-            "under_xsched_shim_daemon_level2": under}
+            "under_xsched_shim_daemon_level2": under,
+            "under_xsched_shim_daemon_level2_XSCHED_SPIN_US_5000": under_polling}
 
 
 def compact_of(line):

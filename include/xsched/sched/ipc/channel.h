@@ -7,6 +7,7 @@
 #pragma once
 
 #include <atomic>
+#include <chrono>
 #include <cstddef>
 #include <cstdint>
 #include <memory>
@@ -53,6 +54,7 @@ private:
     int fd_ = -1;
     int wake_fd_ = -1;
     std::atomic_bool removed_ { false };
+    std::chrono::steady_clock::time_point last_message_ {}; // receiver thread only
 };
 
 class Channel

@@ -16,10 +16,16 @@ XSERVER = os.path.join(ROOT, "xsched_amd", "lib", "xserver")
 CLIENT = os.path.join(ROOT, "tests", "daemon_client.py")
 
 
-@pytest.fixture()
-def daemon():
+@pytest.fixture(params=["blocking", "polling"])
+def daemon(request, monkeypatch):
+    """The daemon and its clients with receivers that block at once (the default) and with
+    receivers that poll for 3 ms after each message (XSCHED_SPIN_US)."""
     if not os.path.exists(XSERVER):
         pytest.fail("xserver has not been built")
+    if request.param == "polling":
+        monkeypatch.setenv("XSCHED_SPIN_US", "3000")
+    else:
+        monkeypatch.delenv("XSCHED_SPIN_US", raising=False)
     sock_dir = tempfile.mkdtemp(prefix="xsched-test-")
     env = dict(os.environ, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="INFO")
     proc = subprocess.Popen([XSERVER, "HPF"], env=env, stderr=subprocess.PIPE, text=True)

@@ -12,6 +12,7 @@
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/def.h"
 #include "xsched/sched/ipc/channel.h"
+#include "spin.h"
 
 namespace xsched::sched::ipc
 {
@@ -92,6 +93,21 @@ std::unique_ptr<Message> Node::Receive()
 {
     if (type_ != NodeType::kReceiver || removed_.load()) return nullptr;
     std::vector<char> buf(kMaxMessageSize);
+    // Poll for a while after the last message before blocking (off unless XSCHED_SPIN_US is set).
+    const auto window = SpinWindow();
+    if (window.count() > 0) {
+        const auto give_up = last_message_ + window;
+        while (std::chrono::steady_clock::now() < give_up && !removed_.load(std::memory_order_relaxed)) {
+            ssize_t n = recv(fd_, buf.data(), buf.size(), MSG_DONTWAIT);
+            if (n >= 0) {
+                last_message_ = std::chrono::steady_clock::now();
+                buf.resize((size_t)n);
+                return std::make_unique<Message>(std::move(buf));
+            }
+            if (errno != EAGAIN && errno != EWOULDBLOCK && errno != EINTR) return nullptr;
+            __builtin_ia32_pause();
+        }
+    }
     while (true) {
         pollfd fds[2] = { { fd_, POLLIN, 0 }, { wake_fd_, POLLIN, 0 } };
         int rc = poll(fds, 2, -1);
@@ -100,6 +116,7 @@ std::unique_ptr<Message> Node::Receive()
         if (!(fds[0].revents & POLLIN)) continue;
         ssize_t n = recv(fd_, buf.data(), buf.size(), 0);
         if (n < 0) { if (errno == EINTR || errno == EAGAIN) continue; return nullptr; }
+        last_message_ = std::chrono::steady_clock::now();
         buf.resize((size_t)n);
         return std::make_unique<Message>(std::move(buf));
     }

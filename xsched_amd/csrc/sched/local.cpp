@@ -10,6 +10,7 @@
 // sched/src/scheduler/local.cpp:42-446; tests replay recorded event scripts through both.
 #include <algorithm>
 #include <array>
+#include <atomic>
 #include <condition_variable>
 #include <map>
 #include <mutex>
@@ -23,6 +24,7 @@
 #include "xsched/sched/policy/policy.h"
 #include "xsched/sched/protocol/status.h"
 #include "xsched/sched/scheduler/local.h"
+#include "spin.h"
 
 using namespace xsched::protocol;
 
@@ -58,6 +60,7 @@ public:
     void Put(EventPtr event)
     {
         { std::lock_guard<std::mutex> g(mu_); waiting_.push_back(std::move(event)); }
+        n_put_.fetch_add(1, std::memory_order_release);
         cv_.notify_one();
     }
 
@@ -78,6 +81,18 @@ public:
     void Take(std::vector<EventPtr> *batch)
     {
         batch->clear();
+        // Poll for a while after the last batch before blocking (off unless XSCHED_SPIN_US is
+        // set); alarms are looked at by the blocking path, which the poll leaves in time.
+        const auto window = SpinWindow();
+        if (window.count() > 0) {
+            const uint64_t seen = n_taken_;
+            auto give_up = last_batch_ + window;
+            {
+                std::lock_guard<std::mutex> g(mu_);
+                if (!alarms_.empty() && alarms_.top() < give_up) give_up = alarms_.top();
+            }
+            while (n_put_.load(std::memory_order_acquire) == seen && Clock::now() < give_up) __builtin_ia32_pause();
+        }
         std::unique_lock<std::mutex> g(mu_);
         while (waiting_.empty()) {
             if (alarms_.empty()) { cv_.wait(g); continue; }
@@ -88,12 +103,17 @@ public:
             return;
         }
         batch->swap(waiting_);
+        n_taken_ = n_put_.load(std::memory_order_acquire); // under mu_: every Put() counted so far is in the batch
+        last_batch_ = Clock::now();
     }
 
 private:
     std::mutex mu_;
     std::condition_variable cv_;
     std::vector<EventPtr> waiting_;
+    std::atomic<uint64_t> n_put_ { 0 };
+    uint64_t n_taken_ = 0;          // round thread only
+    TimePoint last_batch_ {};       // round thread only
     std::priority_queue<TimePoint, std::vector<TimePoint>, std::greater<TimePoint>> alarms_;
 };
 
