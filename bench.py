@@ -390,7 +390,38 @@ def config3(H, a):
                          "level2_overhead_frac_min_max": [l2_frac[0], l2_frac[-1]],
                          "rounds": len(rounds), "launches_per_round_and_form": 24, "untimed_launches_before_each": 40}
         line["preempt_us"] = preempt_block(H, H.GEMM, bg_n, compact)
+        line["vendor_library"] = vendor_gemm(bg_n, tf(ms_plain))
     return line
+
+
+def vendor_gemm(n, ours_tflops):
+    """The vendor library's bf16 GEMM of the same shape on the same box, for scale: hipBLASLt
+    through torch.matmul, 40 launches after 40 untimed ones, median of five rounds. None when
+    torch has no GPU."""
+    try:
+        import torch
+        if not torch.cuda.is_available():
+            return None
+        a = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+        b = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+        for _ in range(40):
+            c = a @ b
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        rounds = []
+        for _ in range(5):
+            e0.record()
+            for _ in range(40):
+                c = a @ b  # noqa: F841
+            e1.record()
+            torch.cuda.synchronize()
+            rounds.append(e0.elapsed_time(e1) / 40)
+        ms = sorted(rounds)[2]
+        vendor = gemm_flops(n) / ms / 1e9
+        return {"what": "hipBLASLt through torch.matmul, bf16 %d^3, same process" % n, "ms_per_launch": ms,
+                "TFLOPs": vendor, "this_kernel_over_vendor": ours_tflops / vendor}
+    except Exception as e:  # informational only
+        return {"what": "unavailable: %s" % e}
 
 
 def config4(H, a):
@@ -608,7 +639,7 @@ def compact_of(line):
     if "preempt_us" in line:
         keep["preempt_us"] = {k: v for k, v in line["preempt_us"].items()
                               if k.startswith("level2_device_drain") or k.startswith("level2_resume") or k.startswith("level2_suspend")}
-    for k in ("deadline_miss_rate", "bit_exact"):
+    for k in ("deadline_miss_rate", "bit_exact", "vendor_library"):
         if k in line:
             keep[k] = line[k]
     if "per_priority_latency_us" in line:
