@@ -34,9 +34,26 @@ def check_axpy(b, which, q, lane_id, n, seed=0, first=0, count=None):
     x = oracle.fill_uniform(seed, s0, first, count)
     y = oracle.fill_uniform(seed, s1, first, count)
     want = oracle.axpy(0.5, x, y, applied)
-    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), \
-        f"axpy lane {lane_id}: output differs from {applied} uninterrupted applications"
+    if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+        raise AssertionError(f"axpy lane {lane_id}: output differs from {applied} uninterrupted applications: "
+                             + describe_axpy_mismatch(got, x, y, applied, first))
     return applied
+
+
+def describe_axpy_mismatch(got, x, y, applied, first):
+    """Which 1024-element chunks differ, and whether they hold one application more or fewer."""
+    bad = np.flatnonzero(got.view(np.uint32) != oracle.axpy(0.5, x, y, applied).view(np.uint32))
+    chunks = np.unique((bad + first) // 1024)
+    notes = []
+    for k in (applied - 2, applied - 1, applied + 1, applied + 2):
+        if k < 0:
+            continue
+        alt = oracle.axpy(0.5, x, y, k)
+        notes.append("%d of them equal %d applications" % (int(np.sum(got[bad].view(np.uint32) == alt[bad].view(np.uint32))), k))
+    runs = np.split(chunks, np.flatnonzero(np.diff(chunks) != 1) + 1)
+    spans = ["%d-%d" % (r[0], r[-1]) if len(r) > 1 else str(r[0]) for r in runs[:12]]
+    return "%d elements in %d chunks of 1024 (%s%s); %s" % (len(bad), len(chunks), ", ".join(spans),
+                                                           ", ..." if len(runs) > 12 else "", "; ".join(notes))
 
 
 def check_hist(b, which, q, lane_id, n, seed=0):

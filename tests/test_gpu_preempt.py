@@ -320,6 +320,58 @@ def test_launches_of_a_flushed_epoch_do_not_run(xs, gpu, kind):
     assert np.array_equal(ran, after), "a launch of the next epoch did not run exactly once"
 
 
+def test_first_commands_of_fresh_queues_on_non_blocking_streams_are_applied_once(xs, gpu):
+    """A queue's first guarded command gets a progress map in memory that was allocated a
+    moment ago. Whatever prepares that memory must be ordered before the command's kernel on
+    the queue's own stream: a stream created with hipStreamNonBlocking does not wait for work
+    on the null stream (hipMemset on device memory returns before its fill has run, and the
+    fills of several queues wait for each other there). Cleared late, a map loses the bytes of
+    the first work-groups, and a replay applies those work-groups a second time. Eight fresh
+    queues on fresh non-blocking streams start their first commands together, each is
+    suspended and resumed while its kernel runs: every element holds exactly one application."""
+    import ctypes
+    torch = gpu
+    hip = ctypes.CDLL("libamdhip64.so")
+    n, n_queues, trials = 1 << 24, 8, 4
+    print(f"case fresh-queues-first-command n={n} queues={n_queues} trials={trials}", flush=True)
+    x_h = oracle.fill_uniform(31, 1, 0, n)
+    y_h = oracle.fill_uniform(31, 2, 0, n)
+    want = oracle.axpy(0.5, x_h, y_h, 1).view(np.uint32)
+    x = torch.from_numpy(x_h).cuda()
+    p = xs.preempt()
+    replays = 0
+    for trial in range(trials):
+        ys = [torch.from_numpy(y_h.copy()).cuda() for _ in range(n_queues)]
+        torch.cuda.synchronize()
+        streams, hwqs, xqs = [], [], []
+        for _ in range(n_queues):
+            stream = ctypes.c_void_p()
+            assert hip.hipStreamCreateWithFlags(byref(stream), 1) == 0   # hipStreamNonBlocking
+            streams.append(stream)
+            hwqs.append(xs.hip_queue_create(stream.value))
+            xqs.append(xs.xqueue_create(hwqs[-1], 2))
+        cmds = [axpy_cmd(xs, 0.5, x, y, n, 1) for y in ys]
+        for xq, cmd in zip(xqs, cmds):
+            xs.check(p.XQueueSubmit(xq, cmd))
+        for _ in range(1 + trial % 2):
+            for xq in xqs:
+                xs.check(p.XQueueSuspend(xq, 0))
+            for xq in xqs:
+                xs.check(p.XQueueResume(xq, 0))
+        for xq in xqs:
+            xs.check(p.XQueueWaitAll(xq))
+        replays += sum(hip_stats(xs, hwq)[1] for hwq in hwqs)
+        got = [y.cpu().numpy().view(np.uint32) for y in ys]
+        for xq, hwq, stream in zip(xqs, hwqs, streams):
+            xs.check(p.XQueueDestroy(xq))
+            xs.check(p.HwQueueDestroy(hwq))
+            assert hip.hipStreamDestroy(stream) == 0
+        for i, g in enumerate(got):
+            assert np.array_equal(g, want), f"trial {trial}, queue {i}: {int((g != want).sum())} elements differ from one application"
+    print("replays", replays, flush=True)
+    assert replays > 0, "no command was replayed: the test did not exercise level 2"
+
+
 def test_user_written_guarded_kernel_is_flushed_and_replayed_exactly_once(xs, gpu):
     """A kernel outside the library (tests/user_guarded_kernel.hip: in place, not idempotent)
     with the guard compiled in, submitted through HipGuardedKernelCommandCreate: suspended and

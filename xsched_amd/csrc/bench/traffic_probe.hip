@@ -40,6 +40,7 @@ int main(int argc, char **argv)
     CHECK_HIP(hipMalloc((void **)&y, n * 4));
     CHECK_HIP(hipMemset(x, 0, n * 4));
     CHECK_HIP(hipMemset(y, 0, n * 4));
+    CHECK_HIP(hipDeviceSynchronize()); // hipMemset returns before the fill has run; the stream below would not wait for it
     hipStream_t stream;
     CHECK_HIP(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
 

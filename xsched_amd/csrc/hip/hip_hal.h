@@ -69,10 +69,10 @@ public:
     /// Returns once the latest Deactivate() is visible to the device.
     void WaitFlagWritten(hipStream_t op_stream);
 
-    /// A progress map with a fresh generation tag. The map is not cleared: bytes of
-    /// earlier owners carry other tags. Only when the 8-bit tag wraps does the caller
-    /// have to clear it (needs_clear). Blocks on the device only when a new arena has
-    /// to be allocated.
+    /// A progress map with a fresh generation tag. The map is normally not cleared: bytes of
+    /// earlier owners carry other tags. The caller has to clear it, in the order of its own
+    /// stream, for the slot's first owner (fresh memory) and whenever the 8-bit tag wraps
+    /// (needs_clear). Blocks on the device only when a new arena has to be allocated.
     Slot AcquireSlot();
     void ReleaseSlot(const Slot &slot);
     uint64_t SlotsInUse();

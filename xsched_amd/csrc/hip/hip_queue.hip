@@ -211,8 +211,11 @@ GuardState::Slot GuardState::AcquireSlot()
         RelaxedCaptureScope relaxed;
         uint8_t *arena = nullptr;
         const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
+        // Not cleared here: hipMemset() on device memory returns before the fill has run,
+        // and a kernel launched afterwards on a non-blocking stream overtakes it (its first
+        // progress bytes were then wiped, and a replay applied those work-groups again).
+        // Every slot is cleared in the order of its owner's stream instead, see Enqueue().
         HIP_ASSERT(hipMalloc((void **)&arena, bytes));
-        HIP_ASSERT(hipMemset(arena, 0, bytes));
         arenas_.push_back(arena);
         for (uint32_t i = 0; i < kSlotsPerArena; ++i) {
             free_slots_.push_back((uint32_t)slot_ptr_.size());
@@ -225,7 +228,9 @@ GuardState::Slot GuardState::AcquireSlot()
     free_slots_.pop_back();
     slot.done = slot_ptr_[slot.index];
     uint32_t gen = slot_gen_[slot.index] + 1;
-    if (gen > 255) { gen = 1; slot.needs_clear = true; } // tags of 255 owners ago could collide
+    if (gen > 255) gen = 1;
+    // first owner: the memory is as hipMalloc left it; later: tags of 255 owners ago could collide
+    slot.needs_clear = gen == 1;
     slot_gen_[slot.index] = gen;
     slot.gen = gen;
     in_use_++;
@@ -302,9 +307,16 @@ HipGuardedCommand::~HipGuardedCommand()
     if (slot_.done != nullptr) guard_state_->ReleaseSlot(slot_);
 }
 
+// Zeroes one progress-map slot, in stream order in front of its owner's first launch.
+__global__ __launch_bounds__(256) void ClearSlotKernel(uint4 *slot)
+{
+    slot[blockIdx.x * 256 + threadIdx.x] = uint4 { 0, 0, 0, 0 };
+}
+
 // Level 1 (or guard_mode 0): the plain kernel, nothing else on the stream.
-// Level 2: the first launch takes a progress map (no clearing: its generation tag is
-// new); every launch (first or replay) carries the epoch current at enqueue time.
+// Level 2: the first launch takes a progress map (cleared only for the slot's first owner
+// and every 255th after it: otherwise the generation tag is new); every launch (first or
+// replay) carries the epoch current at enqueue time.
 hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
 {
     const bool level2 = q.Level() >= kPreemptLevelDeactivate;
@@ -325,7 +337,10 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
             guard_state_ = q.Guard();
             slot_ = guard_state_->AcquireSlot();
             if (slot_.needs_clear) {
-                hipError_t err = hipMemsetAsync(slot_.done, 0, GuardState::kSlotBytes, q.Stream());
+                // a kernel, not hipMemsetAsync: a stream under capture records no memset node
+                static_assert(GuardState::kSlotBytes % (16 * 256) == 0, "one 16-byte store per thread");
+                ClearSlotKernel<<<dim3((unsigned)(GuardState::kSlotBytes / 16 / 256)), dim3(256), 0, q.Stream()>>>((uint4 *)slot_.done);
+                hipError_t err = hipGetLastError();
                 if (err != hipSuccess) return err;
             }
         }
