@@ -6,9 +6,7 @@
 #pragma once
 
 #include <memory>
-#include <thread>
 
-#include "xsched/sched/ipc/channel.h"
 #include "xsched/sched/scheduler/scheduler.h"
 
 namespace xsched::sched
@@ -18,19 +16,17 @@ class GlobalScheduler : public Scheduler
 {
 public:
     GlobalScheduler();
-    virtual ~GlobalScheduler();
+    ~GlobalScheduler() override;
 
-    virtual void Run() override;
-    virtual void Stop() override;
-    virtual void RecvEvent(std::shared_ptr<const Event> event) override;
+    void Run() override;
+    void Stop() override;
+    void RecvEvent(std::shared_ptr<const Event> event) override;
 
 private:
-    void Worker();
-
-    ipc::ChannelKey client_key_ = 0;
-    std::unique_ptr<std::thread> thread_;
-    std::unique_ptr<ipc::Node> recv_chan_;
-    std::unique_ptr<ipc::Node> send_chan_;
+    /// The two ends of the conversation with the daemon and the thread that listens;
+    /// exists between Run() and Stop().
+    struct DaemonLink;
+    std::unique_ptr<DaemonLink> link_;
 };
 
 } // namespace xsched::sched
