@@ -163,6 +163,7 @@ GuardState::GuardState(int device): device_(device)
     }
     HIP_ASSERT(hipExtMallocWithFlags((void **)&flag_dev_, bytes, hipDeviceMallocFinegrained));
     HIP_ASSERT(hipMemset(flag_dev_, 0, bytes));
+    // hipMemset returns before its fills have run: nothing may be launched against the words before this
     HIP_ASSERT(hipDeviceSynchronize());
 
     const std::string how = GetEnv("XSCHED_HIP_FLAG_WRITE");
