@@ -8,7 +8,8 @@
 //   shim_app --load SECONDS       device-filling kernels back to back on one stream
 //   shim_app --probe N PERIOD_US  a short kernel every PERIOD_US, launch-to-completion latency
 //   shim_app --leak               leaves main() with streams, events and memory never released
-//   shim_app --load-guarded SECONDS  like --load with a kernel that has the XSched guard compiled in
+//   shim_app --load-guarded SECONDS [SPLIT]  like --load with a kernel that has the XSched guard compiled in
+//                                 (SPLIT times as many work-groups, each that much shorter)
 //
 // The guard (xsched/hip/guard.h) is the one thing here that belongs to XSched: a kernel with
 // an XGuardArgs as its last parameter. The program launches it like any other kernel and
@@ -157,11 +158,13 @@ void AffineGuarded(float *y, float b, uint32_t n, XGuardArgs g)
     guard.Commit();
 }
 
-static int LoadGuarded(double seconds)
+// `split` > 1 cuts the same work into `split` times as many work-groups, each that much
+// shorter: what a flush throws away is the progress of the work-groups that were running.
+static int LoadGuarded(double seconds, uint32_t split)
 {
     hipStream_t s;
     uint32_t *runs;
-    constexpr uint32_t kGroups = 2048;
+    const uint32_t kGroups = 2048 * split;
     CHECK(hipStreamCreate(&s));
     CHECK(hipMalloc(&runs, kGroups * 4));
     CHECK(hipMemset(runs, 0, kGroups * 4));
@@ -169,7 +172,7 @@ static int LoadGuarded(double seconds)
     const auto t0 = std::chrono::steady_clock::now();
     uint32_t kernels = 0;
     while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < seconds) {
-        for (int i = 0; i < 8; ++i) BusyGuarded<<<kGroups, 256, 0, s>>>(runs, 92160, XGuardArgs {});   // about 5 ms: long enough that waiting for its end hurts
+        for (int i = 0; i < 8; ++i) BusyGuarded<<<kGroups, 256, 0, s>>>(runs, 92160 / split, XGuardArgs {});   // about 5 ms: long enough that waiting for its end hurts
         CHECK(hipStreamSynchronize(s));
         kernels += 8;
     }
@@ -257,7 +260,7 @@ int main(int argc, char **argv)
     if (argc >= 2 && strcmp(argv[1], "--leak") == 0) return Leak();
     if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
     if (argc >= 3 && strcmp(argv[1], "--load") == 0) return Load(atof(argv[2]));
-    if (argc >= 3 && strcmp(argv[1], "--load-guarded") == 0) return LoadGuarded(atof(argv[2]));
+    if (argc >= 3 && strcmp(argv[1], "--load-guarded") == 0) return LoadGuarded(atof(argv[2]), argc >= 4 ? (uint32_t)atoi(argv[3]) : 1u);
     if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));
     const char *module_path = argc >= 2 ? argv[1] : nullptr;
     // Under the kernel-trace profiler the program without any library of this repository in it
