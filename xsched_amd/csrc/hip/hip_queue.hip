@@ -48,6 +48,25 @@ int64_t SyncSpinMicros()
     return us;
 }
 
+namespace
+{
+/// Polls the event for up to `spin_us` (no system call, no sleep / wake latency); true once
+/// it has completed, false when the time is up (the caller then blocks in the driver, so a
+/// long wait does not burn a core).
+bool PollEvent(hipEvent_t ev, int64_t spin_us)
+{
+    if (spin_us <= 0) return false;
+    const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_us);
+    for (int probes = 1;; ++probes) {
+        const hipError_t err = hipEventQuery(ev);
+        if (err == hipSuccess) return true;
+        XASSERT(err == hipErrorNotReady, "hipEventQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
+        if ((probes & 7) == 0 && std::chrono::steady_clock::now() >= deadline) return false;
+        __builtin_ia32_pause();
+    }
+}
+} // namespace
+
 // ---- EventPool ---------------------------------------------------------------
 
 EventPool &EventPool::Instance()
@@ -282,20 +301,9 @@ void HipCommand::Synchronize()
 {
     XASSERT(marker_ != nullptr, "Synchronize() needs EnableSynchronization() before launch");
     RelaxedCaptureScope relaxed;
-    const int64_t spin_us = SyncSpinMicros();
-    if (spin_us > 0) {
-        const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_us);
-        int probes = 0;
-        while (true) {
-            hipError_t err = hipEventQuery(marker_);
-            if (err == hipSuccess) {
-                if (queue_) queue_->n_wait_polled.fetch_add(1, std::memory_order_relaxed);
-                return;
-            }
-            XASSERT(err == hipErrorNotReady, "hipEventQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
-            if ((++probes & 7) == 0 && std::chrono::steady_clock::now() >= deadline) break;
-            __builtin_ia32_pause();
-        }
+    if (PollEvent(marker_, SyncSpinMicros())) {
+        if (queue_) queue_->n_wait_polled.fetch_add(1, std::memory_order_relaxed);
+        return;
     }
     if (queue_) queue_->n_wait_blocked.fetch_add(1, std::memory_order_relaxed);
     HIP_ASSERT(hipEventSynchronize(marker_));
@@ -471,16 +479,7 @@ void HipQueue::Synchronize()
     hipEvent_t marker = EventPool::Instance().Pop();
     hipError_t err = hipEventRecord(marker, stream_);
     XASSERT(err == hipSuccess, "hipEventRecord failed: %d (%s)", (int)err, hipGetErrorString(err));
-    const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(SyncSpinMicros());
-    bool done = false;
-    for (int probes = 1; !done; ++probes) {
-        err = hipEventQuery(marker);
-        if (err == hipSuccess) { done = true; break; }
-        XASSERT(err == hipErrorNotReady, "hipEventQuery failed: %d (%s)", (int)err, hipGetErrorString(err));
-        if ((probes & 7) == 0 && std::chrono::steady_clock::now() >= give_up) break;
-        __builtin_ia32_pause();
-    }
-    if (!done) HIP_ASSERT(hipEventSynchronize(marker));
+    if (!PollEvent(marker, SyncSpinMicros())) HIP_ASSERT(hipEventSynchronize(marker));
     EventPool::Instance().Push(marker);
 }
 
