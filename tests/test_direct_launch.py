@@ -171,3 +171,69 @@ def test_environment_switch():
                              text=True, timeout=60, check=True).stdout.split()
         assert out[0] == "5"
         assert (int(out[1]) > 0) == want_direct
+
+
+def test_a_wait_on_a_queue_paused_after_a_direct_launch_ends_with_the_resume(xs):
+    """The submitter launches, the queue is paused before the submitter starts to wait, and it
+    is resumed a moment later: the wait returns with the resume. (The launcher stands by for
+    callers that launch themselves; a waiter that left the device to it whenever the queue
+    was paused got its answer only when the stand-by of 500 us had passed.) The smallest of
+    several trials is what is checked: it cannot be lowered by a busy machine."""
+    p, h = xs.preempt(), xs.halhost()
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+    hwq = xs.host_queue_create()
+    xq = xs.xqueue_create(hwq)
+    xs.check(p.XQueueSetLaunchConfig(xq, 8, 4))
+    n = 1024
+    ones = np.ones(n, np.float32); acc = np.zeros(n, np.float32)
+    waits = []
+    for trial in range(12):
+        wait_idle(xs, xq)
+        cmd = c_uint64()
+        xs.check(h.HostVecAddCommandCreate(byref(cmd), acc.ctypes.data, ones.ctypes.data, acc.ctypes.data, n, 0))
+        before = direct_count(xs, xq)
+        xs.check(p.XQueueSubmit(xq, cmd.value))
+        assert direct_count(xs, xq) == before + 1, "the command was not launched by the submitter"
+        xs.check(p.XQueueSuspend(xq, 0))
+        resumer = threading.Thread(target=lambda: (time.sleep(0.00005), xs.check(p.XQueueResume(xq, 0))))
+        t0 = time.perf_counter()
+        resumer.start()
+        xs.check(p.XQueueWaitAll(xq))
+        waits.append(time.perf_counter() - t0)
+        resumer.join()
+        assert np.all(acc == trial + 1)
+    print("waits (us):", [round(w * 1e6) for w in waits])
+    assert min(waits) < 400e-6, "every wait took as long as the launcher's stand-by"
+    xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hwq))
+
+
+def test_a_command_launched_by_the_launcher_is_waited_for_by_the_launcher_at_once(xs):
+    """Submitted while the queue is paused, a command is launched by the launcher once the
+    queue runs again, and the submitter sleeps on the completion number: the launcher has to
+    wait for the device right away, not stand by as it does after a submitter's own launch."""
+    p, h = xs.preempt(), xs.halhost()
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+    hwq = xs.host_queue_create()
+    xq = xs.xqueue_create(hwq)
+    xs.check(p.XQueueSetLaunchConfig(xq, 8, 4))
+    n = 1024
+    ones = np.ones(n, np.float32); acc = np.zeros(n, np.float32)
+    waits = []
+    for trial in range(12):
+        wait_idle(xs, xq)
+        cmd = c_uint64()
+        xs.check(h.HostVecAddCommandCreate(byref(cmd), acc.ctypes.data, ones.ctypes.data, acc.ctypes.data, n, 0))
+        xs.check(p.XQueueSuspend(xq, 0))
+        before = direct_count(xs, xq)
+        xs.check(p.XQueueSubmit(xq, cmd.value))
+        assert direct_count(xs, xq) == before, "a paused queue launched on the submitter's thread"
+        resumer = threading.Thread(target=lambda: (time.sleep(0.00005), xs.check(p.XQueueResume(xq, 0))))
+        t0 = time.perf_counter()
+        resumer.start()
+        xs.check(p.XQueueWaitAll(xq))
+        waits.append(time.perf_counter() - t0)
+        resumer.join()
+        assert np.all(acc == trial + 1)
+    print("waits (us):", [round(w * 1e6) for w in waits])
+    assert min(waits) < 400e-6, "every wait took as long as the launcher's stand-by"
+    xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hwq))

@@ -3,6 +3,8 @@
 // the rule each block keeps).
 #include <chrono>
 
+#include <sys/prctl.h>
+
 #include "ring_queue.h"
 #include "xsched/utils/env.h"
 #include "xsched/utils/xassert.h"
@@ -18,7 +20,8 @@ namespace
 constexpr size_t kInitialRingSlots = 256;
 constexpr int64_t kSpinMicros = 150; // a waiter polls this long before it sleeps
 constexpr int64_t kStandByMicros = 500;      // how long the launcher leaves the device to callers that launch themselves
-constexpr int64_t kStandBySliceMicros = 100; // how often it looks whether their commands have retired
+constexpr int64_t kStandBySliceMicros = 25;  // how often it looks whether their commands have retired
+constexpr unsigned long kLauncherTimerSlackNanos = 1000; // timed waits of the launcher end on time (the default slack is 50 us)
 
 size_t PowerOfTwoAtLeast(size_t n)
 {
@@ -47,6 +50,7 @@ RingXQueue::RingXQueue(std::shared_ptr<HwQueue> hwq, XPreemptLevel level, int64_
     // the constructor returns once that has happened (async_xqueue.cpp:25-29).
     std::atomic<bool> up { false };
     launcher_ = std::thread([this, &up]() {
+        (void)prctl(PR_SET_TIMERSLACK, kLauncherTimerSlackNanos, 0, 0, 0);
         kHwQueue->OnXQueueCreate();
         up.store(true, std::memory_order_release);
         up.notify_all();
@@ -113,7 +117,8 @@ void RingXQueue::Submit(std::shared_ptr<HwCommand> hw_cmd)
         // The launcher is parked and nothing waits in the ring: launching here keeps
         // submission order, and the ring lock keeps it so against other submitters.
         const bool launched = caller_may_launch_ && parked_ && ring_count_ == 0 && TryLaunchOnCaller(hw_cmd);
-        if (!launched) PushLocked(Slot::kCommand, wait_for_launch ? hw_cmd : std::move(hw_cmd));
+        if (launched) caller_launched_ = true;
+        else PushLocked(Slot::kCommand, wait_for_launch ? hw_cmd : std::move(hw_cmd));
         // A launcher that already stands by for callers (see NextStep) needs no wake-up for a
         // command that is on the device already; it looks again by itself.
         wake = parked_ && (!launched || launcher_owed_nothing);
@@ -142,12 +147,15 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
             }
         }
         out->cmd = nullptr;
-        if (owed_ != Owed::kNothing && caller_may_launch_ && stood_by_for_ != handed_over_.load(std::memory_order_acquire)) {
+        if (owed_ != Owed::kNothing && caller_launched_) {
             // Callers launch and wait for themselves: the launcher stands by, still parked as
             // far as submitters are concerned, until what they launched has retired (then the
             // waits it owes return at once), something is queued for it, or the stand-by has
             // lasted long enough that nobody seems to be waiting. It does not ask the device
             // meanwhile: a second thread polling the runtime slows the callers' launches.
+            // Only for launches of callers: after a launch of its own the launcher is the one
+            // who has to wait for the device, a submitter that waits for that command sleeps
+            // on the completion number until the launcher has done so.
             const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(kStandByMicros);
             parked_ = true;
             while (ring_count_ == 0 && retired_.load(std::memory_order_acquire) < handed_over_.load(std::memory_order_acquire) &&
@@ -157,7 +165,7 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
                 ring_cv_.wait_until(g, std::chrono::system_clock::now() + std::chrono::microseconds(kStandBySliceMicros));
             }
             parked_ = false;
-            stood_by_for_ = handed_over_.load(std::memory_order_acquire);
+            caller_launched_ = false;
             if (ring_count_ != 0) continue;
         }
         if (owed_ == Owed::kBatchThenDrain) { owed_ = Owed::kDrain; return Step::kBatch; }
@@ -257,9 +265,12 @@ void RingXQueue::WaitAll()
     if (ticket < 0 || retired_.load(std::memory_order_acquire) >= ticket) return;
     if (caller_may_launch_ && handed_over_.load(std::memory_order_acquire) >= ticket) {
         // Everything is on the device already: the caller asks the device itself instead of
-        // waiting for the launcher to wake up and do so. One thread asks at a time.
+        // waiting for the launcher to wake up and do so. One thread asks at a time. A queue
+        // that was paused after the launch is waited for as well (AwaitQueue holds until it
+        // runs again): the launcher stands by for this caller and would only look after the
+        // whole stand-by has passed.
         Guard g(win_mu_);
-        if (!queue_wait_active_ && run_ == Run::kRunning) AwaitQueue(g);
+        if (!queue_wait_active_ && run_ != Run::kStopped) AwaitQueue(g);
     }
     AwaitRetired(ticket);
 }

@@ -91,7 +91,7 @@ private:
     size_t ring_head_ = 0, ring_count_ = 0;
     Owed owed_ = Owed::kNothing;
     bool parked_ = false;
-    int64_t stood_by_for_ = -1;         // handed_over_ at the launcher's last stand-by
+    bool caller_launched_ = false;      // a submitter has launched since the launcher last stood by
     XQueueState reported_ = kQueueStateIdle;
     uint64_t idle_round_ = 0;
 
