@@ -45,6 +45,11 @@ public:
     /// launched on the submitting thread, i.e. its BeforeLaunch() never blocks.
     virtual bool DirectLaunchable() { return false; }
 
+    /// Extension, same purpose: true when the device is known to have completed this
+    /// (synchronizable, launched) command; never blocks. A submitter that finds the window
+    /// full asks the oldest marker this way before it gives the launch to the launch thread.
+    virtual bool CompletedWithoutWaiting() { return false; }
+
     /// 1-based submission index inside its XQueue; -1 before submission.
     int64_t GetIdx() const { return idx_; }
     void SetIdx(int64_t idx) { idx_ = idx; }

@@ -5,6 +5,7 @@
 //
 //   shim_app [module.co]          the checks (module checks only if a code object is given)
 //   shim_app --bench N            N launches of a tiny kernel on one stream, us per launch
+//   shim_app --bench-paced N GAP_US  N launches with GAP_US of host work between them: cost of the launch call
 //   shim_app --load SECONDS       device-filling kernels back to back on one stream
 //   shim_app --probe N PERIOD_US  a short kernel every PERIOD_US, launch-to-completion latency
 //   shim_app --leak               leaves main() with streams, events and memory never released
@@ -113,6 +114,33 @@ static int Bench(int launches)
     const double submit = std::chrono::duration<double, std::micro>(t1 - t0).count() / launches;
     const double total = std::chrono::duration<double, std::micro>(t2 - t0).count() / launches;
     printf("bench launches=%d submit_us_per_launch=%.3f total_us_per_launch=%.3f\n", launches, submit, total);
+    CHECK(hipStreamDestroy(s));
+    return 0;
+}
+
+// The same launches with `gap_us` of host work between them, the way a framework issues
+// kernels: what is timed is the launch call itself.
+static int BenchPaced(int launches, int gap_us)
+{
+    hipStream_t s;
+    CHECK(hipStreamCreate(&s));
+    for (int i = 0; i < 200; ++i) Bump<<<1, 64, 0, s>>>();
+    CHECK(hipStreamSynchronize(s));
+    std::vector<double> cost((size_t)launches);
+    using Clock = std::chrono::steady_clock;
+    for (int i = 0; i < launches; ++i) {
+        const auto t0 = Clock::now();
+        Bump<<<1, 64, 0, s>>>();
+        const auto t1 = Clock::now();
+        cost[(size_t)i] = std::chrono::duration<double, std::micro>(t1 - t0).count();
+        while (Clock::now() < t1 + std::chrono::microseconds(gap_us)) {}
+    }
+    CHECK(hipStreamSynchronize(s));
+    std::sort(cost.begin(), cost.end());
+    double sum = 0;
+    for (double c : cost) sum += c;
+    printf("bench-paced launches=%d gap_us=%d call_us_mean=%.3f p50=%.3f p99=%.3f\n", launches, gap_us, sum / launches,
+           cost[cost.size() / 2], cost[cost.size() * 99 / 100]);
     CHECK(hipStreamDestroy(s));
     return 0;
 }
@@ -259,6 +287,7 @@ int main(int argc, char **argv)
 {
     if (argc >= 2 && strcmp(argv[1], "--leak") == 0) return Leak();
     if (argc >= 3 && strcmp(argv[1], "--bench") == 0) return Bench(atoi(argv[2]));
+    if (argc >= 4 && strcmp(argv[1], "--bench-paced") == 0) return BenchPaced(atoi(argv[2]), atoi(argv[3]));
     if (argc >= 3 && strcmp(argv[1], "--load") == 0) return Load(atof(argv[2]));
     if (argc >= 3 && strcmp(argv[1], "--load-guarded") == 0) return LoadGuarded(atof(argv[2]), argc >= 4 ? (uint32_t)atoi(argv[3]) : 1u);
     if (argc >= 4 && strcmp(argv[1], "--probe") == 0) return Probe(atoi(argv[2]), atoi(argv[3]));

@@ -237,3 +237,37 @@ def test_a_command_launched_by_the_launcher_is_waited_for_by_the_launcher_at_onc
     print("waits (us):", [round(w * 1e6) for w in waits])
     assert min(waits) < 400e-6, "every wait took as long as the launcher's stand-by"
     xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hwq))
+
+
+def test_a_submitter_that_never_waits_hands_its_launches_to_the_launcher(xs):
+    """Direct launch is for submitters that wait for what they submit. After eight
+    submissions in a row with no wait in between, the rest of the stream goes through the
+    ring (the launcher makes the launches on another core while the submitter goes on);
+    a wait re-arms it. The computed values are the same either way."""
+    p, h = xs.preempt(), xs.halhost()
+    xs.check(p.XHintSetScheduler(xs.kSchedulerAppManaged, 0))
+    hwq = xs.host_queue_create()
+    xq = xs.xqueue_create(hwq)
+    xs.check(p.XQueueSetLaunchConfig(xq, 16, 8))
+    n, k = 2048, 40
+    ones = np.ones(n, np.float32); acc = np.zeros(n, np.float32)
+
+    def stream_of(count, gap):
+        for _ in range(count):
+            cmd = c_uint64()
+            xs.check(h.HostVecAddCommandCreate(byref(cmd), acc.ctypes.data, ones.ctypes.data, acc.ctypes.data, n, 0))
+            xs.check(p.XQueueSubmit(xq, cmd.value))
+            time.sleep(gap)     # long enough for the launcher to go back to sleep in between
+
+    wait_idle(xs, xq)
+    stream_of(k, 0.002)
+    streamed = direct_count(xs, xq)
+    xs.check(p.XQueueWaitAll(xq))
+    assert np.all(acc == k)
+    assert 1 <= streamed <= 8, f"{streamed} of {k} unwaited submissions were launched by the submitter"
+    wait_idle(xs, xq)
+    stream_of(3, 0.002)
+    assert direct_count(xs, xq) == streamed + 3, "a wait did not re-arm the direct launch"
+    xs.check(p.XQueueWaitAll(xq))
+    assert np.all(acc == k + 3)
+    xs.check(p.XQueueDestroy(xq)); xs.check(p.HwQueueDestroy(hwq))

@@ -143,6 +143,7 @@ public:
     /// Every command of this adapter except the host-side event wait only enqueues on
     /// the stream, so it may be launched on the submitting thread.
     virtual bool DirectLaunchable() override { return true; }
+    virtual bool CompletedWithoutWaiting() override;
 
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) = 0;

@@ -294,6 +294,15 @@ hipError_t HipCommand::LaunchWrapper(HipQueue &q, bool replay)
     return err;
 }
 
+bool HipCommand::CompletedWithoutWaiting()
+{
+    if (marker_ == nullptr) return false;
+    RelaxedCaptureScope relaxed;
+    const hipError_t err = hipEventQuery(marker_);
+    if (err != hipSuccess) (void)hipGetLastError();
+    return err == hipSuccess;
+}
+
 // Marker wait, sized for device work in the 10 us .. 1 ms range: poll the event
 // for a bounded time (no system call, no sleep/wake latency), then fall back to
 // the driver's blocking wait so that a long wait does not burn a core.

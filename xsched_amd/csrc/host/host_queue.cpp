@@ -51,6 +51,12 @@ public:
     // `override`: this file is also compiled against the plugin interface without the
     // direct-launch extension.)
     virtual bool DirectLaunchable() { return true; }
+    // (same: an extension of the plugin interface)
+    virtual bool CompletedWithoutWaiting()
+    {
+        std::lock_guard<std::mutex> lock(mtx_);
+        return marked_ && launches_ != 0 && retired_launches_ == launches_;
+    }
 
     bool Finished() const
     {

@@ -19,6 +19,7 @@ namespace
 {
 constexpr size_t kInitialRingSlots = 256;
 constexpr int64_t kSpinMicros = 150; // a waiter polls this long before it sleeps
+constexpr int64_t kDirectBurst = 8;           // submissions in a row without a wait that are still launched by the submitter
 constexpr int64_t kStandByMicros = 500;      // how long the launcher leaves the device to callers that launch themselves
 constexpr int64_t kStandBySliceMicros = 25;  // how often it looks whether their commands have retired
 constexpr unsigned long kLauncherTimerSlackNanos = 1000; // timed waits of the launcher end on time (the default slack is 50 us)
@@ -116,7 +117,13 @@ void RingXQueue::Submit(std::shared_ptr<HwCommand> hw_cmd)
         owed_ = Owed::kBatchThenDrain;
         // The launcher is parked and nothing waits in the ring: launching here keeps
         // submission order, and the ring lock keeps it so against other submitters.
-        const bool launched = caller_may_launch_ && parked_ && ring_count_ == 0 && TryLaunchOnCaller(hw_cmd);
+        // A submitter that waits for what it submits wants the launch at once, on its own
+        // thread. One that keeps submitting without waiting (a framework issuing kernel after
+        // kernel) is better off handing the launches to the launcher, which makes them on
+        // another core while the submitter goes on: after kDirectBurst submissions with no
+        // wait in between, the ring it is.
+        const bool streaming = ++unwaited_submits_ > kDirectBurst;
+        const bool launched = caller_may_launch_ && !streaming && parked_ && ring_count_ == 0 && TryLaunchOnCaller(hw_cmd);
         if (launched) caller_launched_ = true;
         else PushLocked(Slot::kCommand, wait_for_launch ? hw_cmd : std::move(hw_cmd));
         // A launcher that already stands by for callers (see NextStep) needs no wake-up for a
@@ -156,10 +163,16 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
             // Only for launches of callers: after a launch of its own the launcher is the one
             // who has to wait for the device, a submitter that waits for that command sleeps
             // on the completion number until the launcher has done so.
-            const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(kStandByMicros);
+            // The stand-by is counted from the callers' latest launch: while they keep
+            // launching, the queue is busy and theirs.
+            auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(kStandByMicros);
+            int64_t seen = handed_over_.load(std::memory_order_acquire);
             parked_ = true;
-            while (ring_count_ == 0 && retired_.load(std::memory_order_acquire) < handed_over_.load(std::memory_order_acquire) &&
-                   std::chrono::steady_clock::now() < until) {
+            while (ring_count_ == 0 && retired_.load(std::memory_order_acquire) < handed_over_.load(std::memory_order_acquire)) {
+                const auto now = std::chrono::steady_clock::now();
+                const int64_t newest = handed_over_.load(std::memory_order_acquire);
+                if (newest != seen) { seen = newest; until = now + std::chrono::microseconds(kStandByMicros); }
+                if (now >= until) break;
                 // (a wait on the system clock: the sanitizer build's runtime does not know the
                 // steady-clock wait of newer C libraries and would lose track of the lock)
                 ring_cv_.wait_until(g, std::chrono::system_clock::now() + std::chrono::microseconds(kStandBySliceMicros));
@@ -214,6 +227,7 @@ int64_t RingXQueue::RequestDrain(std::shared_ptr<XCommand> marker)
     int64_t ticket;
     {
         Guard g(ring_mu_);
+        unwaited_submits_ = 0;
         if (reported_ == kQueueStateIdle) return -1;
         ticket = next_idx_.load(std::memory_order_acquire) - 1;
         // With everything launched already and a caller that may wait for the device itself,
@@ -277,6 +291,7 @@ void RingXQueue::WaitAll()
 
 void RingXQueue::Wait(std::shared_ptr<HwCommand> hw_cmd)
 {
+    { Guard g(ring_mu_); unwaited_submits_ = 0; }
     if (!hw_cmd->Synchronizable()) {
         // No marker of its own: a later marker or a drain retires it.
         hw_cmd->WaitUntil(kCommandStateCompleted);
@@ -385,8 +400,18 @@ bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd)
 {
     if (!cmd->DirectLaunchable() || cmd->GetProps(kCommandPropertyCallback)) return false;
     Guard g(win_mu_);
-    if (run_ != Run::kRunning || win_count_ >= (size_t)threshold_) return false;
+    if (run_ != Run::kRunning) return false;
     std::shared_ptr<HwCommand> marker;
+    if (win_count_ >= (size_t)threshold_) {
+        // A full window is often full of finished commands: a submitter that never waits
+        // (a framework that launches kernel after kernel) has nobody who retires them while
+        // the launcher stands by. One look at the oldest marker, without waiting; the queue
+        // is running and the window lock is held, so a completed marker means what it says.
+        marker = OldestMarker();
+        if (marker == nullptr || !marker->CompletedWithoutWaiting()) return false;
+        RetireThrough(marker->GetIdx());
+        if (win_count_ >= (size_t)threshold_) return false;
+    }
     if (MustDrainFlushablesFirst(*cmd, &marker)) return false;
     cmd->BeforeLaunch(); // does not block for a command that calls itself DirectLaunchable
     HandOver(cmd);

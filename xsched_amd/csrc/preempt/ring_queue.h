@@ -92,6 +92,7 @@ private:
     Owed owed_ = Owed::kNothing;
     bool parked_ = false;
     bool caller_launched_ = false;      // a submitter has launched since the launcher last stood by
+    int64_t unwaited_submits_ = 0;      // submissions since anybody last asked for a drain
     XQueueState reported_ = kQueueStateIdle;
     uint64_t idle_round_ = 0;
 
