@@ -544,6 +544,44 @@ def shim_launch_cost():
     return out
 
 
+def framework_loop_under_shim(alternations=3):
+    """An unmodified PyTorch-ROCm training loop (tests/shim_torch_workload.py --time: about 26
+    kernel launches and fills per step, launch-bound), natively and with the interception shim
+    preloaded (every launch an XQueue command, level 1): microseconds per step. A process of
+    this loop lands in one of two speed classes some 30 % apart whatever is in front of the
+    runtime, so the two forms alternate and every run is reported. Informational; None when
+    the shim has not been built or a run fails."""
+    import re
+    import statistics
+    import subprocess
+    root = os.path.dirname(os.path.abspath(__file__))
+    shim = os.path.join(root, "xsched_amd", "lib", "libshimhip.so")
+    script = os.path.join(root, "tests", "shim_torch_workload.py")
+    if not os.path.exists(shim):
+        return None
+    base = {k: v for k, v in os.environ.items() if not k.startswith("XSCHED_")}
+    preload = " ".join(x for x in (os.environ.get("LD_PRELOAD", ""), shim) if x)
+    forms = (("native", {}),
+             ("under_shim_level1", {"LD_PRELOAD": preload, "XSCHED_AUTO_XQUEUE": "ON", "XSCHED_AUTO_XQUEUE_LEVEL": "1",
+                                    "XSCHED_SCHEDULER": "LCL", "XSCHED_POLICY": "HPF", "XLOG_LEVEL": "WARN"}))
+    runs = {key: [] for key, _ in forms}
+    for _ in range(alternations):
+        for key, extra in forms:
+            try:
+                proc = subprocess.run([sys.executable, script, "--time"], env=dict(base, **extra), capture_output=True,
+                                      text=True, timeout=120)
+            except subprocess.TimeoutExpired:
+                return None
+            m = re.search(r"us_per_step=([\d.]+)", proc.stdout)
+            if proc.returncode != 0 or not m:
+                return None
+            runs[key].append(float(m.group(1)))
+    native, under = statistics.median(runs["native"]), statistics.median(runs["under_shim_level1"])
+    return {"workload": "3-layer MLP, batch 1024, SGD with momentum, 200-step rounds on a side stream, median of 5 rounds per run",
+            "native_us_per_step": runs["native"], "under_shim_level1_us_per_step": runs["under_shim_level1"],
+            "median_native": native, "median_under_shim": under, "shim_over_native": round(under / native, 3)}
+
+
 def transparent_preemption():
     """Two plain HIP processes (tests/shim_app.hip), one filling the device with 5 ms kernels that
     have the guard compiled in (priority 0), one launching a short kernel every 2 ms (priority 1):
@@ -700,6 +738,7 @@ def main():
     if a.config == 2 and not a.quick:
         line["others"] = other_configurations(H, a)
         line["shim_launch_cost"] = shim_launch_cost()
+        line["framework_loop_under_shim"] = framework_loop_under_shim()
         line["transparent_preemption"] = transparent_preemption()
     if a.config == 2 and not a.skip_cpu:
         line["cpu_baseline"] = cpu_baseline(2)

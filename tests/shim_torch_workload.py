@@ -11,7 +11,43 @@ def digest(t):
     return hashlib.sha256(t.detach().float().cpu().numpy().tobytes()).hexdigest()[:16]
 
 
+def timed(steps=200, rounds=5):
+    """`--time`: the same network trained for `rounds` x `steps` steps on a side stream, the
+    median round in microseconds per step (bench.py runs it natively and under the shim)."""
+    import time
+    torch.manual_seed(0)
+    dev = torch.device("cuda")
+    work = torch.cuda.Stream()
+    with torch.cuda.stream(work):
+        model = torch.nn.Sequential(torch.nn.Linear(256, 512), torch.nn.ReLU(),
+                                    torch.nn.Linear(512, 512), torch.nn.Tanh(),
+                                    torch.nn.Linear(512, 10)).to(dev)
+        opt = torch.optim.SGD(model.parameters(), lr=0.05, momentum=0.9)
+        x = torch.randn(1024, 256, device=dev)
+        y = torch.randint(0, 10, (1024,), device=dev)
+
+        def train(n):
+            for _ in range(n):
+                opt.zero_grad()
+                loss = torch.nn.functional.cross_entropy(model(x), y)
+                loss.backward()
+                opt.step()
+            return loss
+
+        train(50)
+        work.synchronize()
+        per_step = []
+        for _ in range(rounds):
+            t0 = time.perf_counter()
+            loss = train(steps)
+            work.synchronize()
+            per_step.append((time.perf_counter() - t0) * 1e6 / steps)
+    print("timed steps=%d rounds=%d us_per_step=%.1f loss=%.6f" % (steps, rounds, sorted(per_step)[rounds // 2], loss.item()))
+
+
 def main():
+    if len(sys.argv) > 1 and sys.argv[1] == "--time":
+        return timed()
     torch.manual_seed(0)
     dev = torch.device("cuda")
     work, side = torch.cuda.Stream(), torch.cuda.Stream()

@@ -178,6 +178,18 @@ State &S()
 void PrintStats()
 {
     const Stats &t = S().stats;
+    // of the commands of the streams that still exist: how many their submitters launched themselves
+    int64_t submitted = 0, launched_by_submitter = 0;
+    {
+        std::shared_lock<std::shared_mutex> lock(S().stream_mtx);
+        for (auto &entry : S().stream_flags) {
+            auto xq = HwQueueManager::GetXQueue((HwQueueHandle)(uintptr_t)entry.first);
+            if (xq == nullptr) continue;
+            submitted += xq->GetHwCommandCount();
+            launched_by_submitter += xq->GetDirectLaunchCount();
+        }
+    }
+    fprintf(stderr, "[xsched shim] live queues: commands=%ld launched_by_submitter=%ld\n", (long)submitted, (long)launched_by_submitter);
     fprintf(stderr, "[xsched shim] kernel_cmds=%lu kernel_drained=%lu kernel_direct=%lu mem_cmds=%lu "
             "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu queue_launches=%lu "
             "deactivations=%lu reactivations=%lu guarded_cmds=%lu replays=%lu\n",
