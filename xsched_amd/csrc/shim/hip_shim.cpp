@@ -189,15 +189,16 @@ void PrintStats()
             launched_by_submitter += xq->GetDirectLaunchCount();
         }
     }
-    fprintf(stderr, "[xsched shim] live queues: commands=%ld launched_by_submitter=%ld\n", (long)submitted, (long)launched_by_submitter);
+
     fprintf(stderr, "[xsched shim] kernel_cmds=%lu kernel_drained=%lu kernel_direct=%lu mem_cmds=%lu "
             "mem_drained=%lu event_cmds=%lu event_waits=%lu known_kernels=%lu queue_launches=%lu "
-            "deactivations=%lu reactivations=%lu guarded_cmds=%lu replays=%lu\n",
+            "deactivations=%lu reactivations=%lu guarded_cmds=%lu replays=%lu live_queue_cmds=%ld "
+            "launched_by_submitter=%ld\n",
             (unsigned long)t.kernel_cmds, (unsigned long)t.kernel_drained, (unsigned long)t.kernel_direct,
             (unsigned long)t.mem_cmds, (unsigned long)t.mem_drained, (unsigned long)t.event_cmds,
             (unsigned long)t.event_waits, (unsigned long)t.known_kernels, (unsigned long)t.queue_launches,
             (unsigned long)t.deactivations, (unsigned long)t.reactivations, (unsigned long)t.guarded_cmds,
-            (unsigned long)t.replays);
+            (unsigned long)t.replays, (long)submitted, (long)launched_by_submitter);
 }
 
 constexpr unsigned kStreamCapturing = 1u << 31; // kept next to the stream's creation flags
