@@ -728,6 +728,10 @@ def main():
         print(json.dumps(line))
         return
 
+    # The package first: like the adapter library it asks the HIP runtime for a larger pool of
+    # completion signals (ROC_SIGNAL_POOL_SIZE, unless set), which the runtime reads when it
+    # starts, i.e. at the first HIP call of the process - torch's device check below.
+    import xsched_amd  # noqa: F401
     import torch  # device presence check only; the harness allocates through HIP itself
     if not torch.cuda.is_available():
         print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)
@@ -735,6 +739,8 @@ def main():
     from xsched_amd import harness as H
 
     line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
+    if isinstance(line.get("config"), dict):
+        line["config"]["runtime_env"] = {"ROC_SIGNAL_POOL_SIZE": os.environ.get("ROC_SIGNAL_POOL_SIZE")}
     if a.config == 2 and not a.quick:
         line["others"] = other_configurations(H, a)
         line["shim_launch_cost"] = shim_launch_cost()

@@ -13,6 +13,23 @@ from ctypes import (CFUNCTYPE, POINTER, byref, c_char_p, c_double, c_float, c_in
 
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 
+
+def _ask_for_larger_signal_pool():
+    """What libhalhip.so does when it is loaded, done here as well because a Python program has
+    usually imported torch (and with it the HIP runtime's library) before it loads the adapter:
+    the runtime reads ROC_SIGNAL_POOL_SIZE at the first HIP call of the process. A value the
+    user has set stays; XSCHED_HIP_SIGNAL_POOL=0 leaves the variable alone, any other number
+    is the size asked for (default 512)."""
+    try:
+        size = int(os.environ.get("XSCHED_HIP_SIGNAL_POOL", "512"))
+    except ValueError:
+        size = 512
+    if size > 0:
+        os.environ.setdefault("ROC_SIGNAL_POOL_SIZE", str(size))
+
+
+_ask_for_larger_signal_pool()
+
 # ---- enumerators (include/xsched/types.h) ------------------------------------
 kXSchedSuccess, kXSchedErrorHardware, kXSchedErrorInvalidValue = 0, 1, 2
 kXSchedErrorNotFound, kXSchedErrorNotAllowed, kXSchedErrorNotSupported = 3, 4, 5
