@@ -218,6 +218,7 @@ void RingXQueue::WaitForIdle()
 XQueueState RingXQueue::Query()
 {
     Guard g(ring_mu_);
+    unwaited_submits_ = 0;   // somebody follows this queue's progress: as good as a wait
     return reported_;
 }
 
