@@ -30,6 +30,11 @@ public:
     /// The id for an operation the caller is about to send to process `pid` itself (the
     /// daemon's configuration requests); 0 for a process that never announced itself.
     OperationId NextOperationId(PID pid);
+    /// Lets the thread that brings an event run the scheduling round itself when no other
+    /// round is under way, instead of waking the scheduler's own thread for it. For owners
+    /// whose event-bringing threads hold no lock that an operation could need (the daemon's
+    /// receiver); off by default, as in-process submitters send Ready under their queue's lock.
+    void RunRoundsOnCallers(bool on);
 
 private:
     class Rounds;

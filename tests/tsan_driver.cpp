@@ -9,7 +9,10 @@
 //      scheduler with the highest-priority-first policy (scheduler thread, two launcher
 //      threads, two executor threads, two submitters);
 //   4. launch-configuration and level changes between bursts, and destroying a queue that is
-//      suspended with work queued.
+//      suspended with work queued;
+//   5. a LocalScheduler of its own whose rounds run on the threads that bring the events (the
+//      daemon's arrangement): four threads report queues ready and idle, a fifth one switches
+//      the policy back and forth, the round thread keeps the laxity policy's alarms.
 // Every guarded work-group must have taken effect exactly once. The sanitizer's verdict is
 // its exit code and stderr; this program only checks the counts.
 #include <atomic>
@@ -22,6 +25,9 @@
 
 #include "xsched/hint.h"
 #include "xsched/xqueue.h"
+#include "xsched/sched/protocol/event.h"
+#include "xsched/sched/protocol/hint.h"
+#include "xsched/sched/scheduler/local.h"
 #include "xsched/host/bench.h"
 #include "xsched/host/hal.h"
 
@@ -140,6 +146,57 @@ int SchedulerWithTwoQueues()
     return ok ? 0 : 1;
 }
 
+int RoundsOnTheCallersThreads()
+{
+    using namespace xsched::sched;
+    LocalScheduler sched(kPolicyHighestPriorityFirst);
+    std::atomic<uint64_t> operations { 0 }, suspended_seen { 0 };
+    sched.SetExecutor([&](std::shared_ptr<const Operation> op) {
+        operations.fetch_add(1);
+        if (op->Type() == kOperationSched) {
+            auto *so = static_cast<const SchedOperation *>(op.get());
+            suspended_seen.fetch_add(so->SuspendedCnt());
+        }
+    });
+    sched.RunRoundsOnCallers(true);
+    sched.Run();
+    const PID pid = GetProcessId();
+    sched.RecvEvent(std::make_shared<ProcessCreateEvent>("tsan_driver"));
+    constexpr int kQueues = 4, kTurns = 600;
+    for (int q = 0; q < kQueues; ++q) {
+        const XQueueHandle h = 0x1000 + (XQueueHandle)q;
+        sched.RecvEvent(std::make_shared<XQueueCreateEvent>(h, (XDevice)1, kPreemptLevelBlock, 16, 8));
+        sched.RecvEvent(std::make_shared<HintEvent>(std::make_shared<PriorityHint>(h, (Priority)q)));
+        sched.RecvEvent(std::make_shared<HintEvent>(std::make_shared<LaxityHint>(h, (Laxity)200, (Priority)0, (Priority)(q + 1))));
+    }
+    std::vector<std::thread> reporters;
+    for (int q = 0; q < kQueues; ++q) {
+        reporters.emplace_back([&, q]() {
+            const XQueueHandle h = 0x1000 + (XQueueHandle)q;
+            for (int i = 0; i < kTurns; ++i) {
+                sched.RecvEvent(std::make_shared<XQueueReadyEvent>(h, std::chrono::system_clock::now()));
+                std::this_thread::sleep_for(std::chrono::microseconds(20 + 13 * q));
+                sched.RecvEvent(std::make_shared<XQueueIdleEvent>(h));
+            }
+        });
+    }
+    std::thread switcher([&]() {
+        for (int i = 0; i < 12; ++i) {
+            std::this_thread::sleep_for(std::chrono::milliseconds(3));
+            sched.SetPolicy(i % 2 ? kPolicyHighestPriorityFirst : kPolicyLaxity);
+        }
+    });
+    for (auto &t : reporters) t.join();
+    switcher.join();
+    for (int q = 0; q < kQueues; ++q) sched.RecvEvent(std::make_shared<XQueueDestroyEvent>(0x1000 + (XQueueHandle)q));
+    sched.Stop();
+    (void)pid;
+    const bool ok = operations.load() >= (uint64_t)kQueues * kTurns && suspended_seen.load() > 0;
+    printf("rounds on the callers' threads: %s (%llu operations)\n", ok ? "ok" : "TOO FEW OPERATIONS",
+           (unsigned long long)operations.load());
+    return ok ? 0 : 1;
+}
+
 } // namespace
 
 int main()
@@ -149,6 +206,7 @@ int main()
     bad += SparseSubmissionsUnderChurn();
     bad += TwoSubmittersOneWaiter();
     bad += SchedulerWithTwoQueues();
+    bad += RoundsOnTheCallersThreads();
     printf("%s\n", bad ? "FAILED" : "done");
     return bad ? 1 : 0;
 }

@@ -66,8 +66,8 @@ public:
 
     void SetAlarm(TimePoint at)
     {
-        std::lock_guard<std::mutex> g(mu_);
-        alarms_.push(at);
+        { std::lock_guard<std::mutex> g(mu_); alarms_.push(at); }
+        cv_.notify_one();   // the round thread may be asleep with no alarm to wake it
     }
 
     void ClearAlarms()
@@ -76,19 +76,20 @@ public:
         while (!alarms_.empty()) alarms_.pop();
     }
 
-    /// Blocks until there are events or an alarm is due; `batch` receives the events (none
-    /// when an alarm ended the wait). Every alarm that is due is struck off together.
-    void Take(std::vector<EventPtr> *batch)
+    /// Blocks until there are events or an alarm is due; removes nothing but the alarms that
+    /// are due (all of them together). True when an alarm ended the wait.
+    bool AwaitWork()
     {
-        batch->clear();
         // Poll for a while after the last batch before blocking (off unless XSCHED_SPIN_US is
         // set); alarms are looked at by the blocking path, which the poll leaves in time.
         const auto window = SpinWindow();
         if (window.count() > 0) {
-            const uint64_t seen = n_taken_;
-            auto give_up = last_batch_ + window;
+            uint64_t seen;
+            TimePoint give_up;
             {
                 std::lock_guard<std::mutex> g(mu_);
+                seen = n_taken_;
+                give_up = last_batch_ + window;
                 if (!alarms_.empty() && alarms_.top() < give_up) give_up = alarms_.top();
             }
             while (n_put_.load(std::memory_order_acquire) == seen && Clock::now() < give_up) __builtin_ia32_pause();
@@ -100,8 +101,16 @@ public:
             const TimePoint now = Clock::now();
             if (now < first) { cv_.wait_until(g, first); continue; }
             while (!alarms_.empty() && !(now < alarms_.top())) alarms_.pop();
-            return;
+            return true;
         }
+        return false;
+    }
+
+    /// `batch` receives the events that are waiting (possibly none); never blocks.
+    void TakeNow(std::vector<EventPtr> *batch)
+    {
+        batch->clear();
+        std::lock_guard<std::mutex> g(mu_);
         batch->swap(waiting_);
         n_taken_ = n_put_.load(std::memory_order_acquire); // under mu_: every Put() counted so far is in the batch
         last_batch_ = Clock::now();
@@ -112,8 +121,8 @@ private:
     std::condition_variable cv_;
     std::vector<EventPtr> waiting_;
     std::atomic<uint64_t> n_put_ { 0 };
-    uint64_t n_taken_ = 0;          // round thread only
-    TimePoint last_batch_ {};       // round thread only
+    uint64_t n_taken_ = 0;          // under mu_
+    TimePoint last_batch_ {};       // under mu_
     std::priority_queue<TimePoint, std::vector<TimePoint>, std::greater<TimePoint>> alarms_;
 };
 
@@ -280,6 +289,12 @@ public:
 
     /// Ledger entries change on the caller's thread: the round thread may be the one that
     /// waits for them. A completion is never queued (reference local.cpp:42-96).
+    ///
+    /// With rounds on the callers' threads switched on, the thread that brings an event runs
+    /// the round itself when nobody else is in one (what waits in the inbox goes first, so
+    /// events are folded in the order in which they came); otherwise the event is queued and
+    /// the round thread, which also keeps the alarms, takes it. That saves the wake-up of the
+    /// round thread, 10-50 us when it sleeps, between an event and the operations it causes.
     void Accept(EventPtr event)
     {
         switch (event->Type()) {
@@ -290,19 +305,33 @@ public:
             return;
         default: break;
         }
+        if (on_callers_.load(std::memory_order_acquire) && round_mu_.try_lock()) {
+            std::lock_guard<std::mutex> round(round_mu_, std::adopt_lock);
+            std::vector<EventPtr> batch;
+            inbox_.TakeNow(&batch);
+            batch.push_back(std::move(event));
+            // the terminate event is the round thread's to see: it goes back in
+            if (Round(batch)) inbox_.Put(std::make_shared<SchedulerTerminateEvent>());
+            return;
+        }
         inbox_.Put(std::move(event));
     }
+
+    void RoundsOnCallers(bool on) { on_callers_.store(on, std::memory_order_release); }
 
     void SwitchTo(XPolicyType type)
     {
         if (type == type_) return;
         const std::string before = GetPolicyTypeName(type_);
         Halt();
-        Install(type);
-        // the new policy starts from "everything runs"
-        std::vector<XQueueHandle> all;
-        for (auto &entry : mirror_.View().xqueue_status) all.push_back(entry.first);
-        for (XQueueHandle h : all) mirror_.Mark(h, false);
+        {
+            std::lock_guard<std::mutex> round(round_mu_); // callers may be running rounds
+            Install(type);
+            // the new policy starts from "everything runs"
+            std::vector<XQueueHandle> all;
+            for (auto &entry : mirror_.View().xqueue_status) all.push_back(entry.first);
+            for (XQueueHandle h : all) mirror_.Mark(h, false);
+        }
         Start();
         XINFO("policy changed from %s to %s", before.c_str(), GetPolicyTypeName(type).c_str());
     }
@@ -315,21 +344,31 @@ private:
     {
         std::vector<EventPtr> batch;
         while (true) {
-            inbox_.Take(&batch);
-            bool last_round = false;
-            for (auto &event : batch) {
-                if (UNLIKELY(event->Type() == kEventSchedulerTerminate)) last_round = true;
-                else Fold(*event);
-            }
-            policy_->Sched(mirror_.View());
-            // one operation per process that has XQueues, whether or not anything changed
-            for (auto &entry : mirror_.View().process_status) {
-                const ProcessStatus &ps = *entry.second;
-                if (ps.running_xqueues.empty() && ps.suspended_xqueues.empty()) continue;
-                owner_->Execute(std::make_shared<SchedOperation>(ledger_.Issue(ps.info.pid), ps));
-            }
-            if (last_round) return;
+            const bool alarm = inbox_.AwaitWork();
+            std::lock_guard<std::mutex> round(round_mu_);
+            inbox_.TakeNow(&batch);
+            if (batch.empty() && !alarm) continue;   // a caller's round has taken what woke this thread
+            if (Round(batch)) return;
         }
+    }
+
+    /// One round (round_mu_ held): fold the events, ask the policy, tell the processes. True
+    /// when the batch held the terminate event.
+    bool Round(const std::vector<EventPtr> &batch)
+    {
+        bool last_round = false;
+        for (auto &event : batch) {
+            if (UNLIKELY(event->Type() == kEventSchedulerTerminate)) last_round = true;
+            else Fold(*event);
+        }
+        policy_->Sched(mirror_.View());
+        // one operation per process that has XQueues, whether or not anything changed
+        for (auto &entry : mirror_.View().process_status) {
+            const ProcessStatus &ps = *entry.second;
+            if (ps.running_xqueues.empty() && ps.suspended_xqueues.empty()) continue;
+            owner_->Execute(std::make_shared<SchedOperation>(ledger_.Issue(ps.info.pid), ps));
+        }
+        return last_round;
     }
 
     // ---- folding one event into the mirror, one function per event type ----------------
@@ -415,6 +454,8 @@ private:
     std::unique_ptr<Policy> policy_;
     Inbox inbox_;
     Ledger ledger_;
+    std::mutex round_mu_;                    // the mirror, the policy, and who takes events out of the inbox
+    std::atomic<bool> on_callers_ { false };
     Mirror mirror_;
     std::thread thread_;
 };
@@ -430,5 +471,6 @@ void LocalScheduler::RecvEvent(std::shared_ptr<const Event> event) { rounds_->Ac
 void LocalScheduler::SetPolicy(XPolicyType type) { rounds_->SwitchTo(type); }
 XPolicyType LocalScheduler::GetPolicy() const { return rounds_->Type(); }
 OperationId LocalScheduler::NextOperationId(PID pid) { return rounds_->IssueId(pid); }
+void LocalScheduler::RunRoundsOnCallers(bool on) { rounds_->RoundsOnCallers(on); }
 
 } // namespace xsched::sched

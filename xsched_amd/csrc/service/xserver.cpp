@@ -58,6 +58,9 @@ public:
     {
         g_recv = std::make_unique<ipc::Node>((ipc::ChannelKey)XSCHED_SERVER_CHANNEL_KEY, ipc::NodeType::kReceiver);
         scheduler_->SetExecutor([this](std::shared_ptr<const Operation> op) { this->Execute(op); });
+        // Events come in on this process's own threads, which hold nothing an operation could
+        // need: they run the scheduling rounds themselves (one wake-up less per preemption).
+        scheduler_->RunRoundsOnCallers(GetEnvOption("XSCHED_SERVER_INLINE_ROUNDS", true));
         scheduler_->Run();
         std::thread reaper([this]() { this->ReapLoop(); });
         if (port_ > 0) {
