@@ -70,6 +70,14 @@ public:
     /// an idle core) out of the submit-to-device path.
     virtual bool SupportDirectLaunch() { return false; }
 
+    /// Extension: true when Deactivate() / Reactivate() concern nothing but launches that
+    /// are in flight (this repository's adapters: a deactivation changes a word that only
+    /// running kernels read). The XQueue then skips both for a queue that is suspended while
+    /// it has nothing in flight: a scheduler that suspends every queue below the one that
+    /// just became ready, busy or not, otherwise pays a device write per idle queue on every
+    /// command, and a round of replays of nothing on every resume.
+    virtual bool DeactivationConcernsInFlightWorkOnly() { return false; }
+
     std::shared_ptr<XQueue> GetXQueue() { return xq_; }
     void SetXQueue(std::shared_ptr<XQueue> xq) { xq_ = xq; }
 

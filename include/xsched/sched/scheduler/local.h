@@ -31,10 +31,13 @@ public:
     /// daemon's configuration requests); 0 for a process that never announced itself.
     OperationId NextOperationId(PID pid);
     /// Lets the thread that brings an event run the scheduling round itself when no other
-    /// round is under way, instead of waking the scheduler's own thread for it. For owners
-    /// whose event-bringing threads hold no lock that an operation could need (the daemon's
-    /// receiver); off by default, as in-process submitters send Ready under their queue's lock.
-    void RunRoundsOnCallers(bool on);
+    /// round is under way, instead of waking the scheduler's own thread for it: for every
+    /// event (owners whose event-bringing threads hold no lock that an operation could need:
+    /// the daemon's receiver), or for XQueueReady events only (in-process: the submitter
+    /// holds its queue's ring lock, which suspending and resuming OTHER queues does not need;
+    /// a resume can take tens of microseconds of launches and stays with the round thread).
+    enum { kRoundsOnCallersOff = 0, kRoundsOnCallersReady = 1, kRoundsOnCallersAll = 2 };
+    void RunRoundsOnCallers(int mode);
 
 private:
     class Rounds;

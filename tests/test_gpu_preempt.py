@@ -27,7 +27,9 @@ def churn(xs, q, stop, seed, flags=0):
     p = xs.preempt()
     cycles = 0
     while not stop.is_set():
-        time.sleep(rnd.uniform(0.0002, 0.002))
+        # the first suspension comes early: a queue is only deactivated on the device when it
+        # has work in flight, and the tests want to see that happen
+        time.sleep(rnd.uniform(0.0002, 0.002) if cycles else 0.0002)
         xs.check(p.XQueueSuspend(q.xq, flags))
         time.sleep(rnd.uniform(0.0001, 0.001))
         xs.check(p.XQueueResume(q.xq, 0))
@@ -112,7 +114,7 @@ def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile):
     monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
     M = N = K = 2048
     times = 12
-    print(f"case gemm-preempt {M}^3 times={times}", flush=True)
+    print(f"case gemm-preempt {M}^3 times={times} x 10", flush=True)
     a_bits = oracle.fill_normal_bf16(13, 1, 0, M * K)
     b_bits = oracle.fill_normal_bf16(13, 2, 0, K * N)
     a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
@@ -128,8 +130,9 @@ def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile):
     stop = threading.Event()
     t = threading.Thread(target=churn, args=(xs, q, stop, 3))
     t.start()
-    for c in outs:
-        q.submit(gemm_cmd(xs, a, b, c, M, N, K, 1))
+    for _ in range(10):      # ~2 ms of work in all: long enough for suspensions to land in it
+        for c in outs:
+            q.submit(gemm_cmd(xs, a, b, c, M, N, K, 1))
     time.sleep(0.02)
     stop.set()
     t.join()
@@ -262,8 +265,8 @@ def test_launches_of_a_flushed_epoch_do_not_run(xs, gpu, kind):
     work-group leaves the epoch of its launch there, and no work-group runs under an epoch
     it finds there. The race itself cannot be staged; the test writes the word the way a
     flushed work-group does and checks both halves of the rule: commands of that epoch
-    leave memory untouched, commands launched after a deactivation / reactivation (a new
-    epoch) run."""
+    leave memory untouched, a command replayed after a deactivation / reactivation (a new
+    epoch) runs."""
     torch = gpu
     print(f"case flushed-epoch {kind}", flush=True)
     q = Queue(xs, torch, level=2, threshold=4, batch=2)
@@ -310,9 +313,12 @@ def test_launches_of_a_flushed_epoch_do_not_run(xs, gpu, kind):
     q.submit(make())
     q.wait()
     untouched = read().copy()
+    # A third command of the flushed epoch, suspended while it is still in the queue's window
+    # (a queue with nothing in flight is not deactivated on the device at all): the
+    # deactivation opens a new epoch, and the reactivation replays the command under it.
+    q.submit(make())
     xs.check(p.XQueueSuspend(q.xq, 0))
     xs.check(p.XQueueResume(q.xq, 0))
-    q.submit(make())
     q.wait()
     ran = read().copy()
     q.close()

@@ -158,7 +158,7 @@ int RoundsOnTheCallersThreads()
             suspended_seen.fetch_add(so->SuspendedCnt());
         }
     });
-    sched.RunRoundsOnCallers(true);
+    sched.RunRoundsOnCallers(LocalScheduler::kRoundsOnCallersAll);
     sched.Run();
     const PID pid = GetProcessId();
     sched.RecvEvent(std::make_shared<ProcessCreateEvent>("tsan_driver"));

@@ -202,6 +202,7 @@ public:
     /// Launch() and Synchronize() only issue stream calls under the caller's lock; the
     /// calling thread's current device is switched for the call and put back.
     virtual bool SupportDirectLaunch() override { return true; }
+    virtual bool DeactivationConcernsInFlightWorkOnly() override { return true; }
 
     hipStream_t Stream() const { return stream_; }
     XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }

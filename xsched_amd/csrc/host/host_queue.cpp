@@ -131,6 +131,7 @@ public:
     virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
     virtual void OnPreemptLevelChange(XPreemptLevel level) override { level_ = level; }
     virtual bool SupportDirectLaunch() { return true; }
+    virtual bool DeactivationConcernsInFlightWorkOnly() { return true; }
 
     void GetStats(uint64_t *executed, uint64_t *skipped, uint64_t *replays) const
     {

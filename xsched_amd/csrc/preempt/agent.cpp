@@ -91,6 +91,16 @@ void SchedAgent::InitScheduler(XSchedulerType scheduler_type, XPolicyType policy
 {
     auto scheduler = CreateScheduler(scheduler_type, policy_type);
     scheduler->SetExecutor(SchedExecutor::Execute);
+    if (auto local = std::dynamic_pointer_cast<LocalScheduler>(scheduler)) {
+        // A queue that becomes ready is what preempts others: its submitter runs that round
+        // itself instead of waking the scheduler's thread (10-50 us when it sleeps). Only
+        // when a suspension waits for nothing: with one of the wait flags it would need the
+        // ring lock of the queue it suspends, which a submitter may be holding - its own.
+        const bool waits = GetEnvOption(XSCHED_SCHEDULER_SUSPEND_WAIT_ALL_ENV_NAME, false) ||
+                           GetEnvOption(XSCHED_SCHEDULER_SUSPEND_WAIT_IDLE_ENV_NAME, false) ||
+                           GetEnvOption(XSCHED_SCHEDULER_SUSPEND_SYNC_HWQ_ENV_NAME, false);
+        if (!waits && GetEnvOption("XSCHED_INLINE_READY_ROUNDS", true)) local->RunRoundsOnCallers(LocalScheduler::kRoundsOnCallersReady);
+    }
     scheduler->Run();
     static const std::string cmdline = ProcessCmdline();
     scheduler->RecvEvent(std::make_shared<ProcessCreateEvent>(cmdline));

@@ -46,6 +46,7 @@ RingXQueue::RingXQueue(std::shared_ptr<HwQueue> hwq, XPreemptLevel level, int64_
     XASSERT(threshold_ >= batch_, "threshold must not be smaller than command batch size");
     ResizeWindow(threshold_);
     caller_may_launch_ = hwq->SupportDirectLaunch() && GetEnvOption(XSCHED_DIRECT_LAUNCH_ENV_NAME, true);
+    lazy_deactivation_ = hwq->DeactivationConcernsInFlightWorkOnly();
 
     // The adapter binds its device to the launcher thread before anything else runs there;
     // the constructor returns once that has happened (async_xqueue.cpp:25-29).
@@ -559,12 +560,16 @@ void RingXQueue::Suspend(int64_t flags)
     if (flags & kQueueSuspendFlagWaitIdle) WaitForIdle();
     else if (flags & kQueueSuspendFlagWaitAll) WaitAll();
 
+    bool in_flight;
     {
         Guard g(win_mu_);
         run_ = Run::kPaused;
         pauses_++;
+        in_flight = win_count_ != 0;   // nothing joins the window while the queue is paused
     }
-    if (level_ >= kPreemptLevelDeactivate) kHwQueue->Deactivate();
+    // With nothing in flight there is nothing to flush (for adapters that say so).
+    deactivated_.store(level_ >= kPreemptLevelDeactivate && (in_flight || !lazy_deactivation_), std::memory_order_release);
+    if (deactivated_.load(std::memory_order_relaxed)) kHwQueue->Deactivate();
     if (level_ >= kPreemptLevelInterrupt) kHwQueue->Interrupt();
     if (flags & kQueueSuspendFlagSyncHwQueue) kHwQueue->Synchronize();
 }
@@ -583,7 +588,7 @@ void RingXQueue::Resume(int64_t flags)
         // the launcher is paused, so the window does not change under the adapter
         const CommandLog log = drop ? CommandLog {} : InFlightLog();
         if (level_ >= kPreemptLevelInterrupt) kHwQueue->Restore(log);
-        if (level_ >= kPreemptLevelDeactivate) kHwQueue->Reactivate(log);
+        if (level_ >= kPreemptLevelDeactivate && deactivated_.exchange(false, std::memory_order_acq_rel)) kHwQueue->Reactivate(log);
     }
     if (drop && level_ > kPreemptLevelBlock) {
         DiscardPending();

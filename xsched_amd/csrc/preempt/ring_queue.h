@@ -134,6 +134,9 @@ private:
     int64_t drop_through_ = -1;         // commands up to this index complete without launching
     bool queue_wait_active_ = false;    // some thread is waiting for the whole hardware queue
 
+    bool lazy_deactivation_ = false;           // the adapter's Deactivate() concerns in-flight launches only
+    std::atomic<bool> deactivated_ { false };  // the current suspension did call Deactivate()
+
     std::atomic<int64_t> next_idx_ { 1 };
     std::atomic<int64_t> handed_over_ { 0 };   // newest index launched or dropped
     std::atomic<int64_t> retired_ { 0 };       // newest index known complete

@@ -26,23 +26,35 @@ XResult XQueueManager::Add(XQueueHandle *xq_hp, HwQueueHandle hwq_h, int64_t lev
     // Only the asynchronous implementation exists.
     if (flags & kQueueCreateFlagBlockingSubmit) return kXSchedErrorNotSupported;
 
-    std::lock_guard<std::mutex> lock(g_xq_mtx);
     auto hwq = HwQueueManager::Get(hwq_h);
     if (hwq == nullptr) {
         XWARN("HwQueue with handle 0x" FMT_64X " does not exist or is not registered", hwq_h);
         return kXSchedErrorNotFound;
     }
 
-    if (auto existing = hwq->GetXQueue()) {
-        // One XQueue per hardware queue: hand out the one that is there.
+    // Creations take turns (two threads must not both build a queue for one hardware queue:
+    // the loser's constructor and destructor would tell the scheduler about a handle that the
+    // winner goes on using). A lock of its own, because the registry lock is not held while
+    // the queue is built, see below.
+    static std::mutex creation_mtx;
+    std::lock_guard<std::mutex> one_at_a_time(creation_mtx);
+
+    // One XQueue per hardware queue: hand out the one that is there.
+    auto hand_out_existing = [&](const std::shared_ptr<XQueue> &existing) {
         XASSERT(g_xqs.count(existing->GetHandle()), "XQueue 0x" FMT_64X " is not registered",
                 existing->GetHandle());
         XWARN("HwQueue 0x" FMT_64X " already has XQueue 0x" FMT_64X, hwq_h, existing->GetHandle());
         *xq_hp = existing->GetHandle();
         return kXSchedSuccess;
+    };
+    {
+        std::lock_guard<std::mutex> lock(g_xq_mtx);
+        if (auto existing = hwq->GetXQueue()) return hand_out_existing(existing);
     }
-
+    // Built outside the registry lock: the constructor starts a thread and tells the scheduler,
+    // and a scheduling round that runs on a submitter's thread looks queues up in this registry.
     auto xq = std::make_shared<RingXQueue>(hwq, (XPreemptLevel)level);
+    std::lock_guard<std::mutex> lock(g_xq_mtx);
     hwq->SetXQueue(xq); // cycle, broken in Del()
     g_xqs[xq->GetHandle()] = xq;
     *xq_hp = xq->GetHandle();

@@ -264,6 +264,8 @@ private:
 
 class LocalScheduler::Rounds
 {
+    static constexpr size_t kMaxQueuesForSubmitterRounds = 8;
+
 public:
     Rounds(LocalScheduler *owner, XPolicyType type): owner_(owner) { Install(type); }
 
@@ -305,8 +307,18 @@ public:
             return;
         default: break;
         }
-        if (on_callers_.load(std::memory_order_acquire) && round_mu_.try_lock()) {
-            std::lock_guard<std::mutex> round(round_mu_, std::adopt_lock);
+        const int mode = on_callers_.load(std::memory_order_acquire);
+        const bool here = mode == kRoundsOnCallersAll || (mode == kRoundsOnCallersReady && event->Type() == kEventXQueueReady);
+        if (here && round_mu_.try_lock()) {
+            std::unique_lock<std::mutex> round(round_mu_, std::adopt_lock);
+            // A round costs its caller a pass over every queue; for a submitter that is time
+            // before its own launch. With many queues the round thread's wake-up is the
+            // smaller price (measured with 16: +3 us at every queue's median).
+            if (mode == kRoundsOnCallersReady && mirror_.View().xqueue_status.size() > kMaxQueuesForSubmitterRounds) {
+                round.unlock();
+                inbox_.Put(std::move(event));
+                return;
+            }
             std::vector<EventPtr> batch;
             inbox_.TakeNow(&batch);
             batch.push_back(std::move(event));
@@ -317,7 +329,7 @@ public:
         inbox_.Put(std::move(event));
     }
 
-    void RoundsOnCallers(bool on) { on_callers_.store(on, std::memory_order_release); }
+    void RoundsOnCallers(int mode) { on_callers_.store(mode, std::memory_order_release); }
 
     void SwitchTo(XPolicyType type)
     {
@@ -455,7 +467,7 @@ private:
     Inbox inbox_;
     Ledger ledger_;
     std::mutex round_mu_;                    // the mirror, the policy, and who takes events out of the inbox
-    std::atomic<bool> on_callers_ { false };
+    std::atomic<int> on_callers_ { kRoundsOnCallersOff };
     Mirror mirror_;
     std::thread thread_;
 };
@@ -471,6 +483,6 @@ void LocalScheduler::RecvEvent(std::shared_ptr<const Event> event) { rounds_->Ac
 void LocalScheduler::SetPolicy(XPolicyType type) { rounds_->SwitchTo(type); }
 XPolicyType LocalScheduler::GetPolicy() const { return rounds_->Type(); }
 OperationId LocalScheduler::NextOperationId(PID pid) { return rounds_->IssueId(pid); }
-void LocalScheduler::RunRoundsOnCallers(bool on) { rounds_->RoundsOnCallers(on); }
+void LocalScheduler::RunRoundsOnCallers(int mode) { rounds_->RoundsOnCallers(mode); }
 
 } // namespace xsched::sched

@@ -60,7 +60,8 @@ public:
         scheduler_->SetExecutor([this](std::shared_ptr<const Operation> op) { this->Execute(op); });
         // Events come in on this process's own threads, which hold nothing an operation could
         // need: they run the scheduling rounds themselves (one wake-up less per preemption).
-        scheduler_->RunRoundsOnCallers(GetEnvOption("XSCHED_SERVER_INLINE_ROUNDS", true));
+        scheduler_->RunRoundsOnCallers(GetEnvOption("XSCHED_SERVER_INLINE_ROUNDS", true) ? LocalScheduler::kRoundsOnCallersAll
+                                                                                          : LocalScheduler::kRoundsOnCallersOff);
         scheduler_->Run();
         std::thread reaper([this]() { this->ReapLoop(); });
         if (port_ > 0) {
