@@ -76,8 +76,12 @@ public:
     Slot AcquireSlot();
     void ReleaseSlot(const Slot &slot);
     uint64_t SlotsInUse();
+    /// Allocates the first arena now (its device must be current), so that the first
+    /// guarded command does not wait for the allocation. Does nothing later on.
+    void ReserveSlots();
 
 private:
+    void AddArenaLocked();
     const int device_;
     bool flag_on_host_ = false;
     uint32_t copies_ = 1;            // power of two

@@ -242,25 +242,34 @@ void GuardState::WaitFlagWritten(hipStream_t op_stream)
     if (!flag_on_host_ && !write_through_bar_) HIP_ASSERT(hipStreamSynchronize(op_stream));
 }
 
+void GuardState::AddArenaLocked()
+{
+    RelaxedCaptureScope relaxed;
+    uint8_t *arena = nullptr;
+    const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
+    // Not cleared here: hipMemset() on device memory returns before the fill has run,
+    // and a kernel launched afterwards on a non-blocking stream overtakes it (its first
+    // progress bytes were then wiped, and a replay applied those work-groups again).
+    // Every slot is cleared in the order of its owner's stream instead, see Enqueue().
+    HIP_ASSERT(hipMalloc((void **)&arena, bytes));
+    arenas_.push_back(arena);
+    for (uint32_t i = 0; i < kSlotsPerArena; ++i) {
+        free_slots_.push_back((uint32_t)slot_ptr_.size());
+        slot_ptr_.push_back(arena + (size_t)i * kSlotBytes);
+        slot_gen_.push_back(0);
+    }
+}
+
+void GuardState::ReserveSlots()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    if (arenas_.empty()) AddArenaLocked();
+}
+
 GuardState::Slot GuardState::AcquireSlot()
 {
     std::lock_guard<std::mutex> lock(mtx_);
-    if (free_slots_.empty()) {
-        RelaxedCaptureScope relaxed;
-        uint8_t *arena = nullptr;
-        const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
-        // Not cleared here: hipMemset() on device memory returns before the fill has run,
-        // and a kernel launched afterwards on a non-blocking stream overtakes it (its first
-        // progress bytes were then wiped, and a replay applied those work-groups again).
-        // Every slot is cleared in the order of its owner's stream instead, see Enqueue().
-        HIP_ASSERT(hipMalloc((void **)&arena, bytes));
-        arenas_.push_back(arena);
-        for (uint32_t i = 0; i < kSlotsPerArena; ++i) {
-            free_slots_.push_back((uint32_t)slot_ptr_.size());
-            slot_ptr_.push_back(arena + (size_t)i * kSlotBytes);
-            slot_gen_.push_back(0);
-        }
-    }
+    if (free_slots_.empty()) AddArenaLocked();
     Slot slot;
     slot.index = free_slots_.back();
     free_slots_.pop_back();
@@ -410,12 +419,6 @@ HipQueue::~HipQueue()
 
 void HipQueue::OnXQueueCreate() { HIP_ASSERT(hipSetDevice(device_)); }
 
-void HipQueue::OnPreemptLevelChange(XPreemptLevel level)
-{
-    XASSERT(level <= kPreemptLevelDeactivate, "unsupported level: %d", level);
-    level_.store(level, std::memory_order_release);
-}
-
 namespace
 {
 
@@ -440,6 +443,19 @@ private:
 };
 
 } // namespace
+
+void HipQueue::OnPreemptLevelChange(XPreemptLevel level)
+{
+    XASSERT(level <= kPreemptLevelDeactivate, "unsupported level: %d", level);
+    if (level >= kPreemptLevelDeactivate) {
+        // the progress maps of the first guarded commands: allocated here, on the thread
+        // that configures the queue, and not in front of the first launch
+        DeviceScope scope(device_);
+        guard_->ReserveSlots();
+    }
+    level_.store(level, std::memory_order_release);
+}
+
 
 ScratchPool::~ScratchPool()
 {
