@@ -389,6 +389,10 @@ void RingXQueue::LaunchFromRing(std::shared_ptr<HwCommand> cmd)
         marker = OldestMarker();
         if (marker) AwaitMarker(g, marker);
         else AwaitQueue(g);
+        // Somebody else may have completed the marker while the queue is paused (a waiting
+        // caller retires what it waited for): the slot is free then, the launch still waits
+        // for the resume. (launch_worker.cpp:200-217 launches in that case.)
+        (void)HoldWhilePaused(g);
     } else {
         const bool running = HoldWhilePaused(g);
         XASSERT(running, "the launcher was asked to launch after it had been stopped");
