@@ -589,6 +589,7 @@ def transparent_preemption():
     scheduling, and with both processes under the interception shim, the scheduler daemon (HPF)
     and level 2. Informational; None when something it needs has not been built or a run fails."""
     import re
+    import shutil
     import subprocess
     import tempfile
     lib = os.path.join(os.path.dirname(os.path.abspath(__file__)), "xsched_amd", "lib")
@@ -614,6 +615,7 @@ def transparent_preemption():
         finally:
             if load.poll() is None:
                 load.kill()
+            load.wait()          # reaped: no zombie is left behind for the rest of the run
         if probe.returncode != 0 or load.returncode != 0:
             return None
         m = re.search(r"ms_per_kernel=([\d.]+) work_groups_not_exactly_once=(\d+)", load_out)
@@ -648,6 +650,8 @@ def transparent_preemption():
                     server.wait(timeout=5)
                 except subprocess.TimeoutExpired:
                     server.kill()
+                    server.wait()
+                shutil.rmtree(sock_dir, ignore_errors=True)
 
         under = under_daemon({})
         # The same with the three threads that relay a preemption (daemon receiver, its round

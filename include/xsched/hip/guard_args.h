@@ -23,7 +23,7 @@ struct XGuardArgs
 //   copy          its copy of the preempt word, read after the launch started
 //   flushed_word  the queue's `flushed` word, read after the launch started
 //   my_tag        its byte of the progress map (only looked at for replays)
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define XGUARD_FN __host__ __device__ static inline
 #else
 #define XGUARD_FN static inline

@@ -14,7 +14,6 @@ Produces, under xsched_amd/lib/:
                     with compressed device code                        (hipcc)
     xserver         scheduler daemon                                   (g++)
     traffic_probe   counter-run driver for the AXPY kernel             (hipcc)
-    launch_tail_probe  plain-HIP launch / record / wait loop: where the slow samples come from (hipcc)
 and, under oracle/, the checker libraries (see oracle/Makefile).
 
 Everything is compiled for gfx950 only; hipcc cross-compiles without a GPU.
@@ -128,9 +127,6 @@ def build_hip(extra, jobs):
     if os.path.exists(probe):
         _run(["hipcc"] + HIPFLAGS + extra + [probe, "-o", os.path.join(LIB, "traffic_probe"),
              "-L", LIB, "-Wl,-rpath,$ORIGIN", "-lhalhip", "-lpreempt", "-pthread"])
-    tail = os.path.join(CSRC, "bench", "launch_tail_probe.hip")
-    if os.path.exists(tail):
-        _run(["hipcc"] + HIPFLAGS + extra + [tail, "-o", os.path.join(LIB, "launch_tail_probe")])
 
 
 def build_oracle():
