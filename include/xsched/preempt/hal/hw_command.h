@@ -41,15 +41,6 @@ public:
     /// Process-unique handle.
     virtual HwCommandHandle GetHandle() { return (uint64_t)this ^ ((uint64_t)GetProcessId() << 48); }
 
-    /// Extension, see HwQueue::SupportDirectLaunch(): true when this command may be
-    /// launched on the submitting thread, i.e. its BeforeLaunch() never blocks.
-    virtual bool DirectLaunchable() { return false; }
-
-    /// Extension, same purpose: true when the device is known to have completed this
-    /// (synchronizable, launched) command; never blocks. A submitter that finds the window
-    /// full asks the oldest marker this way before it gives the launch to the launch thread.
-    virtual bool CompletedWithoutWaiting() { return false; }
-
     /// 1-based submission index inside its XQueue; -1 before submission.
     int64_t GetIdx() const { return idx_; }
     void SetIdx(int64_t idx) { idx_ = idx; }
@@ -63,6 +54,7 @@ public:
     void OnSubmit(std::shared_ptr<XQueue> xqueue);
 
 private:
+    friend class XCommand;   // a completed command lets go of its XQueue
     int64_t idx_ = -1;
     XQueueHandle xqueue_handle_ = 0;
     std::shared_ptr<XQueue> xqueue_ = nullptr;
@@ -73,7 +65,8 @@ class HwCallbackCommand final : public HwCommand
 {
 public:
     HwCallbackCommand(LaunchCallback launch, void *data)
-        : HwCommand(kCommandPropertyCallback), launch_(launch), data_(data) {}
+        : HwCommand(kCommandPropertyNone), launch_(launch), data_(data) {}
+    virtual ~HwCallbackCommand() = default;
 
     virtual void Synchronize()           override {}
     virtual bool Synchronizable()        override { return false; }

@@ -61,23 +61,6 @@ public:
     /// Called on the submitting thread for each command, before it is buffered.
     virtual void OnHwCommandSubmit(std::shared_ptr<HwCommand> hw_cmd) { UNUSED(hw_cmd); }
 
-    /// Extension (no counterpart in the reference; declared last so that adapters written
-    /// against the reference interface keep their virtual layout and get the default).
-    /// True: Launch() and Synchronize() may be called from ANY thread that holds the
-    /// XQueue's launch lock, not only from the launch thread. The XQueue then launches a
-    /// command on the submitting thread when the launch thread is asleep and nothing is
-    /// queued ahead of it, which takes the wake-up of that thread (tens of microseconds on
-    /// an idle core) out of the submit-to-device path.
-    virtual bool SupportDirectLaunch() { return false; }
-
-    /// Extension: true when Deactivate() / Reactivate() concern nothing but launches that
-    /// are in flight (this repository's adapters: a deactivation changes a word that only
-    /// running kernels read). The XQueue then skips both for a queue that is suspended while
-    /// it has nothing in flight: a scheduler that suspends every queue below the one that
-    /// just became ready, busy or not, otherwise pays a device write per idle queue on every
-    /// command, and a round of replays of nothing on every resume.
-    virtual bool DeactivationConcernsInFlightWorkOnly() { return false; }
-
     std::shared_ptr<XQueue> GetXQueue() { return xq_; }
     void SetXQueue(std::shared_ptr<XQueue> xq) { xq_ = xq; }
 

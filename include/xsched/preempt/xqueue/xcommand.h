@@ -2,9 +2,13 @@
 //
 // Type / property / state enumerators and the public methods match reference
 // preempt/include/xsched/preempt/xqueue/xcommand.h:15-139 so that hardware
-// adapters written against XSched compile unchanged. The state word is a
-// lock-free atomic here (waiters sleep on it directly); the mutex only guards
-// the small amount of pointer state subclasses keep.
+// adapters written against XSched compile unchanged, and the data members keep
+// that header's order, types and sizes so that an adapter BUILT against it runs
+// on this library as well (its inline constructor and accessors see the same
+// object). The state word is a lock-free atomic of the enumerator's size
+// (waiters sleep on it directly); the mutex only guards the small amount of
+// pointer state subclasses keep; the condition variable is not used by this
+// implementation and stays for the layout.
 #pragma once
 
 #include <atomic>
@@ -42,9 +46,6 @@ enum XCommandProperty
     kCommandPropertyIdempotent     = 0x0002,
     // Submit() returns only once the command has been launched.
     kCommandPropertyBlockingSubmit = 0x0004,
-    // Internal tag of HwCallbackCommand: the launch thread calls the user's
-    // function instead of HwQueue::Launch() without a run-time type lookup.
-    kCommandPropertyCallback       = 0x40000000,
     kCommandPropertyMaskAll        = -1,
 };
 
@@ -66,7 +67,7 @@ public:
 
     virtual void Wait() { this->WaitUntil(kCommandStateCompleted); }
 
-    XCommandState GetState() const { return (XCommandState)state_.load(std::memory_order_acquire); }
+    XCommandState GetState();
 
     /// States only move forward; listeners see every state passed through.
     void SetState(XCommandState state);
@@ -82,16 +83,13 @@ public:
     XCommandProperties GetProps(XCommandProperties mask = kCommandPropertyMaskAll) const
     { return props_ & mask; }
 
-protected:
-    /// Cheap completion hook for subclasses (no allocation, unlike a listener).
-    void (*on_completed_)(XCommand *) = nullptr;
-
 private:
     const XCommandType kCommandType;
     std::atomic<int32_t> state_ { kCommandStateCreated };
     XCommandProperties props_;
 
     std::mutex mtx_;
+    std::condition_variable state_cv_;
     std::list<std::function<void(XCommandState)>> state_listeners_;
 };
 

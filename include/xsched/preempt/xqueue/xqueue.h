@@ -34,7 +34,6 @@ public:
     virtual void Wait(std::shared_ptr<HwCommand> hw_cmd) = 0;
     virtual XQueueState Query() = 0;
     virtual int64_t GetHwCommandCount() = 0;
-    virtual int64_t GetDirectLaunchCount() { return 0; }
 
     virtual void Suspend(int64_t flags) = 0;
     virtual void Resume(int64_t flags) = 0;

@@ -66,5 +66,5 @@
 // Path of the daemon's Unix-domain socket directory.
 #define XSCHED_SOCKET_DIR_ENV_NAME       "XSCHED_SOCKET_DIR"
 /* ON (default) | OFF: launch on the submitting thread when the launch thread sleeps
- * (adapters that allow it, see HwQueue::SupportDirectLaunch) */
+ * (adapters that allow it, see HwQueueExtension::SupportDirectLaunch) */
 #define XSCHED_DIRECT_LAUNCH_ENV_NAME    "XSCHED_DIRECT_LAUNCH"

@@ -60,7 +60,7 @@ XResult XQueueResume(XQueueHandle xq, int64_t flags);
 XResult XQueueProfileHwCommandCount(XQueueHandle xq, int64_t *count);
 
 /* How many of them were launched on the submitting thread instead of the launch
- * thread (see HwQueue::SupportDirectLaunch). No counterpart in the reference. */
+ * thread (see HwQueueExtension::SupportDirectLaunch). No counterpart in the reference. */
 XResult XQueueProfileDirectLaunchCount(XQueueHandle xq, int64_t *count);
 
 /* Unregister a hardware queue; refused (NotAllowed) while an XQueue is attached.

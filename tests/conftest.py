@@ -18,6 +18,15 @@ def pytest_configure(config):
 def xs():
     import xsched_amd
     xsched_amd.preempt()
+    other = os.environ.get("XSCHED_TEST_HALHOST_LIB")
+    if other:
+        # tests/test_plugin_abi.py re-runs host-adapter tests with another build of the
+        # adapter (compiled against the reference's plugin headers) in the package's place.
+        import ctypes
+        lib = ctypes.CDLL(other)
+        xsched_amd._bind(lib, xsched_amd.HALHOST_API)
+        xsched_amd._halhost = lib
+        print("host adapter under test:", other)
     return xsched_amd
 
 

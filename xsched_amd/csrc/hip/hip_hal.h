@@ -18,6 +18,7 @@
 #include "xsched/hip/guard.h"
 #include "xsched/types.h"
 #include "xsched/utils/xassert.h"
+#include "xsched/preempt/hal/extensions.h"
 #include "xsched/preempt/hal/hw_command.h"
 #include "xsched/preempt/hal/hw_queue.h"
 
@@ -126,7 +127,7 @@ private:
 
 class HipQueue;
 
-class HipCommand : public preempt::HwCommand
+class HipCommand : public preempt::HwCommand, public preempt::HwCommandExtension
 {
 public:
     explicit HipCommand(preempt::XCommandProperties props = preempt::kCommandPropertyNone)
@@ -186,7 +187,7 @@ private:
     GuardState::Slot slot_;
 };
 
-class HipQueue : public preempt::HwQueue
+class HipQueue : public preempt::HwQueue, public preempt::HwQueueExtension
 {
 public:
     explicit HipQueue(hipStream_t stream);

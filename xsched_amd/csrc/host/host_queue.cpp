@@ -11,6 +11,7 @@
 #include "xsched/xqueue.h"
 #include "xsched/utils/xassert.h"
 #include "xsched/protocol/device.h"
+#include "xsched/preempt/hal/extensions.h"
 #include "xsched/preempt/hal/hw_command.h"
 #include "xsched/preempt/hal/hw_queue.h"
 
@@ -30,7 +31,7 @@ struct Ticket
     uint64_t seq;     // position in this queue's launch order
 };
 
-class HostKernelCommand : public HwCommand
+class HostKernelCommand : public HwCommand, public HwCommandExtension
 {
 public:
     HostKernelCommand(HostKernelFn fn, void *arg, uint32_t n_wg, bool guarded)
@@ -47,12 +48,9 @@ public:
     }
     virtual bool Synchronizable() override { return marked_; }
     virtual bool EnableSynchronization() override { marked_ = true; return true; }
-    // Launching is handing a ticket to the executor thread: any thread may do it. (No
-    // `override`: this file is also compiled against the plugin interface without the
-    // direct-launch extension.)
-    virtual bool DirectLaunchable() { return true; }
-    // (same: an extension of the plugin interface)
-    virtual bool CompletedWithoutWaiting()
+    // Launching is handing a ticket to the executor thread: any thread may do it.
+    virtual bool DirectLaunchable() override { return true; }
+    virtual bool CompletedWithoutWaiting() override
     {
         std::lock_guard<std::mutex> lock(mtx_);
         return marked_ && launches_ != 0 && retired_launches_ == launches_;
@@ -78,7 +76,7 @@ private:
     uint64_t retired_launches_ = 0;
 };
 
-class HostQueue : public HwQueue
+class HostQueue : public HwQueue, public HwQueueExtension
 {
 public:
     HostQueue(): handle_(NextHandle())
@@ -130,8 +128,8 @@ public:
     virtual bool SupportDynamicLevel() override { return true; }
     virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
     virtual void OnPreemptLevelChange(XPreemptLevel level) override { level_ = level; }
-    virtual bool SupportDirectLaunch() { return true; }
-    virtual bool DeactivationConcernsInFlightWorkOnly() { return true; }
+    virtual bool SupportDirectLaunch() override { return true; }
+    virtual bool DeactivationConcernsInFlightWorkOnly() override { return true; }
 
     void GetStats(uint64_t *executed, uint64_t *skipped, uint64_t *replays) const
     {

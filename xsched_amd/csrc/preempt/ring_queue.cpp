@@ -2,6 +2,7 @@
 // preempt/src/xqueue/{async_xqueue,command_buffer,launch_worker}.cpp (citations below name
 // the rule each block keeps).
 #include <chrono>
+#include <typeinfo>
 
 #include <sys/prctl.h>
 
@@ -45,8 +46,10 @@ RingXQueue::RingXQueue(std::shared_ptr<HwQueue> hwq, XPreemptLevel level, int64_
     // single marker in it to wait for.
     XASSERT(threshold_ >= batch_, "threshold must not be smaller than command batch size");
     ResizeWindow(threshold_);
-    caller_may_launch_ = hwq->SupportDirectLaunch() && GetEnvOption(XSCHED_DIRECT_LAUNCH_ENV_NAME, true);
-    lazy_deactivation_ = hwq->DeactivationConcernsInFlightWorkOnly();
+    // What the adapter offers beyond the reference's contract, if anything.
+    auto *ext = dynamic_cast<HwQueueExtension *>(hwq.get());
+    caller_may_launch_ = ext != nullptr && ext->SupportDirectLaunch() && GetEnvOption(XSCHED_DIRECT_LAUNCH_ENV_NAME, true);
+    lazy_deactivation_ = ext != nullptr && ext->DeactivationConcernsInFlightWorkOnly();
 
     // The adapter binds its device to the launcher thread before anything else runs there;
     // the constructor returns once that has happened (async_xqueue.cpp:25-29).
@@ -404,7 +407,8 @@ void RingXQueue::LaunchFromRing(std::shared_ptr<HwCommand> cmd)
 // The caller holds the ring lock and has seen the launcher parked on an empty ring.
 bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd)
 {
-    if (!cmd->DirectLaunchable() || cmd->GetProps(kCommandPropertyCallback)) return false;
+    auto *ext = dynamic_cast<HwCommandExtension *>(cmd.get());   // null for callback commands too
+    if (ext == nullptr || !ext->DirectLaunchable()) return false;
     Guard g(win_mu_);
     if (run_ != Run::kRunning) return false;
     std::shared_ptr<HwCommand> marker;
@@ -414,7 +418,8 @@ bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd)
         // the launcher stands by. One look at the oldest marker, without waiting; the queue
         // is running and the window lock is held, so a completed marker means what it says.
         marker = OldestMarker();
-        if (marker == nullptr || !marker->CompletedWithoutWaiting()) return false;
+        auto *marker_ext = dynamic_cast<HwCommandExtension *>(marker.get());
+        if (marker_ext == nullptr || !marker_ext->CompletedWithoutWaiting()) return false;
         RetireThrough(marker->GetIdx());
         if (win_count_ >= (size_t)threshold_) return false;
     }
@@ -437,7 +442,8 @@ void RingXQueue::HandOver(const std::shared_ptr<HwCommand> &cmd)
     }
     if (idx - last_marked_idx_ >= batch_) cmd->EnableSynchronization();
 
-    if (cmd->GetProps(kCommandPropertyCallback)) {
+    // (the class is final: comparing the dynamic type is exact and costs no hierarchy walk)
+    if (typeid(*cmd) == typeid(HwCallbackCommand)) {
         auto *cb = static_cast<HwCallbackCommand *>(cmd.get());
         XASSERT(cb->Launch(kHwQueue->GetHandle()) == kXSchedSuccess, "failed to launch HwCallbackCommand (%p)", (void *)cb);
     } else {

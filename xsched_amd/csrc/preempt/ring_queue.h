@@ -16,7 +16,7 @@
 // Completion is tracked by ONE monotonic number, the index of the newest command known
 // complete (`retired_`). XQueueWaitAll takes the index of the last submission as its ticket
 // and waits for that number to reach it; no marker object is built for it. With an adapter
-// that lets any thread launch and synchronise (HwQueue::SupportDirectLaunch) the submitter
+// that lets any thread launch and synchronise (HwQueueExtension::SupportDirectLaunch) the submitter
 // launches a command itself when the launcher is parked on an empty ring, and a waiter whose
 // commands have all been launched waits for the device itself; the launcher is only woken,
 // off the caller's path, to run the drain sequence that ends in the Idle event.
@@ -35,6 +35,7 @@
 #include <vector>
 
 #include "xsched/protocol/def.h"
+#include "xsched/preempt/hal/extensions.h"
 #include "xsched/preempt/xqueue/xqueue.h"
 
 namespace xsched::preempt
@@ -54,7 +55,8 @@ public:
     void Wait(std::shared_ptr<HwCommand> hw_cmd) override;
     XQueueState Query() override;
     int64_t GetHwCommandCount() override { return next_idx_.load(std::memory_order_acquire) - 1; }
-    int64_t GetDirectLaunchCount() override { return direct_launches_.load(std::memory_order_relaxed); }
+    /// Commands launched on a submitting thread so far (not part of the XQueue interface).
+    int64_t GetDirectLaunchCount() const { return direct_launches_.load(std::memory_order_relaxed); }
 
     void Suspend(int64_t flags) override;
     void Resume(int64_t flags) override;

@@ -16,6 +16,11 @@ namespace xsched::preempt
 
 static constexpr int64_t kWaitSpinMicros = 150;
 
+XCommandState XCommand::GetState()
+{
+    return (XCommandState)state_.load(std::memory_order_acquire);
+}
+
 void XCommand::SetState(XCommandState new_state)
 {
     XASSERT(new_state >= kCommandStateCreated && new_state <= kCommandStateCompleted,
@@ -29,7 +34,14 @@ void XCommand::SetState(XCommandState new_state)
     for (int s = old_state + 1; s <= new_state; ++s) {
         for (auto &listener : state_listeners_) listener(XCommandState(s));
     }
-    if (new_state == kCommandStateCompleted && on_completed_ != nullptr) on_completed_(this);
+    if (new_state == kCommandStateCompleted && kCommandType == kCommandTypeHardware) {
+        // A completed command lets go of its XQueue so the queue can be destroyed while
+        // the application still holds the command (hw_command.cpp:9-16 does this with a
+        // state listener, i.e. two allocations per command).
+        auto *cmd = static_cast<HwCommand *>(this);
+        std::lock_guard<std::mutex> lock(mtx_);
+        cmd->xqueue_ = nullptr;
+    }
 }
 
 // Short waits (a command of a few microseconds) are polled: sleeping on the state
@@ -53,16 +65,7 @@ void XCommand::WaitUntil(XCommandState state)
 
 // ---- HwCommand -------------------------------------------------------------
 
-HwCommand::HwCommand(XCommandProperties props): XCommand(kCommandTypeHardware, props)
-{
-    // A completed command lets go of its XQueue so the queue can be destroyed
-    // while the application still holds the command (hw_command.cpp:9-16).
-    on_completed_ = [](XCommand *self) {
-        auto *cmd = static_cast<HwCommand *>(self);
-        auto lock = cmd->GetLock();
-        cmd->xqueue_ = nullptr;
-    };
-}
+HwCommand::HwCommand(XCommandProperties props): XCommand(kCommandTypeHardware, props) {}
 
 void HwCommand::Wait()
 {

@@ -316,6 +316,7 @@ EXPORT_C_FUNC XResult XQueueProfileDirectLaunchCount(XQueueHandle xq, int64_t *c
 {
     if (count == nullptr) return kXSchedErrorInvalidValue;
     FIND_XQUEUE_OR_RETURN(q, xq);
-    *count = q->GetDirectLaunchCount();
+    auto *ring = dynamic_cast<RingXQueue *>(q.get());
+    *count = ring != nullptr ? ring->GetDirectLaunchCount() : 0;
     return kXSchedSuccess;
 }

@@ -43,6 +43,7 @@
 #include "../hip/shim_hooks.h"
 #include "xsched/hip/hal.h"
 #include "xsched/hip/shim.h"
+#include "xsched/xqueue.h"
 #include "xsched/utils/log.h"
 #include "xsched/preempt/hal/hw_command.h"
 #include "xsched/preempt/hal/hw_queue.h"
@@ -186,7 +187,8 @@ void PrintStats()
             auto xq = HwQueueManager::GetXQueue((HwQueueHandle)(uintptr_t)entry.first);
             if (xq == nullptr) continue;
             submitted += xq->GetHwCommandCount();
-            launched_by_submitter += xq->GetDirectLaunchCount();
+            int64_t direct = 0;
+            if (XQueueProfileDirectLaunchCount(xq->GetHandle(), &direct) == kXSchedSuccess) launched_by_submitter += direct;
         }
     }
 
