@@ -65,6 +65,7 @@ public:
     {
         { std::lock_guard<std::mutex> lock(mtx); Add("D"); flushes++; }
         cv.notify_all();
+        if (on_deactivate) on_deactivate(on_deactivate_arg);   // on whichever thread runs the scheduling operation
     }
 
     virtual void Reactivate(const CommandLog &log) override
@@ -94,6 +95,8 @@ public:
     int64_t last_launched = 0;
     uint64_t flushes = 0;
     bool gate_open = false;
+    void (*on_deactivate)(void *) = nullptr;
+    void *on_deactivate_arg = nullptr;
 
 private:
     const uint64_t handle_;
@@ -158,6 +161,18 @@ EXPORT_C_FUNC XResult RecQueueSetGate(HwQueueHandle hwq, int open)
     if (!q) return kXSchedErrorNotFound;
     { std::lock_guard<std::mutex> lock(q->mtx); q->gate_open = open != 0; }
     q->cv.notify_all();
+    return kXSchedSuccess;
+}
+
+/// `fn(arg)` is called at the end of every Deactivate() of this queue, on the thread that
+/// executes the suspension (a test looks from there at what that thread holds).
+EXPORT_C_FUNC XResult RecQueueOnDeactivate(HwQueueHandle hwq, void (*fn)(void *), void *arg)
+{
+    auto q = Find(hwq);
+    if (!q) return kXSchedErrorNotFound;
+    std::lock_guard<std::mutex> lock(q->mtx);
+    q->on_deactivate = fn;
+    q->on_deactivate_arg = arg;
     return kXSchedSuccess;
 }
 

@@ -253,10 +253,16 @@ static int Probe(int count, int period_us)
         us[i] = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
         std::this_thread::sleep_for(std::chrono::microseconds(period_us));
     }
+    if (const char *dump = getenv("SHIM_APP_PROBE_DUMP")) {   // every sample in arrival order, for a closer look at the tail
+        if (FILE *f = fopen(dump, "w")) {
+            for (double v : us) fprintf(f, "%.1f\n", v);
+            fclose(f);
+        }
+    }
     std::sort(us.begin(), us.end());
     // percentile p = sorted[floor(p * n)]
-    printf("probe n=%d p50_us=%.1f p99_us=%.1f max_us=%.1f\n", count, us[(size_t)(0.5 * count)],
-           us[(size_t)(0.99 * count)], us.back());
+    printf("probe n=%d p50_us=%.1f p99_us=%.1f max_us=%.1f p90_us=%.1f p95_us=%.1f\n", count, us[(size_t)(0.5 * count)],
+           us[(size_t)(0.99 * count)], us.back(), us[(size_t)(0.9 * count)], us[(size_t)(0.95 * count)]);
     CHECK(hipFree(out));
     CHECK(hipStreamDestroy(s));
     return 0;

@@ -60,7 +60,7 @@ class HipEventRecordCommand final : public HipCommand
 {
 public:
     explicit HipEventRecordCommand(hipEvent_t event): HipCommand(kCommandPropertyIdempotent), event_(event) {}
-    virtual void Synchronize() override { HIP_ASSERT(hipEventSynchronize(event_)); }
+    virtual void Synchronize() override { WaitForEvent(event_); }
     virtual bool Synchronizable() override { return true; }
     virtual bool EnableSynchronization() override { return true; }
 protected:

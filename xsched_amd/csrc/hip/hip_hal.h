@@ -145,6 +145,7 @@ public:
     /// Whether Reactivate() must enqueue this command again.
     virtual bool ReplayOnReactivate() const { return false; }
 
+
     /// Every command of this adapter except the host-side event wait only enqueues on
     /// the stream, so it may be launched on the submitting thread.
     virtual bool DirectLaunchable() override { return true; }
@@ -152,6 +153,8 @@ public:
 
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) = 0;
+    /// Polls the event for the marker polling budget (no system call), then blocks in the driver.
+    void WaitForEvent(hipEvent_t event);
     hipEvent_t marker_ = nullptr;
 
 private:
@@ -226,6 +229,12 @@ private:
     std::shared_ptr<GuardState> guard_;
     hipStream_t op_stream_ = nullptr; // flag writes when the word lives in device memory
     std::shared_ptr<ScratchPool> scratch_;
+
+    // The newest command handed to the stream, while it carries a marker that was recorded
+    // right behind it: Synchronize() then waits for that marker instead of putting another
+    // one on the stream.
+    std::mutex tail_mtx_;
+    std::shared_ptr<preempt::HwCommand> tail_marked_;
 };
 
 /// Microseconds a marker wait polls before it blocks in the driver.

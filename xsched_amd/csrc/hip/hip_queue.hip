@@ -336,13 +336,18 @@ bool HipCommand::CompletedWithoutWaiting()
 void HipCommand::Synchronize()
 {
     XASSERT(marker_ != nullptr, "Synchronize() needs EnableSynchronization() before launch");
+    WaitForEvent(marker_);
+}
+
+void HipCommand::WaitForEvent(hipEvent_t event)
+{
     RelaxedCaptureScope relaxed;
-    if (PollEvent(marker_, SyncSpinMicros())) {
+    if (PollEvent(event, SyncSpinMicros())) {
         if (queue_) queue_->n_wait_polled.fetch_add(1, std::memory_order_relaxed);
         return;
     }
     if (queue_) queue_->n_wait_blocked.fetch_add(1, std::memory_order_relaxed);
-    HIP_ASSERT(hipEventSynchronize(marker_));
+    HIP_ASSERT(hipEventSynchronize(event));
 }
 
 // ---- HipGuardedCommand -------------------------------------------------------
@@ -508,16 +513,39 @@ void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)
     hipError_t err = cmd->LaunchWrapper(*this, false);
     XASSERT(err == hipSuccess, "failed to enqueue command: %d (%s)", (int)err, hipGetErrorString(err));
     n_launch.fetch_add(1, std::memory_order_relaxed);
+    {
+        std::lock_guard<std::mutex> lock(tail_mtx_);
+        if (cmd->Synchronizable()) tail_marked_ = std::move(hw_cmd);
+        else tail_marked_ = nullptr;
+    }
 }
 
-// A marker recorded behind whatever the stream holds, then polled like any marker. Asking
-// the runtime about the stream itself (hipStreamQuery / hipStreamSynchronize) is several
-// times slower when the newest operation on it is a kernel: the runtime then has to put a
-// marker of its own behind the kernel first and hears of its completion through its signal
-// thread. Recorded here, the marker is on its way while the kernel still runs.
+// Waits for the marker of the newest command when that command carries one (recorded at
+// launch, so it is on its way through the device's queue together with the command: a wait
+// that begins later finds it done or nearly so). Otherwise a marker is recorded now, behind
+// whatever the stream holds, and polled like any marker: every marker is one more packet
+// the device's command processor works through in order, a few microseconds each, which a
+// command that a submitter waits for at once should not pay twice. Asking the runtime about
+// the stream itself (hipStreamQuery / hipStreamSynchronize) is several times slower when the
+// newest operation on it is a kernel: the runtime then has to put a marker of its own behind
+// the kernel first and hears of its completion through its signal thread.
 void HipQueue::Synchronize()
 {
     DeviceScope scope(device_);
+    std::shared_ptr<HwCommand> tail;
+    {
+        std::lock_guard<std::mutex> lock(tail_mtx_);
+        tail = tail_marked_;
+    }
+    if (tail != nullptr) {
+        // (a replay re-records this marker behind the replayed work: still the stream's end;
+        // an event-record command is waited for through the application's event, as its
+        // XQueue waits for it as a batch marker: hip_command.h:197-219)
+        tail->Synchronize();
+        std::lock_guard<std::mutex> lock(tail_mtx_);
+        if (tail_marked_ == tail) tail_marked_ = nullptr;   // done: nothing of the stream is left to wait for, and the command is let go
+        return;
+    }
     RelaxedCaptureScope relaxed;
     hipEvent_t marker = EventPool::Instance().Pop();
     hipError_t err = hipEventRecord(marker, stream_);
@@ -529,6 +557,7 @@ void HipQueue::Synchronize()
 void HipQueue::Deactivate()
 {
     XASSERT(Level() >= kPreemptLevelDeactivate, "Deactivate() not supported on level-%d", Level());
+    DeviceScope scope(device_);   // the copy variant of the flag write enqueues on this device's side stream
     guard_->Deactivate(op_stream_);
     n_deactivate.fetch_add(1, std::memory_order_relaxed);
 }
@@ -542,7 +571,9 @@ void HipQueue::Deactivate()
 void HipQueue::Reactivate(const CommandLog &log)
 {
     XASSERT(Level() >= kPreemptLevelDeactivate, "Reactivate() not supported on level-%d", Level());
-    HIP_ASSERT(hipSetDevice(device_));
+    // Whoever executes the scheduling operation calls this, possibly an application thread
+    // in the middle of its own submission: its current device is put back afterwards.
+    DeviceScope scope(device_);
     n_reactivate.fetch_add(1, std::memory_order_relaxed);
     // A replay carries the new epoch; the word must already show it, or the replay
     // would flush itself.

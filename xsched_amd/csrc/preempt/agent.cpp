@@ -107,6 +107,7 @@ void SchedAgent::InitScheduler(XSchedulerType scheduler_type, XPolicyType policy
 
     std::unique_lock<std::shared_mutex> lock(mtx_);
     scheduler_ = scheduler;
+    ready_event_first_.store(scheduler->GetType() == kSchedulerGlobal, std::memory_order_relaxed);
 }
 
 void SchedAgent::FiniScheduler()

@@ -4,6 +4,7 @@
 // XHintSetScheduler(). Follows reference preempt/src/sched/agent.cpp:21-140.
 #pragma once
 
+#include <atomic>
 #include <memory>
 #include <shared_mutex>
 
@@ -26,6 +27,15 @@ public:
     static XResult SetScheduler(XSchedulerType scheduler, XPolicyType policy)
     { return Instance().ReplaceScheduler(scheduler, policy); }
 
+    /// Whether a queue that becomes ready should tell the scheduler BEFORE it launches the
+    /// command that made it so. True for the daemon client: its decision comes back through
+    /// two other processes, the longest leg of a preemption, so it starts first and the
+    /// event costs the submitter one datagram. False in-process: the event may run a whole
+    /// scheduling round on the submitter's thread (suspensions, deactivations, replays on
+    /// other queues); the command goes to the device first and the round overlaps with its
+    /// way there, with none of the submitter's queue locks held.
+    static bool ReadyEventGoesFirst() { return Instance().ready_event_first_.load(std::memory_order_relaxed); }
+
 private:
     static SchedAgent &Instance();
     void RelayHint(std::shared_ptr<const sched::Hint> hint);
@@ -37,6 +47,7 @@ private:
     // Relays hold it shared; replacing the scheduler holds it exclusively.
     std::shared_mutex mtx_;
     std::shared_ptr<sched::Scheduler> scheduler_;
+    std::atomic<bool> ready_event_first_ { false };
 };
 
 /// Applies scheduler operations to the XQueues of this process: resume the

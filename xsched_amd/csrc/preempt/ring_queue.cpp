@@ -108,14 +108,28 @@ void RingXQueue::Submit(std::shared_ptr<HwCommand> hw_cmd)
     const bool wait_for_launch = hw_cmd->GetProps(kCommandPropertyBlockingSubmit) != 0;
     hw_cmd->SetState(kCommandStatePending);
 
-    bool wake;
+    // The Ready event either goes out first, under the ring lock (daemon client: one
+    // datagram), or after the launch and with no lock of this queue held (in-process: it may
+    // run a scheduling round on this thread, which suspends, deactivates and replays other
+    // queues; meanwhile this queue's launcher, its other submitters and waiters go on).
+    // (command_buffer.cpp:107-110 sends it under its lock, the scheduler there is always
+    // another thread.)
+    const bool event_first = SchedAgent::ReadyEventGoesFirst();
+    std::shared_ptr<XQueueReadyEvent> ready_event;
+    bool wake, launched;
     {
         Guard g(ring_mu_);
         if (reported_ == kQueueStateIdle) {
-            // Sent with the ring lock held, so a scheduler hears Ready and Idle in the order
-            // in which they happened (command_buffer.cpp:107-110).
             reported_ = kQueueStateReady;
-            SchedAgent::SendEvent(std::make_shared<XQueueReadyEvent>(kHandle, std::chrono::system_clock::now()));
+            ready_event = std::make_shared<XQueueReadyEvent>(kHandle, std::chrono::system_clock::now());
+            if (event_first) {
+                SchedAgent::SendEvent(ready_event);
+                ready_event = nullptr;
+            } else {
+                // Ready and Idle reach the scheduler in the order in which they happened:
+                // the launcher reports no Idle while this Ready is still to be sent.
+                ready_unsent_ = true;
+            }
         }
         const bool launcher_owed_nothing = owed_ == Owed::kNothing;
         owed_ = Owed::kBatchThenDrain;
@@ -127,14 +141,31 @@ void RingXQueue::Submit(std::shared_ptr<HwCommand> hw_cmd)
         // another core while the submitter goes on: after kDirectBurst submissions with no
         // wait in between, the ring it is.
         const bool streaming = ++unwaited_submits_ > kDirectBurst;
-        const bool launched = caller_may_launch_ && !streaming && parked_ && ring_count_ == 0 && TryLaunchOnCaller(hw_cmd);
+        // The first submission after a wait (or a query) is most likely waited for in its turn:
+        // launched here it gets a marker whatever the batch count says, recorded right behind
+        // it, and the wait that follows needs no marker of its own.
+        launched = caller_may_launch_ && !streaming && parked_ && ring_count_ == 0 &&
+                   TryLaunchOnCaller(hw_cmd, unwaited_submits_ == 1);
         if (launched) caller_launched_ = true;
         else PushLocked(Slot::kCommand, wait_for_launch ? hw_cmd : std::move(hw_cmd));
         // A launcher that already stands by for callers (see NextStep) needs no wake-up for a
         // command that is on the device already; it looks again by itself.
         wake = parked_ && (!launched || launcher_owed_nothing);
     }
-    if (wake) ring_cv_.notify_one();
+    // A command in the ring needs the launcher now; one that is on the device already needs
+    // it only for the drain that ends in the Idle event, so the scheduler hears first.
+    if (wake && !launched) ring_cv_.notify_one();
+    if (ready_event != nullptr) {
+        SchedAgent::SendEvent(ready_event);
+        bool idle_waits;
+        {
+            Guard g(ring_mu_);
+            ready_unsent_ = false;
+            idle_waits = idle_held_back_;
+        }
+        if (idle_waits && !(wake && launched)) ring_cv_.notify_one();
+    }
+    if (wake && launched) ring_cv_.notify_one();
     if (wait_for_launch) hw_cmd->WaitUntil(kCommandStateInFlight);
 }
 
@@ -187,14 +218,21 @@ RingXQueue::Step RingXQueue::NextStep(Pending *out)
         }
         if (owed_ == Owed::kBatchThenDrain) { owed_ = Owed::kDrain; return Step::kBatch; }
         if (owed_ == Owed::kDrain) { owed_ = Owed::kNothing; return Step::kDrain; }
+        idle_held_back_ = false;
         if (reported_ == kQueueStateReady) {
-            reported_ = kQueueStateIdle;
-            idle_round_++;
-            idle_cv_.notify_all();
-            SchedAgent::SendEvent(std::make_shared<XQueueIdleEvent>(kHandle));
+            if (ready_unsent_) {
+                // The Ready of this busy period is still with the submitter that caused it:
+                // Idle must not overtake it. That submitter wakes the launcher when it is out.
+                idle_held_back_ = true;
+            } else {
+                reported_ = kQueueStateIdle;
+                idle_round_++;
+                idle_cv_.notify_all();
+                SchedAgent::SendEvent(std::make_shared<XQueueIdleEvent>(kHandle));
+            }
         }
         parked_ = true;
-        ring_cv_.wait(g, [this]() { return ring_count_ != 0 || owed_ != Owed::kNothing; });
+        ring_cv_.wait(g, [this]() { return ring_count_ != 0 || owed_ != Owed::kNothing || (idle_held_back_ && !ready_unsent_); });
         parked_ = false;
     }
 }
@@ -405,7 +443,7 @@ void RingXQueue::LaunchFromRing(std::shared_ptr<HwCommand> cmd)
 
 // The same steps on the submitting thread, taken only when none of them would have to wait.
 // The caller holds the ring lock and has seen the launcher parked on an empty ring.
-bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd)
+bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd, bool mark)
 {
     auto *ext = dynamic_cast<HwCommandExtension *>(cmd.get());   // null for callback commands too
     if (ext == nullptr || !ext->DirectLaunchable()) return false;
@@ -425,14 +463,14 @@ bool RingXQueue::TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd)
     }
     if (MustDrainFlushablesFirst(*cmd, &marker)) return false;
     cmd->BeforeLaunch(); // does not block for a command that calls itself DirectLaunchable
-    HandOver(cmd);
+    HandOver(cmd, mark);
     direct_launches_.fetch_add(1, std::memory_order_relaxed);
     return true;
 }
 
 // win_mu_ held. A dropped command completes here without reaching the adapter; every
 // batch-th command since the last marker gets one (launch_worker.cpp:236-262).
-void RingXQueue::HandOver(const std::shared_ptr<HwCommand> &cmd)
+void RingXQueue::HandOver(const std::shared_ptr<HwCommand> &cmd, bool mark)
 {
     const int64_t idx = cmd->GetIdx();
     if (idx <= drop_through_) {
@@ -440,7 +478,7 @@ void RingXQueue::HandOver(const std::shared_ptr<HwCommand> &cmd)
         handed_over_.store(idx, std::memory_order_release);
         return;
     }
-    if (idx - last_marked_idx_ >= batch_) cmd->EnableSynchronization();
+    if (mark || idx - last_marked_idx_ >= batch_) cmd->EnableSynchronization();
 
     // (the class is final: comparing the dynamic type is exact and costs no hierarchy walk)
     if (typeid(*cmd) == typeid(HwCallbackCommand)) {

@@ -96,6 +96,8 @@ private:
     bool caller_launched_ = false;      // a submitter has launched since the launcher last stood by
     int64_t unwaited_submits_ = 0;      // submissions since anybody last asked for a drain
     XQueueState reported_ = kQueueStateIdle;
+    bool ready_unsent_ = false;         // reported_ turned Ready, the event is still with the submitter
+    bool idle_held_back_ = false;       // the launcher found the queue idle meanwhile and waits for that event to be out
     uint64_t idle_round_ = 0;
 
     // ---- in-flight window (win_mu_) ---------------------------------------------------
@@ -112,8 +114,8 @@ private:
     void ResizeWindow(int64_t threshold);
     void LauncherMain();
     void LaunchFromRing(std::shared_ptr<HwCommand> cmd);
-    bool TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd);
-    void HandOver(const std::shared_ptr<HwCommand> &cmd);         // win_mu_ held
+    bool TryLaunchOnCaller(const std::shared_ptr<HwCommand> &cmd, bool mark);
+    void HandOver(const std::shared_ptr<HwCommand> &cmd, bool mark = false);   // win_mu_ held
     bool MustDrainFlushablesFirst(const HwCommand &cmd, std::shared_ptr<HwCommand> *marker);
     std::shared_ptr<HwCommand> OldestMarker();
     bool HoldWhilePaused(Guard &g);                                // false: stopped
