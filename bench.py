@@ -635,15 +635,24 @@ def transparent_preemption():
             sock_dir = tempfile.mkdtemp(prefix="xsched-bench-")
             server = subprocess.Popen([os.path.join(lib, "xserver"), "HPF"],
                                       env=dict(base, XSCHED_SOCKET_DIR=sock_dir, XLOG_LEVEL="WARN", **extra))
+            started = time.time()
             try:
                 deadline = time.time() + 5
                 while not os.path.exists(os.path.join(sock_dir, "xsched-1.sock")) and time.time() < deadline:
                     time.sleep(0.01)
                 common = dict({"XSCHED_SOCKET_DIR": sock_dir, "XSCHED_SCHEDULER": "GLB", "XSCHED_AUTO_XQUEUE": "ON",
                                "XSCHED_AUTO_XQUEUE_LEVEL": "2", "XSCHED_SHIM_STATS": "1", "XLOG_LEVEL": "WARN"}, **extra)
-                return next_to("shim_app", dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
-                                                XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"),
-                               dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
+                out = next_to("shim_app", dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="0", XSCHED_AUTO_XQUEUE_THRESHOLD="2",
+                                               XSCHED_AUTO_XQUEUE_BATCH_SIZE="1"),
+                              dict(common, XSCHED_AUTO_XQUEUE_PRIORITY="1"))
+                if out is not None:
+                    try:   # what the daemon's threads cost while the two clients ran
+                        import psutil
+                        t = psutil.Process(server.pid).cpu_times()
+                        out["daemon_cpu_cores"] = round((t.user + t.system) / (time.time() - started), 3)
+                    except Exception:
+                        out["daemon_cpu_cores"] = None
+                return out
             finally:
                 server.terminate()
                 try:
@@ -653,9 +662,11 @@ def transparent_preemption():
                     server.wait()
                 shutil.rmtree(sock_dir, ignore_errors=True)
 
+        # Default: receivers poll briefly after each message and are up ahead of a periodic
+        # sender's next burst (csrc/sched/spin.h). Beside it: receivers that only block, and
+        # receivers that poll for 5 ms after each message, i.e. all the time here.
         under = under_daemon({})
-        # The same with the three threads that relay a preemption (daemon receiver, its round
-        # thread, the load's receiver) polling for 5 ms after each message instead of sleeping.
+        under_blocking = under_daemon({"XSCHED_WAKE_AHEAD": "OFF"})
         under_polling = under_daemon({"XSCHED_SPIN_US": "5000"})
     except (OSError, subprocess.SubprocessError, AttributeError):
         return None
@@ -665,6 +676,9 @@ def transparent_preemption():
                         "5 ms back to back; two processes, plain HIP host code, percentile = sorted[floor(p*n)]",
             "fg_alone_us": percentiles(alone.stdout), "hardware_scheduling_only": native,
             "under_xsched_shim_daemon_level2": under,
+            "p99_over_alone": (round(under["fg"]["p99"] / percentiles(alone.stdout)["p99"], 3)
+                               if under.get("fg") and percentiles(alone.stdout) else None),
+            "under_xsched_shim_daemon_level2_XSCHED_WAKE_AHEAD_OFF": under_blocking,
             "under_xsched_shim_daemon_level2_XSCHED_SPIN_US_5000": under_polling}
 
 

@@ -54,7 +54,18 @@ private:
     int fd_ = -1;
     int wake_fd_ = -1;
     std::atomic_bool removed_ { false };
-    std::chrono::steady_clock::time_point last_message_ {}; // receiver thread only
+
+    // Receiver thread only: when messages came, to be awake when the next one does.
+    using Clock = std::chrono::steady_clock;
+    std::unique_ptr<Message> TryReceive();
+    std::unique_ptr<Message> Arrived(std::unique_ptr<Message> msg);
+    Clock::time_point last_message_ {};
+    Clock::time_point burst_start_ {};       // first message after a pause; with a rhythm: the last beat
+    Clock::duration intervals_[3] {};        // between the last four such moments
+    Clock::duration period_ {};              // their common value when they agree, else zero
+    int missed_ = 0;                         // predictions in a row that nothing came of
+    bool slack_set_ = false;
+    char rx_[kMaxMessageSize];
 };
 
 class Channel

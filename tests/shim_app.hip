@@ -245,17 +245,19 @@ static int Probe(int count, int period_us)
     for (int i = 0; i < 20; ++i) Busy<<<256, 256, 0, s>>>(out, 5000);
     CHECK(hipStreamSynchronize(s));
     printf("ready\n"); fflush(stdout);
-    std::vector<double> us(count);
+    std::vector<double> us(count), launch_us(count);
     for (int i = 0; i < count; ++i) {
         const auto t0 = std::chrono::steady_clock::now();
         Busy<<<256, 256, 0, s>>>(out, 5000);
+        const auto t1 = std::chrono::steady_clock::now();
         CHECK(hipStreamSynchronize(s));
         us[i] = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+        launch_us[i] = std::chrono::duration<double, std::micro>(t1 - t0).count();
         std::this_thread::sleep_for(std::chrono::microseconds(period_us));
     }
-    if (const char *dump = getenv("SHIM_APP_PROBE_DUMP")) {   // every sample in arrival order, for a closer look at the tail
+    if (const char *dump = getenv("SHIM_APP_PROBE_DUMP")) {   // every sample in arrival order (total, of which the launch call), for a closer look at the tail
         if (FILE *f = fopen(dump, "w")) {
-            for (double v : us) fprintf(f, "%.1f\n", v);
+            for (int i = 0; i < count; ++i) fprintf(f, "%.1f %.1f\n", us[i], launch_us[i]);
             fclose(f);
         }
     }

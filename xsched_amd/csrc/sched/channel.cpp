@@ -1,7 +1,9 @@
 // Datagram channel over Unix-domain sockets.
 #include <cerrno>
 #include <cstring>
+#include <algorithm>
 #include <poll.h>
+#include <sys/prctl.h>
 #include <sys/eventfd.h>
 #include <sys/socket.h>
 #include <sys/stat.h>
@@ -89,36 +91,123 @@ bool Node::Send(const void *data, size_t size)
     }
 }
 
+// One datagram if one is there, without blocking; nullptr otherwise (errno tells which).
+std::unique_ptr<Message> Node::TryReceive()
+{
+    ssize_t n = recv(fd_, rx_, sizeof(rx_), MSG_DONTWAIT);
+    if (n < 0) return nullptr;
+    return std::make_unique<Message>(std::vector<char>(rx_, rx_ + n));
+}
+
+// Bookkeeping for every message. A message after a pause starts a burst. Without a rhythm,
+// the times between the last four burst starts become the period when they agree within an
+// eighth. With one, a burst that starts a whole number of periods after the last beat (within
+// an eighth of the period) is the next beat and corrects the period; any other burst is
+// somebody else's (another client's queue going idle, a hint) and changes nothing: the rhythm
+// is only given up when its own beats stop coming (Receive counts those).
+std::unique_ptr<Message> Node::Arrived(std::unique_ptr<Message> msg)
+{
+    const auto now = Clock::now();
+    if (now - last_message_ > kBurstWindow) {
+        if (period_ > Clock::duration::zero()) {
+            const auto since = now - burst_start_;
+            const int64_t beats = (since + period_ / 2) / period_;
+            const auto expected = period_ * beats;
+            const auto off = since > expected ? since - expected : expected - since;
+            if (beats >= 1 && off * kLatenessDivisor <= period_) {
+                if (beats == 1) period_ = (period_ * 3 + since) / 4;
+                burst_start_ = now;
+                missed_ = 0;
+            }
+        } else {
+            if (burst_start_ != Clock::time_point {}) {
+                intervals_[0] = intervals_[1];
+                intervals_[1] = intervals_[2];
+                intervals_[2] = now - burst_start_;
+                const auto mean = (intervals_[0] + intervals_[1] + intervals_[2]) / 3;
+                bool steady = intervals_[0] > Clock::duration::zero() && mean >= kShortestPeriod && mean <= kLongestPeriod;
+                for (const auto &i : intervals_) {
+                    const auto off = i > mean ? i - mean : mean - i;
+                    steady = steady && off * kLatenessDivisor <= mean;
+                }
+                if (steady) { period_ = mean; missed_ = 0; }
+            }
+            burst_start_ = now;
+        }
+    }
+    last_message_ = now;
+    return msg;
+}
+
 std::unique_ptr<Message> Node::Receive()
 {
     if (type_ != NodeType::kReceiver || removed_.load()) return nullptr;
-    std::vector<char> buf(kMaxMessageSize);
-    // Poll for a while after the last message before blocking (off unless XSCHED_SPIN_US is set).
-    const auto window = SpinWindow();
-    if (window.count() > 0) {
-        const auto give_up = last_message_ + window;
-        while (std::chrono::steady_clock::now() < give_up && !removed_.load(std::memory_order_relaxed)) {
-            ssize_t n = recv(fd_, buf.data(), buf.size(), MSG_DONTWAIT);
-            if (n >= 0) {
-                last_message_ = std::chrono::steady_clock::now();
-                buf.resize((size_t)n);
-                return std::make_unique<Message>(std::move(buf));
-            }
+    const bool ahead = WakeAhead();
+    if (ahead && !slack_set_) {
+        // the timed sleep below is meant to end on time (the default slack of a thread's timers is 50 us)
+        (void)prctl(PR_SET_TIMERSLACK, 1000UL, 0, 0, 0);
+        slack_set_ = true;
+    }
+    // 1. Poll for a while after the last message before blocking: XSCHED_SPIN_US when it is
+    //    set, else the length of a burst.
+    const auto window = SpinWindow().count() > 0 ? Clock::duration(SpinWindow()) : (ahead ? Clock::duration(kBurstWindow) : Clock::duration::zero());
+    auto poll_until = [this](Clock::time_point give_up) -> std::unique_ptr<Message> {
+        while (Clock::now() < give_up && !removed_.load(std::memory_order_relaxed)) {
+            if (auto msg = TryReceive()) return msg;
             if (errno != EAGAIN && errno != EWOULDBLOCK && errno != EINTR) return nullptr;
             __builtin_ia32_pause();
         }
+        return nullptr;
+    };
+    if (window > Clock::duration::zero()) {
+        auto until = last_message_ + window;
+        // No rhythm yet, but the last two bursts came close together: the next one is
+        // expected as soon, and learning a rhythm takes four of them. Polling through
+        // that one pause makes the second and third burst of a periodic sender find the
+        // receiver awake already (and a sender that is not periodic but this busy, always).
+        if (ahead && period_ == Clock::duration::zero() && intervals_[2] > Clock::duration::zero() &&
+            intervals_[2] <= kDensePause && last_message_ - burst_start_ <= kBurstWindow) {
+            until = std::max(until, burst_start_ + intervals_[2] + intervals_[2] / 4);
+        }
+        if (auto msg = poll_until(until)) return Arrived(std::move(msg));
+    }
+    // 2. A steady rhythm: sleep until shortly before the next burst is due, then poll until
+    //    it comes or is clearly late. kBeatsToGiveUp beats in a row that do not come and the
+    //    rhythm is forgotten.
+    Clock::time_point sleep_until {};
+    if (ahead && period_ > Clock::duration::zero() && missed_ < kBeatsToGiveUp) {
+        const auto due = burst_start_ + period_ * (missed_ + 1);
+        const auto late = std::max<Clock::duration>(period_ / kLatenessDivisor, Clock::duration(WakeAheadMargin()));
+        if (Clock::now() < due + late) sleep_until = due - WakeAheadMargin();
     }
     while (true) {
         pollfd fds[2] = { { fd_, POLLIN, 0 }, { wake_fd_, POLLIN, 0 } };
-        int rc = poll(fds, 2, -1);
+        int rc;
+        if (sleep_until != Clock::time_point {}) {
+            const auto left = sleep_until - Clock::now();
+            const auto ns = std::chrono::duration_cast<std::chrono::nanoseconds>(left).count();
+            timespec ts { (time_t)(ns > 0 ? ns / 1000000000 : 0), (long)(ns > 0 ? ns % 1000000000 : 0) };
+            rc = ppoll(fds, 2, &ts, nullptr);
+        } else {
+            rc = poll(fds, 2, -1);
+        }
         if (rc < 0) { if (errno == EINTR) continue; return nullptr; }
         if (fds[1].revents != 0 || removed_.load()) return nullptr;
+        if (rc == 0) {
+            // up ahead of the burst
+            const auto due = burst_start_ + period_ * (missed_ + 1);
+            const auto late = std::max<Clock::duration>(period_ / kLatenessDivisor, Clock::duration(WakeAheadMargin()));
+            sleep_until = Clock::time_point {};
+            if (auto msg = poll_until(due + late)) return Arrived(std::move(msg));
+            missed_++;
+            if (missed_ < kBeatsToGiveUp && !removed_.load()) sleep_until = burst_start_ + period_ * (missed_ + 1) - WakeAheadMargin();
+            else { period_ = Clock::duration::zero(); intervals_[0] = intervals_[1] = intervals_[2] = Clock::duration::zero(); }
+            continue;
+        }
         if (!(fds[0].revents & POLLIN)) continue;
-        ssize_t n = recv(fd_, buf.data(), buf.size(), 0);
-        if (n < 0) { if (errno == EINTR || errno == EAGAIN) continue; return nullptr; }
-        last_message_ = std::chrono::steady_clock::now();
-        buf.resize((size_t)n);
-        return std::make_unique<Message>(std::move(buf));
+        if (auto msg = TryReceive()) return Arrived(std::move(msg));
+        if (errno == EINTR || errno == EAGAIN || errno == EWOULDBLOCK) continue;
+        return nullptr;
     }
 }
 

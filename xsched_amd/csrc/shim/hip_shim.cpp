@@ -994,8 +994,16 @@ hipError_t hipStreamSynchronize(hipStream_t stream)
     if (xq == nullptr) return REAL(hipStreamSynchronize)(stream);
     xq->WaitAll();
     // Work that was handed to the runtime outside the XQueue (launches after a drain, graph
-    // launches, host functions, stream-ordered allocation) may still be running on the stream;
-    // on an empty stream this call returns at once.
+    // launches, host functions, stream-ordered allocation, calls this library does not
+    // intercept) may still be running on the stream: the runtime is asked as well. With a
+    // query first: the runtime's hipStreamSynchronize on a stream whose work was already
+    // waited for through an event takes 25-40 us longer once every 29 calls (measured with
+    // plain HIP: kernel, hipEventRecord, hipEventQuery until done, hipStreamSynchronize),
+    // which was the p95 of a program that launches one kernel and waits for it; its
+    // hipStreamQuery does not.
+    const hipError_t idle = REAL(hipStreamQuery)(stream);
+    if (idle == hipSuccess) return hipSuccess;
+    (void)hipGetLastError(); // "not ready" is no error of the application's call
     return REAL(hipStreamSynchronize)(stream);
 }
 
