@@ -151,12 +151,20 @@ def recorded_traffic(summary, applies=True):
     return None
 
 
-def cpu_baseline(config=2):
+def cpu_baseline(config=2, compact=False):
     """The same workload on host cores, on XSched's own host loop compiled from the reference
     sources (oracle/_ref, kind "reference"); bounded sample."""
     try:
         from oracle import cpu_baseline as cb
-        return cb.run_config1_sample(150) if config == 1 else cb.run_config2_sample(15.0, samples=300)
+        if config == 1:
+            return cb.run_config1_sample(150)
+        if config == 3:
+            return cb.run_config3_sample(100 if compact else 300)
+        if config == 4:
+            return cb.run_config4_sample(200 if compact else 600)
+        if config == 5:
+            return cb.run_config5_sample(2.0 if compact else 4.0)
+        return cb.run_config2_sample(15.0, samples=300)
     except Exception as e:  # checker libraries not built
         return {"value": None, "unit": "us", "cores": 0, "kind": "reference", "sample": f"unavailable: {e}"}
 
@@ -219,6 +227,35 @@ def full_buffer_check(H, bg_n, fg_n):
         out["level2_guarded_preempted_slices"] = {"bg": dict(check_axpy_buffer(b, 0, 0, 1, bg_n),
                                                              replayed_launches=int(res.stats[1]))}
     return out
+
+
+def check_hist_bins(b, which, q, lane_id, n, seed=0, bins=65536):
+    """All bins of a histogram lane against `applied` times the oracle's counts of the lane's
+    seeded Zipf keys (modulo 2^32), bit for bit."""
+    import numpy as np
+    import oracle
+    got, applied = b.read(which, q, 0, bins, np.uint32)
+    one = oracle.histogram(oracle.fill_zipf(seed, lane_id * 4, 0, n), bins).astype(np.uint64)
+    ok = int(one.sum()) == n and np.array_equal(got.astype(np.uint64), (one * applied) & 0xFFFFFFFF)
+    return {"ok": bool(ok), "applied": applied, "bins_checked": bins}
+
+
+def check_gemm_rows(b, which, q, lane_id, n, rows, seed=0):
+    """Rows [r, r + 4) of C, for each r, against the oracle's product of the lane's seeded
+    matrices (ascending-k fmaf, one rounding to bf16): the matrix cores sum in another order,
+    so the bar is the stated tolerance 2^-8 * |ref| + 2^-16 * sqrt(K); bit-exactness of this
+    kernel is the separate comparison of a preempted run's C with an uninterrupted one's."""
+    import numpy as np
+    import oracle
+    bmat = oracle.fill_normal_bf16(seed, lane_id * 4 + 1, 0, n * n)
+    worst, applied = 0.0, None
+    for r in rows:
+        got, applied = b.read(which, q, r * n, 4 * n, np.uint16)
+        a = oracle.fill_normal_bf16(seed, lane_id * 4, r * n, 4 * n)
+        _, want = oracle.gemm_bf16(a, bmat, 4, n, n, want_f32=True)
+        tol = np.abs(want) * 2.0 ** -8 + 2.0 ** -16 * np.sqrt(n)
+        worst = max(worst, float(np.max(np.abs(oracle.bf16_bits_to_f32(got).reshape(4, n) - want) / tol)))
+    return {"ok": bool(worst <= 1.0), "applied": applied, "rows_checked": 4 * len(rows), "worst_error_over_tolerance": round(worst, 3)}
 
 
 def breakdown_block(b, H, samples):
@@ -350,7 +387,23 @@ def config3(H, a):
     bg_n, fg_n = 8192, 1024
     cfg = H.Config(H.HPF, 1, H.spec(H.GEMM, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 1),
                    H.spec(H.GEMM, fg_n, 0, 1, 8, 4, 2, period_us=5000), 64, 0)
-    r = contended_run(H, cfg, a.steps, a.warmup, bg_warm=40, bg_cmds=24)
+    def after(b):
+        """C of the background queue after the timed phases (hundreds of commands, flushed and
+        replayed whenever the foreground became ready), then after a run of suspensions in
+        flight, then after one more command that nothing interrupts: the same bits each time.
+        Rows of both queues' C against the oracle."""
+        import numpy as np
+        contended, n_cont = b.read(0, 0, 0, bg_n * bg_n, np.uint16)
+        _, _, pres = b.preempt(20)
+        preempted, _ = b.read(0, 0, 0, bg_n * bg_n, np.uint16)
+        b.bg_alone(1)
+        clean, n_clean = b.read(0, 0, 0, bg_n * bg_n, np.uint16)
+        same = bool(np.array_equal(contended, clean) and np.array_equal(preempted, clean))
+        return {"bg_preempted_equals_uninterrupted": {"ok": same, "commands_applied": n_clean, "elements_compared": bg_n * bg_n,
+                                                      "replayed_launches": int(pres.stats[1]), "deactivations": int(pres.stats[2])},
+                "bg_rows_vs_oracle": check_gemm_rows(b, 0, 0, 1, bg_n, [0, bg_n // 2, bg_n - 4]),
+                "fg_rows_vs_oracle": check_gemm_rows(b, 1, 0, 0, fg_n, [0, fg_n - 4])}
+    r = contended_run(H, cfg, a.steps, a.warmup, bg_warm=40, bg_cmds=24, keep=after)
     fg = fg_summary(H, r["fg_alone"], r["fg_contended"])
     per_launch_ms = r["bg_alone_ms"]
     achieved = gemm_flops(bg_n) / (per_launch_ms * 1e-3) / 1e12
@@ -359,6 +412,7 @@ def config3(H, a):
                      {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
     line["dtype"] = "bf16"
     line["fg_latency_us"] = fg
+    line["bit_exact"] = dict(r["kept"], all_ok=all(v["ok"] for v in r["kept"].values()))
     line["bg"] = {"alone_TFLOPs": achieved,
                   "contended_TFLOPs": gemm_flops(bg_n) * r["bg_cont_cmds"] / r["bg_cont_elapsed"] / 1e12,
                   "commands_in_timed_region": r["bg_cont_cmds"], "level2_stats": r["stats"]}
@@ -436,7 +490,14 @@ def config4(H, a):
         cfg = H.Config(H.LAX, 4, H.spec(H.HIST, bg_n, 1, 2, BG_THRESHOLD, BG_BATCH, 0),
                        H.spec(H.HIST, fg_n, 0, 1, 8, 4, 1, laxity_us=lax, period_us=2000, lax_priority=0,
                               deadline_us=deadline), 16, 0)
-        runs[lax] = contended_run(H, cfg, a.steps, a.warmup, bg_warm=2, bg_cmds=6)
+        def after(b):
+            """Every bin of the four background queues and of the foreground queue after the
+            timed phases (repeated deactivations and replays): `applied` times the oracle's
+            counts of that queue's keys."""
+            out = {"bg%d" % q: check_hist_bins(b, 0, q, q + 1, bg_n) for q in range(4)}
+            out["fg"] = check_hist_bins(b, 1, 0, 0, fg_n)
+            return out
+        runs[lax] = contended_run(H, cfg, a.steps, a.warmup, bg_warm=2, bg_cmds=6, keep=after if lax == 300 else None)
     head = runs[300]
     fg = fg_summary(H, head["fg_alone"], head["fg_contended"])
     # Roofline of the kernel itself: one queue streaming it back to back, Level 2, guarded.
@@ -452,6 +513,7 @@ def config4(H, a):
                      {"bg_threshold": BG_THRESHOLD, "bg_batch": BG_BATCH, "fg_threshold": 8, "fg_batch": 4})
     line["dtype"] = "u32"
     line["fg_latency_us"] = fg
+    line["bit_exact"] = dict(head["kept"], all_ok=all(v["ok"] for v in head["kept"].values()))
     line["deadline_miss_rate"] = head["deadline_miss"] / a.steps
     line["by_laxity_us"] = {
         str(lax): {"deadline_miss_rate": r["deadline_miss"] / a.steps,
@@ -485,16 +547,32 @@ def config5(H, a):
     # seconds of arrivals, ~200 commands per queue and second
     duration = 2.0 if getattr(a, "compact", False) else max(min(a.steps / 100.0, 4.0), 1.0)
     cfg = H.StressConfig(H.HPF, nq, 2, 1, 4, 2, axpy_n, gemm_n, hist_n, 5000.0, 7)
+    alone_s = 0.3 if getattr(a, "compact", False) else 0.5
     with H.Bench(cfg) as b:
         b.stress(0.2)  # warm-up
+        # every queue by itself first, the other fifteen idle, with its own arrival process:
+        # what its commands take with the device to themselves
+        alone = [b.stress(alone_s, only=[i])[0][i] for i in range(nq)]
         t0 = time.perf_counter()
         lat, res = b.stress(duration)
         wall = time.perf_counter() - t0
         stats = list(res.stats)
+        # every queue's buffer against the oracle, for as many commands as were applied to it
+        exact = {}
+        for i in range(nq):
+            if i % 3 == 0:
+                exact[str(i)] = check_axpy_buffer(b, 0, i, i + 1, axpy_n, seed=7)
+            elif i % 3 == 1:
+                exact[str(i)] = check_gemm_rows(b, 0, i, i + 1, gemm_n, [0, gemm_n // 2, gemm_n - 4], seed=7)
+            else:
+                exact[str(i)] = check_hist_bins(b, 0, i, i + 1, hist_n, seed=7)
     counts = [len(x) for x in lat]
     kinds = ["axpy", "gemm", "hist"]
     by_prio = {str(i): {"kernel": kinds[i % 3], "commands": counts[i], "p50": H.pct(lat[i], 0.5),
-                        "p99": H.pct(lat[i], 0.99)} for i in range(nq)}
+                        "p99": H.pct(lat[i], 0.99), "alone_commands": len(alone[i]), "alone_p50": H.pct(alone[i], 0.5),
+                        "alone_p99": H.pct(alone[i], 0.99),
+                        "p99_ratio": (H.pct(lat[i], 0.99) / H.pct(alone[i], 0.99)) if alone[i] else None}
+               for i in range(nq)}
     hbm_bytes = sum(counts[i] * (axpy_bytes(axpy_n) if i % 3 == 0 else hist_bytes(hist_n) if i % 3 == 2 else 0)
                     for i in range(nq))
     flops = sum(counts[i] * gemm_flops(gemm_n) for i in range(nq) if i % 3 == 1)
@@ -504,6 +582,8 @@ def config5(H, a):
                      {"threshold": 4, "batch": 2, "arrival_seconds": duration})
     line["dtype"] = "mixed f32/bf16/u32"
     line["per_priority_latency_us"] = by_prio
+    line["bit_exact"] = dict(exact, all_ok=all(v["ok"] for v in exact.values()),
+                             note="axpy: slices of y, hist: all bins, bit for bit; gemm: rows within the stated tolerance of the oracle")
     line["aggregate"] = {"commands": sum(counts), "elapsed_s": res.elapsed_s,
                          "hbm_GBs": hbm_bytes / res.elapsed_s / 1e9,
                          "hbm_frac_of_peak": hbm_bytes / res.elapsed_s / 1e9 / HBM_PEAK_GBS,
@@ -698,8 +778,12 @@ def compact_of(line):
     for k in ("deadline_miss_rate", "bit_exact", "vendor_library"):
         if k in line:
             keep[k] = line[k]
+    if isinstance(keep.get("bit_exact"), dict) and "all_ok" in keep["bit_exact"]:
+        keep["bit_exact"] = keep["bit_exact"]["all_ok"]
     if "per_priority_latency_us" in line:
         keep["p99_by_priority_us"] = {k: v["p99"] for k, v in line["per_priority_latency_us"].items()}
+        keep["p99_ratio_by_priority"] = {k: (round(v["p99_ratio"], 2) if v["p99_ratio"] else None)
+                                         for k, v in line["per_priority_latency_us"].items()}
         keep["aggregate"] = {k: line["aggregate"][k] for k in ("commands", "hbm_frac_of_peak", "mfma_frac_of_peak")}
     return keep
 
@@ -717,6 +801,12 @@ def other_configurations(H, a):
         except Exception as e:  # one configuration failing must not take the headline line with it
             out[name] = {"error": repr(e)}
         out[name]["seconds"] = round(time.perf_counter() - t0, 1)
+        if name != "cfg1" and not a.skip_cpu:
+            # the same configuration on host cores (reduced sizes, stated in `sample`), on XSched's own host loop
+            base = cpu_baseline(int(name[3:]), compact=True)
+            out[name]["cpu_baseline"] = {k: base.get(k) for k in ("value", "unit", "cores", "kind", "sample", "bit_exact",
+                                                                  "fg_alone_p99_us", "deadline_miss_rate", "p99_by_priority_us")
+                                         if base.get(k) is not None}
     return out
 
 
@@ -764,11 +854,10 @@ def main():
         line["shim_launch_cost"] = shim_launch_cost()
         line["framework_loop_under_shim"] = framework_loop_under_shim()
         line["transparent_preemption"] = transparent_preemption()
-    if a.config == 2 and not a.skip_cpu:
-        line["cpu_baseline"] = cpu_baseline(2)
+    if not a.skip_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.config)
     else:
-        line["cpu_baseline"] = {"value": None, "unit": "us", "cores": 0, "kind": "reference",
-                                "sample": "skipped" if a.config == 2 else "measured for the headline workload and for --config 1"}
+        line["cpu_baseline"] = {"value": None, "unit": "us", "cores": 0, "kind": "reference", "sample": "skipped"}
     print(json.dumps(line))
 
 

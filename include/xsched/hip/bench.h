@@ -144,6 +144,13 @@ XBench *XBenchCreateStress(const XBenchStressConfig *cfg);
 XResult XBenchRunStress(XBench *b, double duration_s, double *latency_us, uint64_t cap,
                         uint64_t *counts, XBenchPhaseResult *res);
 
+/* The same with only the queues whose bit is set in `queue_mask` (bit i = queue i) taking
+ * arrivals, each with its own arrival process as above; the others stay idle. One bit set:
+ * that queue's latency with the device to itself, the figure its latency in the full run is
+ * compared with. */
+XResult XBenchRunStressQueues(XBench *b, double duration_s, uint64_t queue_mask, double *latency_us,
+                              uint64_t cap, uint64_t *counts, XBenchPhaseResult *res);
+
 /* Copy `count` elements starting at `first` of a result buffer to the host:
  * which = 0: background queue `q` output (axpy y / gemm C / hist bins),
  * which = 1: foreground output. Element size: axpy 4, gemm 2, hist 4 bytes.

@@ -10,6 +10,7 @@
 //   libhostbench.so         the shipped libpreempt.so + libhalhost.so
 // The reference ships no CPU adapter, so both builds use this repository's host adapter
 // (xsched_amd/csrc/host/host_queue.cpp) compiled against the respective headers.
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cstring>
@@ -23,7 +24,15 @@
 extern "C" {
 // oracle/kernels.c
 uint64_t oracle_stream_key(uint64_t seed, uint64_t stream);
+uint64_t oracle_bits(uint64_t key, uint64_t i);
 void oracle_fill_uniform(float *out, uint64_t first, uint64_t n, uint64_t key);
+void oracle_fill_normal_bf16(uint16_t *dst, uint64_t first, uint64_t count, uint64_t key);
+void oracle_zipf_table(uint32_t *table, uint32_t n_bins, double s);
+void oracle_fill_zipf(int32_t *dst, uint64_t first, uint64_t count, uint64_t key, const uint32_t *table, uint32_t n_bins);
+uint16_t oracle_f32_to_bf16(float f);
+void oracle_gemm_bf16(const uint16_t *A, const uint16_t *B, uint16_t *C, float *c_f32, int M, int N, int K);
+void oracle_histogram(const int32_t *keys, size_t n, uint32_t *bins, uint32_t n_bins);
+void oracle_axpy(float alpha, const float *x, float *y, size_t n);
 }
 
 namespace
@@ -148,4 +157,253 @@ int hostbench_run_fg_bg_vecadd(uint64_t bg_n, uint64_t fg_n, int64_t period_us, 
 {
     return Run(Op::kVecAdd, bg_n, fg_n, period_us, samples, threshold, batch, threshold, batch, bg_burst, alone_us,
                contended_us, bg_commands, contended_seconds, checksum);
+}
+
+
+// ---- the other configurations on host cores ------------------------------------------------
+// A lane = one XQueue over one host hardware queue with seeded inputs and one of the three
+// kernels as a host "kernel" (a function called once per work-group, so that level 2 can
+// flush and replay between work-groups exactly as on the device):
+//   AXPY       the host adapter's own command (16384 elements per work-group)
+//   GEMM       bf16 in, fp32 accumulate with one fmaf per product in ascending k, bf16 out
+//              (the oracle's arithmetic), 8 rows of C per work-group
+//   histogram  bins[key]++ with one atomic add per key, 16384 keys per work-group
+// After a run every lane's output is compared with the plain oracle functions applied as
+// often as commands were submitted (`exact`).
+#include <cmath>
+#include <memory>
+
+namespace
+{
+constexpr uint32_t kBins = 65536;
+
+struct CpuLane
+{
+    int kind = 0;              // 0 AXPY, 1 GEMM, 2 histogram
+    uint64_t n = 0;            // elements / matrix edge / keys
+    HwQueueHandle hwq = 0;
+    XQueueHandle xq = 0;
+    std::vector<float> x, y, y0;                 // AXPY
+    std::vector<uint16_t> a, b, c;               // GEMM (bf16 bits)
+    std::vector<float> a_f, bt_f;                //   A and B transposed as floats
+    std::vector<int32_t> keys;                   // histogram
+    std::vector<uint32_t> bins;
+    std::atomic<uint64_t> submitted { 0 };
+    int guarded = 0;
+
+    static float Bf16(uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; }
+
+    static void GemmWg(void *arg, uint32_t wg, uint32_t)
+    {
+        auto *l = (CpuLane *)arg;
+        const size_t n = l->n;
+        for (size_t m = (size_t)wg * 8; m < (size_t)wg * 8 + 8 && m < n; ++m) {
+            const float *arow = &l->a_f[m * n];
+            for (size_t j = 0; j < n; ++j) {
+                const float *bcol = &l->bt_f[j * n];
+                float acc = 0.f;
+                for (size_t k = 0; k < n; ++k) acc = fmaf(arow[k], bcol[k], acc);
+                l->c[m * n + j] = oracle_f32_to_bf16(acc);
+            }
+        }
+    }
+
+    static void HistWg(void *arg, uint32_t wg, uint32_t)
+    {
+        auto *l = (CpuLane *)arg;
+        const size_t lo = (size_t)wg * 16384, hi = std::min<size_t>(lo + 16384, l->n);
+        for (size_t i = lo; i < hi; ++i) {
+            const uint32_t k = (uint32_t)l->keys[i];
+            if (k < kBins) __atomic_fetch_add(&l->bins[k], 1u, __ATOMIC_RELAXED);
+        }
+    }
+
+    int Setup(int kind_, uint64_t n_, uint64_t seed, uint64_t lane_id, int level, int threshold, int batch, const uint32_t *zipf)
+    {
+        kind = kind_; n = n_; guarded = level >= 2 ? 1 : 0;
+        const uint64_t s0 = oracle_stream_key(seed, lane_id * 4), s1 = oracle_stream_key(seed, lane_id * 4 + 1);
+        if (kind == 0) {
+            x.resize(n); y.resize(n);
+            oracle_fill_uniform(x.data(), 0, n, s0);
+            oracle_fill_uniform(y.data(), 0, n, s1);
+            y0 = y;
+        } else if (kind == 1) {
+            a.resize(n * n); b.resize(n * n); c.assign(n * n, 0); a_f.resize(n * n); bt_f.resize(n * n);
+            oracle_fill_normal_bf16(a.data(), 0, n * n, s0);
+            oracle_fill_normal_bf16(b.data(), 0, n * n, s1);
+            for (size_t i = 0; i < n * n; ++i) a_f[i] = Bf16(a[i]);
+            for (size_t k = 0; k < n; ++k) for (size_t j = 0; j < n; ++j) bt_f[j * n + k] = Bf16(b[k * n + j]);
+        } else {
+            keys.resize(n); bins.assign(kBins, 0);
+            oracle_fill_zipf(keys.data(), 0, n, s0, zipf, kBins);
+        }
+        HB_CHECK(HostQueueCreate(&hwq));
+        HB_CHECK(XQueueCreate(&xq, hwq, (XPreemptLevel)level, kQueueCreateFlagNone));
+        HB_CHECK(XQueueSetLaunchConfig(xq, threshold, batch));
+        return 0;
+    }
+
+    int Submit()
+    {
+        HwCommandHandle cmd = 0;
+        if (kind == 0) HB_CHECK(HostAxpyCommandCreate(&cmd, 0.5f, x.data(), y.data(), n, guarded));
+        else if (kind == 1) HB_CHECK(HostKernelCommandCreate(&cmd, &GemmWg, this, (uint32_t)((n + 7) / 8), guarded));
+        else HB_CHECK(HostKernelCommandCreate(&cmd, &HistWg, this, (uint32_t)((n + 16383) / 16384), guarded));
+        HB_CHECK(XQueueSubmit(xq, cmd));
+        submitted++;
+        return 0;
+    }
+
+    /// The lane's output against the oracle's functions applied `submitted` times.
+    bool Exact()
+    {
+        if (XQueueWaitAll(xq) != kXSchedSuccess) return false;
+        if (kind == 0) {
+            std::vector<float> want = y0;
+            for (uint64_t t = 0, times = submitted.load(); t < times; ++t) oracle_axpy(0.5f, x.data(), want.data(), n);
+            return memcmp(want.data(), y.data(), n * 4) == 0;
+        }
+        if (kind == 1) {
+            if (submitted == 0) return true;
+            std::vector<uint16_t> want(n * n);
+            oracle_gemm_bf16(a.data(), b.data(), want.data(), nullptr, (int)n, (int)n, (int)n);
+            return memcmp(want.data(), c.data(), n * n * 2) == 0;
+        }
+        std::vector<uint32_t> one(kBins, 0);
+        oracle_histogram(keys.data(), n, one.data(), kBins);
+        const uint64_t times = submitted.load();
+        for (uint32_t k = 0; k < kBins; ++k) if (bins[k] != (uint32_t)(one[k] * times)) return false;
+        return true;
+    }
+
+    int Teardown()
+    {
+        HB_CHECK(XQueueDestroy(xq));
+        HB_CHECK(HwQueueDestroy(hwq));
+        return 0;
+    }
+};
+} // namespace
+
+// One foreground queue against `n_bg` background queues of the same kernel `kind`, at
+// `level`, under HPF (policy 1: background priority 1, foreground 2) or LAX (policy 8:
+// background constant priority 0, foreground priority 0 until `laxity_us` after it became
+// ready, then 1). `samples` foreground commands alone, then as many beside the background
+// queues streaming back to back (window 2 / 1; foreground 8 / 4). Outputs as for the AXPY
+// run, plus the foreground commands later than `deadline_us` in the contended phase and
+// whether every queue's result equals the oracle's (`exact`).
+extern "C" __attribute__((visibility("default")))
+int hostbench_run_fg_bg_kernel(int kind, uint64_t bg_n, uint64_t fg_n, int n_bg, int level, int policy,
+                               int64_t laxity_us, int64_t period_us, int64_t deadline_us, int samples,
+                               double *alone_us, double *contended_us, uint64_t *bg_commands,
+                               double *contended_seconds, uint64_t *deadline_misses, int *exact)
+{
+    std::vector<uint32_t> zipf(kBins);
+    if (kind == 2) oracle_zipf_table(zipf.data(), kBins, 1.1);
+    HB_CHECK(XHintSetScheduler(kSchedulerLocal, (XPolicyType)policy));
+    CpuLane fg;
+    std::vector<std::unique_ptr<CpuLane>> bg;
+    if (int rc = fg.Setup(kind, fg_n, 0, 0, level, 8, 4, zipf.data())) return rc;
+    for (int i = 0; i < n_bg; ++i) {
+        bg.emplace_back(std::make_unique<CpuLane>());
+        if (int rc = bg.back()->Setup(kind, bg_n, 0, (uint64_t)i + 1, level, 2, 1, zipf.data())) return rc;
+    }
+    if (policy == kPolicyLaxity) {
+        HB_CHECK(XHintLaxity(fg.xq, laxity_us, 0, 1));
+        for (auto &l : bg) HB_CHECK(XHintLaxity(l->xq, 0, 0, 0));
+    } else {
+        HB_CHECK(XHintPriority(fg.xq, 2));
+        for (auto &l : bg) HB_CHECK(XHintPriority(l->xq, 1));
+    }
+    auto run_fg = [&](double *out, uint64_t *misses) {
+        auto next = Clock::now();
+        for (int i = 0; i < samples; ++i) {
+            std::this_thread::sleep_until(next);
+            const auto t0 = Clock::now();
+            if (fg.Submit() != 0 || XQueueWaitAll(fg.xq) != kXSchedSuccess) { out[i] = -1; continue; }
+            out[i] = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+            if (misses && deadline_us > 0 && out[i] > (double)deadline_us) ++*misses;
+            next += std::chrono::microseconds(period_us);
+        }
+    };
+    run_fg(alone_us, nullptr);
+
+    std::atomic<bool> stop { false };
+    std::vector<std::thread> drivers;
+    for (auto &l : bg) {
+        drivers.emplace_back([&stop, lane = l.get()]() {
+            while (!stop.load()) {
+                for (int k = 0; k < 4 && !stop.load(); ++k) if (lane->Submit() != 0) return;
+                XQueueWaitAll(lane->xq);
+            }
+        });
+    }
+    std::this_thread::sleep_for(std::chrono::milliseconds(50));
+    uint64_t before = 0, after = 0;
+    for (auto &l : bg) before += l->submitted;
+    const auto t0 = Clock::now();
+    *deadline_misses = 0;
+    run_fg(contended_us, deadline_misses);
+    *contended_seconds = std::chrono::duration<double>(Clock::now() - t0).count();
+    for (auto &l : bg) after += l->submitted;
+    *bg_commands = after - before;
+    stop.store(true);
+    for (auto &t : drivers) t.join();
+
+    bool ok = fg.Exact();
+    for (auto &l : bg) ok = l->Exact() && ok;
+    *exact = ok ? 1 : 0;
+    if (int rc = fg.Teardown()) return rc;
+    for (auto &l : bg) if (int rc = l->Teardown()) return rc;
+    return 0;
+}
+
+// The mixed stress configuration: n_queues XQueues with priorities 0..n-1 under HPF at
+// `level`, kernels AXPY / GEMM / histogram by queue index mod 3, window 4 / 2; each queue gets
+// commands at exponentially distributed intervals (mean `mean_us`, interval k of queue i from
+// the top 53 bits of synthetic stream (seed, 1000 + i) at index k, as on the device) for
+// `duration_s` seconds and waits for each. latency_us: n_queues rows of `cap` values
+// (completion minus arrival); counts[i]: commands of queue i.
+extern "C" __attribute__((visibility("default")))
+int hostbench_run_stress(int n_queues, int level, uint64_t axpy_n, uint64_t gemm_n, uint64_t hist_n, double mean_us,
+                         uint64_t seed, double duration_s, double *latency_us, uint64_t cap, uint64_t *counts,
+                         double *elapsed_s, int *exact)
+{
+    std::vector<uint32_t> zipf(kBins);
+    oracle_zipf_table(zipf.data(), kBins, 1.1);
+    HB_CHECK(XHintSetScheduler(kSchedulerLocal, kPolicyHighestPriorityFirst));
+    std::vector<std::unique_ptr<CpuLane>> lanes;
+    for (int i = 0; i < n_queues; ++i) {
+        lanes.emplace_back(std::make_unique<CpuLane>());
+        const int kind = i % 3;
+        if (int rc = lanes.back()->Setup(kind, kind == 0 ? axpy_n : kind == 1 ? gemm_n : hist_n, seed, (uint64_t)i + 1, level, 4, 2, zipf.data())) return rc;
+        HB_CHECK(XHintPriority(lanes.back()->xq, i));
+    }
+    const auto t_begin = Clock::now() + std::chrono::milliseconds(5);
+    std::vector<std::thread> threads;
+    for (int i = 0; i < n_queues; ++i) {
+        counts[i] = 0;
+        threads.emplace_back([&, i]() {
+            CpuLane &lane = *lanes[i];
+            const uint64_t key = oracle_stream_key(seed, 1000 + (uint64_t)i);
+            double t_us = 0;
+            for (uint64_t k = 0;; ++k) {
+                const double u = (double)(oracle_bits(key, k) >> 11) * (1.0 / 9007199254740992.0);
+                t_us += -mean_us * std::log1p(-u);
+                if (t_us > duration_s * 1e6) break;
+                const auto arrival = t_begin + std::chrono::nanoseconds((int64_t)(t_us * 1e3));
+                std::this_thread::sleep_until(arrival);
+                if (lane.Submit() != 0 || XQueueWaitAll(lane.xq) != kXSchedSuccess) return;
+                const double us = std::chrono::duration<double, std::micro>(Clock::now() - arrival).count();
+                if (counts[i] < cap) latency_us[(uint64_t)i * cap + counts[i]++] = us;
+            }
+        });
+    }
+    for (auto &t : threads) t.join();
+    *elapsed_s = std::chrono::duration<double>(Clock::now() - t_begin).count();
+    bool ok = true;
+    for (auto &l : lanes) ok = l->Exact() && ok;
+    *exact = ok ? 1 : 0;
+    for (auto &l : lanes) if (int rc = l->Teardown()) return rc;
+    return 0;
 }

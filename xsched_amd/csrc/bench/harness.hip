@@ -632,7 +632,13 @@ EXPORT_C_FUNC XBench *XBenchCreateStress(const XBenchStressConfig *cfg)
 EXPORT_C_FUNC XResult XBenchRunStress(XBench *b, double duration_s, double *latency_us, uint64_t cap,
                                       uint64_t *counts, XBenchPhaseResult *res)
 {
-    if (b == nullptr || b->stress.n_queues <= 0 || (size_t)b->stress.n_queues != b->bg.size() ||
+    return XBenchRunStressQueues(b, duration_s, ~0ull, latency_us, cap, counts, res);
+}
+
+EXPORT_C_FUNC XResult XBenchRunStressQueues(XBench *b, double duration_s, uint64_t queue_mask, double *latency_us,
+                                            uint64_t cap, uint64_t *counts, XBenchPhaseResult *res)
+{
+    if (b == nullptr || b->stress.n_queues <= 0 || b->stress.n_queues > 64 || (size_t)b->stress.n_queues != b->bg.size() ||
         duration_s <= 0 || latency_us == nullptr || counts == nullptr || cap == 0) {
         return kXSchedErrorInvalidValue;
     }
@@ -644,6 +650,7 @@ EXPORT_C_FUNC XResult XBenchRunStress(XBench *b, double duration_s, double *late
     std::vector<std::thread> threads;
     for (int i = 0; i < nq; ++i) {
         counts[i] = 0;
+        if (!((queue_mask >> i) & 1)) continue;
         threads.emplace_back([&, i]() {
             Lane &lane = *b->bg[i];
             const uint64_t key = synth_stream_key(b->stress.seed, 1000 + (uint64_t)i);

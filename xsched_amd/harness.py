@@ -56,6 +56,8 @@ def lib():
         h.XBenchRunPreemptDeviceTimed.argtypes = [c_void_p, c_int, POINTER(c_double), POINTER(PhaseResult)]
         h.XBenchRunStress.argtypes = [c_void_p, c_double, POINTER(c_double), c_uint64, POINTER(c_uint64),
                                       POINTER(PhaseResult)]
+        h.XBenchRunStressQueues.argtypes = [c_void_p, c_double, c_uint64, POINTER(c_double), c_uint64,
+                                            POINTER(c_uint64), POINTER(PhaseResult)]
         h.XBenchReadOutput.argtypes = [c_void_p, c_int, c_int, c_uint64, c_uint64, c_void_p,
                                        POINTER(c_uint64)]
         _lib = h
@@ -123,10 +125,13 @@ class Bench:
         xsched_amd.check(lib().XBenchRunPreemptDeviceTimed(self.h, samples, drain, byref(res)))
         return list(drain), res
 
-    def stress(self, duration_s, cap=4096):
+    def stress(self, duration_s, cap=4096, only=None):
+        """Per-queue latency lists of a stress run; `only` = the queues that take arrivals
+        (all of them when None)."""
         nq = self.cfg.n_queues
+        mask = (1 << nq) - 1 if only is None else sum(1 << i for i in only)
         lat, counts, res = (c_double * (nq * cap))(), (c_uint64 * nq)(), PhaseResult()
-        xsched_amd.check(lib().XBenchRunStress(self.h, duration_s, lat, cap, counts, byref(res)))
+        xsched_amd.check(lib().XBenchRunStressQueues(self.h, duration_s, mask, lat, cap, counts, byref(res)))
         return [list(lat[i * cap:i * cap + counts[i]]) for i in range(nq)], res
 
     def read(self, which, q, first, count, np_dtype):
