@@ -4,6 +4,10 @@
 //                                     level 1, guarded at level 2)
 //   traffic_probe [n] [reps] hist     histogram of 2^26 Zipf keys, plain and guarded at level 2
 //   traffic_probe [n] [reps] gemm     bf16 GEMM 8192^3, plain and guarded at level 2
+//   traffic_probe [n] [reps] gemmk K  plain bf16 GEMM 8192 x 8192 x K (random bf16 inputs of about
+//                                     unit variance): the same 1024 tiles with a loop K / 64 steps
+//                                     long, prints the time per launch (how much of a launch is
+//                                     per-tile fixed cost)
 // Run it under `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`: the copy kernel's
 // counters give the scale factor of the counter, the other rows the kernels' real HBM
 // traffic per launch.
@@ -31,6 +35,56 @@ __global__ void PlainCopyKernel(const f4 *src, f4 *dst, size_t n4)
     }
 }
 
+// bf16 bits of a value in [-2, 2) from a hash of the index: cheap, and the matrix cores' power
+// draw depends on the data (all-zero inputs run at a higher clock than real ones).
+__global__ void FillRandomBf16(uint16_t *dst, size_t n, uint32_t seed)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        uint32_t h = (uint32_t)i * 2654435761u + seed;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        dst[i] = (uint16_t)((h & 0x8000u) | (0x3F00u + (h & 0xFFu)));   // sign, exponent 126..127, 7 mantissa bits
+    }
+}
+
+static int GemmOfDepth(int k, int reps, hipStream_t stream)
+{
+    const int mn = 8192;
+    uint16_t *a = nullptr, *b = nullptr, *c = nullptr;
+    CHECK_HIP(hipMalloc((void **)&a, (size_t)mn * k * 2));
+    CHECK_HIP(hipMalloc((void **)&b, (size_t)k * mn * 2));
+    CHECK_HIP(hipMalloc((void **)&c, (size_t)mn * mn * 2));
+    hipLaunchKernelGGL(FillRandomBf16, dim3(4096), dim3(256), 0, stream, a, (size_t)mn * k, 1u);
+    hipLaunchKernelGGL(FillRandomBf16, dim3(4096), dim3(256), 0, stream, b, (size_t)k * mn, 2u);
+    CHECK_HIP(hipStreamSynchronize(stream));
+    HwQueueHandle hwq;
+    XQueueHandle xq;
+    CHECK_X(HipQueueCreate(&hwq, stream));
+    CHECK_X(XQueueCreate(&xq, hwq, kPreemptLevelBlock, kQueueCreateFlagNone));
+    CHECK_X(XQueueSetLaunchConfig(xq, 2, 1));
+    auto run = [&](int count) {
+        for (int i = 0; i < count; ++i) {
+            HwCommandHandle cmd;
+            CHECK_X(HipGemmBf16CommandCreate(&cmd, a, b, c, mn, mn, k, 0));
+            CHECK_X(XQueueSubmit(xq, cmd));
+        }
+        CHECK_X(XQueueWaitAll(xq));
+    };
+    run(reps);   // the clock settles
+    hipEvent_t e0, e1;
+    CHECK_HIP(hipEventCreate(&e0)); CHECK_HIP(hipEventCreate(&e1));
+    CHECK_HIP(hipEventRecord(e0, stream));
+    run(reps);
+    CHECK_HIP(hipEventRecord(e1, stream));
+    CHECK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    printf("traffic_probe: gemmk 8192x8192x%d reps=%d ms_per_launch=%.4f TFLOPs=%.1f\n", k, reps, ms / reps,
+           2.0 * mn * mn * k / (ms / reps * 1e-3) / 1e12);
+    CHECK_X(XQueueDestroy(xq));
+    CHECK_X(HwQueueDestroy(hwq));
+    return 0;
+}
+
 int main(int argc, char **argv)
 {
     const size_t n = argc > 1 ? (size_t)atoll(argv[1]) : (size_t)1 << 28;
@@ -50,6 +104,7 @@ int main(int argc, char **argv)
     CHECK_HIP(hipStreamSynchronize(stream));
 
     CHECK_X(XHintSetScheduler(kSchedulerAppManaged, kPolicyUnknown));
+    if (argc > 4 && strcmp(argv[3], "gemmk") == 0) return GemmOfDepth(atoi(argv[4]), reps, stream);
     if (argc > 3) {
         // The harness of bench.py fills the seeded inputs and streams `reps` background commands.
         const bool hist = strcmp(argv[3], "hist") == 0;
