@@ -89,7 +89,10 @@ XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t
  *   - every call on one GPU uses that GPU's one array: calls whose kernels can overlap on a
  *     GPU (different streams, no ordering between them) race; calls on one stream do not;
  *   - nothing of the array has to be zero: each launch overwrites all it reads;
- *   - the launches are not flushable (no guard): level-2 preemption does not apply.
+ *   - the launches are not flushable (no guard): level-2 preemption does not apply;
+ *   - the address of the array on a GPU is looked up once, when the first hardware queue is
+ *     created on that GPU (HipQueueCreate) or else at the first call there: a caller that
+ *     captures this call into a graph does one of the two before the capture begins.
  * Returns after enqueueing; the caller synchronises the stream. */
 XResult HipHistogramLaunchNoAlloc(void *stream, const void *keys, size_t n, void *bins,
                                   uint32_t n_bins);

@@ -92,8 +92,17 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     stop = threading.Event()
     t = threading.Thread(target=churn, args=(xs, q, stop, 2))
     t.start()
-    for _ in range(times):
-        q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+    # A command takes some 15 us: rounds of `times` commands until the suspensions have caught
+    # the queue with work in flight a few times (one that finds nothing in flight deactivates
+    # nothing), at most a hundred rounds.
+    rounds = 0
+    while rounds < 100:
+        for _ in range(times):
+            q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+        rounds += 1
+        if hip_stats(xs, q.hwq)[2] >= 3:
+            break
+    times *= rounds
     time.sleep(0.05)
     stop.set()
     t.join()
@@ -102,7 +111,7 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     got = bins.cpu().numpy().view(np.uint32)
     q.close()
     one = oracle.histogram(keys_h, n_bins).astype(np.uint64)
-    print("stats", st, flush=True)
+    print("stats", st, "rounds", rounds, flush=True)
     assert st[2] > 0
     assert int(got.sum()) == times * n
     assert np.array_equal(got.astype(np.uint64), one * times)

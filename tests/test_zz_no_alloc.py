@@ -77,3 +77,44 @@ def test_no_alloc_histogram_refuses_what_its_array_cannot_hold(xs, gpu):
     assert h.HipHistogramLaunchNoAlloc(s, keys.data_ptr(), 0, bins.data_ptr(), 16) == xs.kXSchedSuccess
     torch.cuda.synchronize()
     assert int(bins.sum()) == 0
+
+
+def test_no_alloc_histogram_inside_a_captured_graph(xs, gpu):
+    """What the entry point is for: two calls captured into one HIP graph (the capture would
+    refuse an allocation), the graph replayed three times with eager work and a
+    synchronisation between the replays, the bins after every replay against the oracle. The
+    array's address is looked up before the capture begins (here by an eager call)."""
+    torch = gpu
+    h = xs.halhip()
+    n_a, n_b, n_bins = (1 << 22) + 77, (1 << 18) - 3, N_BINS
+    keys_a_h = oracle.fill_zipf(0, 5, 0, n_a)
+    keys_b_h = (np.random.default_rng(4).integers(0, 4096, size=n_b)).astype(np.int32)
+    keys_a, keys_b = torch.from_numpy(keys_a_h).cuda(), torch.from_numpy(keys_b_h).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    once = oracle.histogram(keys_a_h, n_bins).astype(np.uint64) + oracle.histogram(keys_b_h, n_bins).astype(np.uint64)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        xs.check(h.HipHistogramLaunchNoAlloc(side.cuda_stream, keys_b.data_ptr(), n_b, bins.data_ptr(), n_bins))   # set-up: before the capture
+    side.synchronize()
+    bins.zero_()
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    print("capturing two HipHistogramLaunchNoAlloc calls", flush=True)
+    with torch.cuda.graph(graph, stream=side):
+        xs.check(h.HipHistogramLaunchNoAlloc(side.cuda_stream, keys_a.data_ptr(), n_a, bins.data_ptr(), n_bins))
+        xs.check(h.HipHistogramLaunchNoAlloc(side.cuda_stream, keys_b.data_ptr(), n_b, bins.data_ptr(), n_bins))
+    torch.cuda.synchronize()
+    assert int(bins.sum()) == 0, "capturing must not run anything"
+
+    other = torch.zeros(1 << 20, device="cuda")
+    for replay in (1, 2, 3):
+        print("replay", replay, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = bins.cpu().numpy().view(np.uint32).astype(np.uint64)
+        assert np.array_equal(got, once * replay), "replay %d" % replay
+        other.add_(1.0)                          # the program's own eager work between the replays
+        torch.cuda.synchronize()
+    assert float(other[0]) == 3.0

@@ -174,6 +174,12 @@ public:
     virtual bool ReplayOnReactivate() const override { return guard_mode_ != 0; }
     uint32_t WorkGroups() const { return n_wg_; }
 
+    /// What the first launch would otherwise take with the XQueue's locks held: the progress
+    /// map (level 2) and whatever PrepareLaunch() borrows from the queue. Either can mean a
+    /// hipMalloc, which synchronises the device; called from HipQueue::OnHwCommandSubmit(),
+    /// on the submitting thread and before any lock of the XQueue is taken.
+    void PrepareOnSubmit(HipQueue &q);
+
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) override final;
     /// Called before every LaunchKernel() with the queue the command is launched on, for
@@ -186,6 +192,7 @@ protected:
     const int guard_mode_;
 
 private:
+    void TakeSlot(HipQueue &q);
     std::shared_ptr<GuardState> guard_state_; // keeps the slot's arena alive
     GuardState::Slot slot_;
 };
@@ -207,6 +214,7 @@ public:
     virtual XPreemptLevel GetMaxSupportedLevel() override { return kPreemptLevelDeactivate; }
     virtual void OnPreemptLevelChange(XPreemptLevel level) override;
     virtual void OnXQueueCreate() override;
+    virtual void OnHwCommandSubmit(std::shared_ptr<preempt::HwCommand> hw_cmd) override;
     /// Launch() and Synchronize() only issue stream calls under the caller's lock; the
     /// calling thread's current device is switched for the call and put back.
     virtual bool SupportDirectLaunch() override { return true; }
@@ -239,5 +247,24 @@ private:
 
 /// Microseconds a marker wait polls before it blocks in the driver.
 int64_t SyncSpinMicros();
+
+/// While a stream of the process captures a graph in the default (global) mode, the runtime
+/// refuses waits, queries and allocations from every thread that has not declared itself
+/// relaxed, and invalidates the capture on top. The adapter's own waits and allocations
+/// concern its own streams and markers, never a capturing one (the shim leaves a capturing
+/// stream to the runtime), so they run relaxed; the thread's mode is put back afterwards
+/// because the thread may be the application's.
+class RelaxedCaptureScope
+{
+public:
+    RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
+    ~RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
+private:
+    hipStreamCaptureMode mode_ = hipStreamCaptureModeRelaxed;
+};
+
+/// Looks up, once per device, where HipHistogramLaunchNoAlloc's static scratch array lives on
+/// `device` (which must be the calling thread's current device). False if the runtime refuses.
+bool ResolveNoAllocScratch(int device);
 
 } // namespace xsched::hip

@@ -30,28 +30,30 @@ namespace
 /// pool's size is read from the environment when the runtime starts, so it is asked for when
 /// this library is loaded; a value the user has set stays, and XSCHED_HIP_SIGNAL_POOL=0 keeps
 /// this library from touching the variable (any other number is the size asked for).
+bool g_signal_pool_asked_for = false;   // this library set the variable (it was not set before)
+
 __attribute__((constructor)) void AskForLargerSignalPool()
 {
     int64_t size = 512;
     GetEnvInt64("XSCHED_HIP_SIGNAL_POOL", size);
     if (size <= 0) return;
+    g_signal_pool_asked_for = getenv("ROC_SIGNAL_POOL_SIZE") == nullptr;
     (void)setenv("ROC_SIGNAL_POOL_SIZE", std::to_string(size).c_str(), 0 /* keep what is set */);
 }
 
-/// While a stream of the process captures a graph in the default (global) mode, the runtime
-/// refuses waits, queries and allocations from every thread that has not declared itself
-/// relaxed, and invalidates the capture on top. The adapter's own waits and allocations
-/// concern its own streams and markers, never a capturing one (the shim leaves a capturing
-/// stream to the runtime), so they run relaxed; the thread's mode is put back afterwards
-/// because the thread may be the application's.
-class RelaxedCaptureScope
+/// Said once, when the first queue is created: what the variable holds and who set it. The
+/// runtime reads it at its first call in the process, so a value set by this library only
+/// counts if the library was loaded before that (a program that used the GPU first, then
+/// loaded the adapter, has the runtime's own pool of 64 whatever the variable says now).
+void ReportSignalPool()
 {
-public:
-    RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
-    ~RelaxedCaptureScope() { (void)hipThreadExchangeStreamCaptureMode(&mode_); }
-private:
-    hipStreamCaptureMode mode_ = hipStreamCaptureModeRelaxed;
-};
+    static std::once_flag once;
+    std::call_once(once, []() {
+        const char *v = getenv("ROC_SIGNAL_POOL_SIZE");
+        XINFO("ROC_SIGNAL_POOL_SIZE=%s (%s); the HIP runtime reads it at its first call in the process", v ? v : "(unset)",
+              g_signal_pool_asked_for ? "set by this library when it was loaded" : "as found in the environment");
+    });
+}
 
 } // namespace
 
@@ -382,17 +384,14 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
     g.flushed = q.Guard()->FlushedDevPtr();
 
     if (guarded && level2) {
-        if (slot_.done == nullptr) {
-            XASSERT(n_wg_ <= GuardState::kMaxWorkGroups, "too many work-groups for a guarded command");
-            guard_state_ = q.Guard();
-            slot_ = guard_state_->AcquireSlot();
-            if (slot_.needs_clear) {
-                // a kernel, not hipMemsetAsync: a stream under capture records no memset node
-                static_assert(GuardState::kSlotBytes % (16 * 256) == 0, "one 16-byte store per thread");
-                ClearSlotKernel<<<dim3((unsigned)(GuardState::kSlotBytes / 16 / 256)), dim3(256), 0, q.Stream()>>>((uint4 *)slot_.done);
-                hipError_t err = hipGetLastError();
-                if (err != hipSuccess) return err;
-            }
+        if (slot_.done == nullptr) TakeSlot(q);   // normally taken at submission already
+        if (slot_.needs_clear) {
+            slot_.needs_clear = false;
+            // a kernel, not hipMemsetAsync: a stream under capture records no memset node
+            static_assert(GuardState::kSlotBytes % (16 * 256) == 0, "one 16-byte store per thread");
+            ClearSlotKernel<<<dim3((unsigned)(GuardState::kSlotBytes / 16 / 256)), dim3(256), 0, q.Stream()>>>((uint4 *)slot_.done);
+            hipError_t err = hipGetLastError();
+            if (err != hipSuccess) return err;
         }
         g.done = slot_.done;
         g.gen = slot_.gen;
@@ -400,6 +399,19 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
     hipError_t err = PrepareLaunch(q);
     if (err != hipSuccess) return err;
     return LaunchKernel(q.Stream(), guarded, g);
+}
+
+void HipGuardedCommand::TakeSlot(HipQueue &q)
+{
+    XASSERT(n_wg_ <= GuardState::kMaxWorkGroups, "too many work-groups for a guarded command");
+    guard_state_ = q.Guard();
+    slot_ = guard_state_->AcquireSlot();
+}
+
+void HipGuardedCommand::PrepareOnSubmit(HipQueue &q)
+{
+    if (guard_mode_ != 0 && q.Level() >= kPreemptLevelDeactivate && slot_.done == nullptr) TakeSlot(q);
+    (void)PrepareLaunch(q);   // idempotent; Enqueue() calls it again and reports what it returns
 }
 
 // ---- HipQueue ----------------------------------------------------------------
@@ -413,6 +425,10 @@ HipQueue::HipQueue(hipStream_t stream): stream_(stream)
     guard_ = std::make_shared<GuardState>(device_);
     scratch_ = std::make_shared<ScratchPool>(device_);
     HIP_ASSERT(hipStreamCreateWithFlags(&op_stream_, hipStreamNonBlocking)); // default priority
+    // The entry point that allocates nothing needs the address of its static array on this
+    // device; looked up here, at set-up, it never has to be looked up under a graph capture.
+    ResolveNoAllocScratch(device_);
+    ReportSignalPool();
     // Nothing of the application may still be running on the stream (hip_queue.cpp:35-36).
     HIP_ASSERT(hipStreamSynchronize(stream_));
 }
@@ -503,6 +519,18 @@ size_t ScratchPool::Buffers()
 {
     std::lock_guard<std::mutex> lock(mtx_);
     return buffers_.size();
+}
+
+// On the submitting thread, before the XQueue takes any of its locks: a guarded command takes
+// its progress map and scratch buffer here, so that a launch under those locks (the launch
+// thread's, or the submitter's own direct launch) never waits for an allocation, and a
+// scheduler's Suspend() never waits for such a launch.
+void HipQueue::OnHwCommandSubmit(std::shared_ptr<HwCommand> hw_cmd)
+{
+    auto *guarded = dynamic_cast<HipGuardedCommand *>(hw_cmd.get());
+    if (guarded == nullptr) return;
+    DeviceScope scope(device_);
+    guarded->PrepareOnSubmit(*this);
 }
 
 void HipQueue::Launch(std::shared_ptr<HwCommand> hw_cmd)

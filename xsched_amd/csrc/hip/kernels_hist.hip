@@ -782,11 +782,17 @@ std::mutex g_scratch_mtx;
 uint32_t *g_scratch_ptr[kNoAllocMaxDevices] = {};
 
 /// Device address of `scratch` on `device`, which must be the calling thread's current device.
-/// Looked up once per device; nullptr (and a warning) if the runtime refuses.
+/// Looked up once per device (when a hardware queue is created there, else at the entry
+/// point's first call on it); nullptr (and a warning) if the runtime refuses. The first
+/// lookup may load the code object, which allocates: it runs with the thread's capture mode
+/// relaxed, so a capture under way on ANOTHER stream is not invalidated by it, but it cannot
+/// be part of a capture itself: the first call on a device comes before the capture begins.
 uint32_t *ScratchOnCurrentDevice(int device)
 {
+    if (device < 0 || device >= kNoAllocMaxDevices) return nullptr;
     std::lock_guard<std::mutex> lock(g_scratch_mtx);
     if (g_scratch_ptr[device] != nullptr) return g_scratch_ptr[device];
+    RelaxedCaptureScope relaxed;
     uint32_t *ptr = nullptr;
     const hipError_t err = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess || ptr == nullptr) {
@@ -798,6 +804,11 @@ uint32_t *ScratchOnCurrentDevice(int device)
     return ptr;
 }
 } // namespace
+
+namespace xsched::hip
+{
+bool ResolveNoAllocScratch(int device) { return ScratchOnCurrentDevice(device) != nullptr; }
+} // namespace xsched::hip
 
 EXPORT_C_FUNC XResult HipHistogramLaunchNoAlloc(void *stream_ptr, const void *keys, size_t n, void *bins,
                                                 uint32_t n_bins)
@@ -828,13 +839,8 @@ EXPORT_C_FUNC XResult HipHistogramLaunchNoAlloc(void *stream_ptr, const void *ke
         // As few groups as the limit allows, each with a whole number of load units; every
         // group stores its complete partial (all-zero after an overflow recount), so nothing
         // of an earlier call's contents is read and nothing has to be cleared.
-        uint32_t chunk = hist::ChunkFor(n, hist::kMergeMinChunk);
-        uint64_t n_wg = (n + chunk - 1) / chunk;
-        if (n_wg > kNoAllocMaxGroups) {
-            const uint64_t per = (n + kNoAllocMaxGroups - 1) / kNoAllocMaxGroups;
-            chunk = (uint32_t)((per + hist::kMinChunk - 1) / hist::kMinChunk * hist::kMinChunk);
-            n_wg = (n + chunk - 1) / chunk;
-        }
+        const uint32_t chunk = hist::ChunkFor(n, hist::kMergeMinChunk);   // grows with n: at most 256 groups up to 2^26 keys
+        const uint64_t n_wg = (n + chunk - 1) / chunk;
         XASSERT(n_wg <= kNoAllocMaxGroups && chunk <= hist::kMaxChunk, "group count %llu / chunk %u out of range",
                 (unsigned long long)n_wg, chunk);
         const XGuardArgs inert {};

@@ -1,6 +1,8 @@
 // See http.h.
+#include <algorithm>
 #include <arpa/inet.h>
 #include <cerrno>
+#include <chrono>
 #include <cstring>
 #include <netinet/in.h>
 #include <poll.h>
@@ -17,6 +19,7 @@ namespace
 {
 
 constexpr size_t kMaxRequestBytes = 1 << 16;
+constexpr int kRequestDeadlineSeconds = 3;   // for a whole request, headers and body
 
 int HexDigit(char c)
 {
@@ -49,6 +52,7 @@ const char *Reason(int status)
     case 400: return "Bad Request";
     case 404: return "Not Found";
     case 405: return "Method Not Allowed";
+    case 408: return "Request Timeout";
     case 413: return "Payload Too Large";
     default:  return "Internal Server Error";
     }
@@ -125,15 +129,24 @@ void HttpServer::Serve()
 
 void HttpServer::ServeOne(int fd)
 {
+    // One thread serves every client, so a request has a deadline as a whole, not only per
+    // read: a client that sends a byte every second would otherwise hold the control plane
+    // (and Stop()) for as long as it likes. Past the deadline it is answered 408 and dropped.
+    const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(kRequestDeadlineSeconds);
+    bool timed_out = false;
+    auto read_more = [&](char *into, size_t cap) -> ssize_t {
+        while (true) {
+            const auto left = std::chrono::duration_cast<std::chrono::milliseconds>(deadline - std::chrono::steady_clock::now()).count();
+            if (left <= 0 || stop_.load()) { timed_out = true; return -1; }
+            pollfd pfd { fd, POLLIN, 0 };
+            const int rc = poll(&pfd, 1, (int)std::min<int64_t>(left, 100));
+            if (rc < 0 && errno != EINTR) return -1;
+            if (rc > 0) return recv(fd, into, cap, 0);
+        }
+    };
     std::string raw;
     size_t header_end = std::string::npos;
     char buf[4096];
-    while (header_end == std::string::npos && raw.size() < kMaxRequestBytes) {
-        const ssize_t n = recv(fd, buf, sizeof(buf), 0);
-        if (n <= 0) return;
-        raw.append(buf, (size_t)n);
-        header_end = raw.find("\r\n\r\n");
-    }
     HttpResponse res;
     HttpRequest req;
     auto reply = [&]() {
@@ -142,6 +155,12 @@ void HttpServer::ServeOne(int fd)
         head += "Content-Length: " + std::to_string(res.body.size()) + "\r\nConnection: close\r\n\r\n";
         SendAll(fd, head + res.body);
     };
+    while (header_end == std::string::npos && raw.size() < kMaxRequestBytes) {
+        const ssize_t n = read_more(buf, sizeof(buf));
+        if (n <= 0) { if (timed_out) { res.status = 408; reply(); } return; }
+        raw.append(buf, (size_t)n);
+        header_end = raw.find("\r\n\r\n");
+    }
     if (header_end == std::string::npos) { res.status = 413; reply(); return; }
 
     // request line
@@ -188,8 +207,8 @@ void HttpServer::ServeOne(int fd)
     }
     req.body = raw.substr(header_end + 4);
     while (req.body.size() < content_length) {
-        const ssize_t n = recv(fd, buf, sizeof(buf), 0);
-        if (n <= 0) return;
+        const ssize_t n = read_more(buf, sizeof(buf));
+        if (n <= 0) { if (timed_out) { res.status = 408; reply(); } return; }
         req.body.append(buf, (size_t)n);
     }
     req.body.resize(content_length);
