@@ -262,9 +262,19 @@ private:
 
 } // namespace
 
+/// Up to how many queues a submitter runs the round that its own Ready event asks for
+/// (XSCHED_INLINE_READY_ROUNDS_MAX_QUEUES).
+static size_t MaxQueuesForSubmitterRounds()
+{
+    static const size_t n = []() {
+        int64_t v = 8;
+        return GetEnvInt64("XSCHED_INLINE_READY_ROUNDS_MAX_QUEUES", v) && v >= 0 ? (size_t)v : (size_t)8;
+    }();
+    return n;
+}
+
 class LocalScheduler::Rounds
 {
-    static constexpr size_t kMaxQueuesForSubmitterRounds = 8;
 
 public:
     Rounds(LocalScheduler *owner, XPolicyType type): owner_(owner) { Install(type); }
@@ -314,7 +324,7 @@ public:
             // A round costs its caller a pass over every queue; for a submitter that is time
             // before its own launch. With many queues the round thread's wake-up is the
             // smaller price (measured with 16: +3 us at every queue's median).
-            if (mode == kRoundsOnCallersReady && mirror_.View().xqueue_status.size() > kMaxQueuesForSubmitterRounds) {
+            if (mode == kRoundsOnCallersReady && mirror_.View().xqueue_status.size() > MaxQueuesForSubmitterRounds()) {
                 round.unlock();
                 inbox_.Put(std::move(event));
                 return;
