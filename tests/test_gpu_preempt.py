@@ -453,3 +453,34 @@ def test_user_written_guarded_kernel_is_flushed_and_replayed_exactly_once(xs, gp
     assert h.HipGuardedKernelCommandCreate(byref(cmd), func, 0, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipGuardedKernelCommandCreate(byref(cmd), func, (1 << 18) + 1, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipGuardedKernelCommandCreate(byref(cmd), None, 4, 256, 1, 1, None, None, 0, 0) == xs.kXSchedErrorInvalidValue
+
+
+def test_an_event_destroyed_after_its_record_command_completed_is_not_asked_again(xs, gpu):
+    """The adapter waits for a queue through the marker of the newest command, and for an
+    event-record command that marker is the application's own event. Once the XQueue has seen
+    the command complete the application may destroy the event: a later wait for the (empty)
+    hardware queue, here the one inside XQueueSuspend(SyncHwQueue), must not touch it."""
+    import ctypes
+    torch = gpu
+    hip = ctypes.CDLL("libamdhip64.so")
+    event = ctypes.c_void_p()
+    assert hip.hipEventCreateWithFlags(byref(event), 2) == 0  # hipEventDisableTiming
+    n = 1 << 20
+    print("case destroyed-event", flush=True)
+    x = torch.ones(n, device="cuda"); y = torch.zeros(n, device="cuda")
+    q = Queue(xs, torch, level=2, threshold=4, batch=2)
+    record = c_uint64()
+    xs.check(xs.halhip().HipEventRecordCommandCreate(byref(record), event))
+    q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    q.submit(record.value)                   # the newest command on the stream
+    q.wait()
+    assert hip.hipEventDestroy(event) == 0
+    p = xs.preempt()
+    for _ in range(3):
+        xs.check(p.XQueueSuspend(q.xq, xs.kQueueSuspendFlagSyncHwQueue))
+        xs.check(p.XQueueResume(q.xq, 0))
+    q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+    q.wait()
+    got = y.cpu().numpy()
+    q.close()
+    assert np.all(got == 1.0)

@@ -568,8 +568,11 @@ void HipQueue::Synchronize()
     if (tail != nullptr) {
         // (a replay re-records this marker behind the replayed work: still the stream's end;
         // an event-record command is waited for through the application's event, as its
-        // XQueue waits for it as a batch marker: hip_command.h:197-219)
-        tail->Synchronize();
+        // XQueue waits for it as a batch marker: hip_command.h:197-219. Once its XQueue has
+        // seen the command complete, the application is free to destroy that event, so a
+        // completed command is not asked again: nothing newer is on the stream, or it would
+        // be the tail.)
+        if (tail->GetState() < kCommandStateCompleted) tail->Synchronize();
         std::lock_guard<std::mutex> lock(tail_mtx_);
         if (tail_marked_ == tail) tail_marked_ = nullptr;   // done: nothing of the stream is left to wait for, and the command is let go
         return;
