@@ -83,7 +83,7 @@ XResult HipHistogramCommandCreate(HwCommandHandle *cmd, const void *keys, size_t
  * No counterpart in the reference. It is for callers that cannot allocate device memory where
  * they call it: code under HIP graph capture, tight serving loops, harnesses that forbid
  * allocation. The partial histograms that HipHistogramCommandCreate keeps in a buffer of its
- * queue's pool live in a static device array of 17 MiB (256 partials) instead, which every
+ * queue's pool live in a static device array of 16.25 MiB (256 partials) instead, which every
  * GPU the library has run this call on holds until the process ends. Limits and rules:
  *   - n <= 2^26 keys (InvalidValue and a warning above that); n_bins <= 65536;
  *   - every call on one GPU uses that GPU's one array: calls whose kernels can overlap on a

@@ -113,8 +113,10 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     one = oracle.histogram(keys_h, n_bins).astype(np.uint64)
     print("stats", st, "rounds", rounds, flush=True)
     assert st[2] > 0
-    assert int(got.sum()) == times * n
-    assert np.array_equal(got.astype(np.uint64), one * times)
+    # The bins are 32-bit and add with wrap-around: after enough rounds the hottest bin of a
+    # Zipf key set passes 2^32, in the device's counters as in the oracle's.
+    assert np.array_equal(got.astype(np.uint64), (one * times) & 0xFFFFFFFF)
+    assert int(got.sum()) % (1 << 32) == (times * n) % (1 << 32)
 
 
 @pytest.mark.parametrize("tile", [128, 256])

@@ -25,7 +25,7 @@
 // bins w, w + 16384, w + 32768, w + 49152 in its bytes 0..3, one ds_add of
 // 1 << 8 * (key >> 14) per key. One vote per iteration tells whether every key of the wave is
 // below n_bins, so the add needs no branch. The group then stores a partial histogram of
-// 68 KiB (the byte words as they are, the per-lane counters summed) into a scratch buffer,
+// 65 KiB (the byte words as they are, the per-lane counters summed) into a scratch buffer,
 // and a second kernel sums the partials column by column and adds the totals to the result
 // with one 64-bit atomic per pair of bins. A byte overflows only when one bin outside the
 // first 256 takes 256 keys of a chunk (0.1 % of it; the hottest such bin of a Zipf(1.1)
@@ -35,7 +35,7 @@
 // all-zero partial and recounts its chunk the slow way (32-bit counters, two passes over its
 // keys, atomic sweep into the result). The first version of this layout kept 16-bit halves
 // for every bin and ballot counters for bins 0 and 1: partials of 128 KiB (32 MiB written
-// and read back per 2^26 keys, now 17 MiB), 14 vector instructions per key (now 10), and
+// and read back per 2^26 keys, now 16.25 MiB), 14 vector instructions per key (now 10), and
 // LDS adds that serialised on the hot bins.
 //
 // One kernel (above 2^28 keys, where the partials would need more than 128 MiB of
@@ -104,13 +104,28 @@ constexpr uint32_t kColdWords = 1u << 14;           // byte counters: word w, by
 constexpr uint32_t kWarmBins = 256;                 // bins below this have 32-bit counters of their own
 constexpr uint32_t kCountWords = kColdWords + kWarmBins * 64;   // LDS words in use: byte words, then a counter per warm bin and lane
 static_assert(kCountWords <= kLdsBins, "the merge layout's counters fit the group's LDS array");
-// A partial histogram in memory is kMergeGroups columns, one per merge group: 64 byte words,
-// then one 32-bit word with the count of bin <column> (the sum of its per-lane counters),
-// then padding to a multiple of 16 bytes.
+// The partial histograms of a launch in memory, n_part of them (one per counting group): the
+// byte words column by column, one column per merge group, and within a column partial by
+// partial: column c of partial p is the 64 words (256 bytes, two whole cache lines) at
+// ((c * n_part) + p) * 64. A merge group therefore reads ONE contiguous run of n_part * 256
+// bytes, and a counting group stores its partial as 256 pieces of two lines each. (Partial by
+// partial, column by column inside, a merge group read 272 bytes out of every 68 KiB: three
+// lines touched for two and a bit used, 1.41 times its bytes in traffic.) Behind the byte
+// words: the counts of bins 0..255, which are kept outside the bytes, partial by partial
+// (1 KiB each).
 constexpr uint32_t kMergeGroups = 256;
 constexpr uint32_t kMergeWords = kColdWords / kMergeGroups;          // byte words per column (64)
-constexpr uint32_t kColumnWords = kMergeWords + 4;
-constexpr uint32_t kPartialWords = kMergeGroups * kColumnWords;      // 68 KiB
+constexpr uint32_t kPartialWords = kColdWords + kWarmBins;           // 65 KiB of scratch per counting group
+
+/// Where column `column` of partial `p` lies, and where that partial's 256 outside counts do.
+__host__ __device__ inline size_t ColumnAt(uint32_t column, uint32_t p, uint32_t n_part)
+{
+    return ((size_t)column * n_part + p) * kMergeWords;
+}
+__host__ __device__ inline size_t OutsideAt(uint32_t p, uint32_t n_part)
+{
+    return (size_t)n_part * kColdWords + (size_t)p * kWarmBins;
+}
 constexpr uint32_t kMaxPartials = 1024;
 static_assert(kWarmBins == kMergeGroups && kHotBins <= kWarmBins, "column j carries the outside count of bin j");
 constexpr uint64_t kMergeMinKeys = 1;             // the two-kernel layout wins at every size measured
@@ -500,11 +515,17 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 
     const uint32_t rot = (blockIdx.x * 37u) & (kSegs - 1);
     if (kMerge) {
-        uint32_t *part = partials + (size_t)blockIdx.x * kPartialWords;
+        const uint32_t me = blockIdx.x, n_part = gridDim.x;
+        uint32_t *const outside = partials + OutsideAt(me, n_part);
         uint32_t counted = 0;
-        for (uint32_t i = tid * 4; i < kColdWords; i += kThreads * 4) {
+        // Every group starts at a column of its own: column c of all partials is one run of
+        // n_part * 256 bytes, and groups that all wrote column 0 first, then column 1, would
+        // all be storing into the same few DRAM pages at any moment.
+        const uint32_t turn = ((me * 37u) & (kMergeGroups - 1)) * kMergeWords;
+        for (uint32_t k = tid * 4; k < kColdWords; k += kThreads * 4) {
+            const uint32_t i = (k + turn) & (kColdWords - 1);
             const u32x4 w = *(const u32x4 *)&sh.bins[i];
-            *(u32x4 *)&part[(i / kMergeWords) * kColumnWords + i % kMergeWords] = w;
+            *(u32x4 *)&partials[ColumnAt(i / kMergeWords, me, n_part) + i % kMergeWords] = w;
             counted += ByteSum(w);
         }
         {
@@ -519,7 +540,7 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             counted += warm;
             warm += __shfl_xor(warm, 1);
             warm += __shfl_xor(warm, 2);
-            if (tid % 4 == 0) *(u32x4 *)&part[(tid / 4) * kColumnWords + kMergeWords] = u32x4 { warm, 0, 0, 0 };
+            if (tid % 4 == 0) outside[tid / 4] = warm;
         }
         LdsAdd(&sh.sum, counted);
         __syncthreads();
@@ -531,7 +552,10 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
             // A byte counter overflowed: this group's partial counts nothing, and the chunk
             // is counted again with 32-bit counters, one half of the bins at a time.
             __syncthreads();
-            for (uint32_t i = tid * 4; i < kPartialWords; i += kThreads * 4) *(u32x4 *)&part[i] = u32x4 { 0, 0, 0, 0 };
+            for (uint32_t i = tid * 4; i < kColdWords; i += kThreads * 4) {
+                *(u32x4 *)&partials[ColumnAt(i / kMergeWords, me, n_part) + i % kMergeWords] = u32x4 { 0, 0, 0, 0 };
+            }
+            if (tid < kWarmBins) outside[tid] = 0;
             for (uint32_t first = 0; first < n_bins; first += kLdsBins) {
                 const uint32_t count = n_bins - first < kLdsBins ? n_bins - first : kLdsBins;
                 ClearBins(sh);
@@ -573,8 +597,10 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 /// Sums the partial histograms of the counting groups and adds the totals to bins. Group j
 /// owns column j of every partial: 64 words of byte counters (word w, byte b = bin
 /// w + b * 16384) and the count of bin j, which is kept outside the bytes. Thread (row, col)
-/// reads four byte words of its column from partials row, row + 64, ...; the threads of
-/// col 0 also read the outside count. The group's progress byte is first_wg + j.
+/// reads four byte words of its column from partials row, row + 64, ... (the sixteen threads
+/// of a row one partial's 256 bytes, the four rows of a wave four neighbouring partials: one
+/// KiB in a piece); the threads of col 0 also read the outside count. The group's progress
+/// byte is first_wg + j.
 template <bool kGuard>
 __global__ __launch_bounds__(kThreads)
 void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part, uint32_t *__restrict__ bins,
@@ -590,12 +616,11 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
     const uint32_t tid = threadIdx.x;
     const uint32_t col = tid % kCols, row = tid / kCols;
     const uint32_t column = blockIdx.x;
-    const uint32_t word0 = column * kColumnWords + col * 4;
     auto load_words = [&](uint32_t p) {
-        return p < n_part ? *(const u32x4 *)(partials + (size_t)p * kPartialWords + word0) : u32x4 { 0, 0, 0, 0 };
+        return p < n_part ? *(const u32x4 *)(partials + ColumnAt(column, p, n_part) + col * 4) : u32x4 { 0, 0, 0, 0 };
     };
     auto load_outside = [&](uint32_t p) {
-        return col == 0 && p < n_part ? partials[(size_t)p * kPartialWords + column * kColumnWords + kMergeWords] : 0u;
+        return col == 0 && p < n_part ? partials[OutsideAt(p, n_part) + column] : 0u;
     };
     // even[i] holds bytes 0 and 2 of word i in its halves, odd[i] bytes 1 and 3; a thread adds
     // at most kMaxPartials / kRows = 16 values of 255 into a half.
@@ -775,7 +800,7 @@ constexpr uint32_t kNoAllocMaxGroups = 256;                       // counting wo
 constexpr uint64_t kNoAllocMaxKeys = (uint64_t)kNoAllocMaxGroups * hist::kMaxChunk; // 2^26
 constexpr size_t kNoAllocScratchWords = (size_t)kNoAllocMaxGroups * hist::kPartialWords;
 
-static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];          // 17 MiB
+static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];          // 16.25 MiB
 
 constexpr int kNoAllocMaxDevices = 64;
 std::mutex g_scratch_mtx;
