@@ -502,11 +502,11 @@ def config4(H, a):
     fg = fg_summary(H, head["fg_alone"], head["fg_contended"])
     # Roofline of the kernel itself: one queue streaming it back to back, Level 2, guarded.
     # Five alternating rounds of 120 commands, the median of each form: a single round moves
-    # by a microsecond with where the buffers of that round happen to lie. 240 untimed
-    # commands (15 ms) come first: on some boxes the first 10 ms of this kernel after an idle
-    # stretch run at 80-95 us per command, with either form, before settling at 57-59.
-    rounds = [(bg_ms_per_launch(H, H.HIST, bg_n, 2, 1, 120, 240),
-               None if a.quick else bg_ms_per_launch(H, H.HIST, bg_n, 1, 0, 120, 240)) for _ in range(3 if compact else 5)]
+    # by a microsecond with where the buffers of that round happen to lie. 120 untimed
+    # commands come first (the first ones allocate the queue's scratch buffers and clear
+    # their progress maps: 61-63 us per command over the first 120, 55-57 afterwards).
+    rounds = [(bg_ms_per_launch(H, H.HIST, bg_n, 2, 1, 120, 120),
+               None if a.quick else bg_ms_per_launch(H, H.HIST, bg_n, 1, 0, 120, 120)) for _ in range(3 if compact else 5)]
     per_launch_ms = sorted(r[0] for r in rounds)[len(rounds) // 2]
     achieved = hist_bytes(bg_n) / (per_launch_ms * 1e-3) / 1e9
     line = base_line(a, fg["contended_p99"], head["wall_s"],

@@ -37,6 +37,12 @@ XResult HipQueueCreate(HwQueueHandle *hwq, void *stream);
  * block in the driver, [6] progress-map slots in use, [7] current preempt epoch. */
 XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
 
+/* Device memory the queue's pools hold for guarded commands, for tests. `out` receives 4
+ * values: [0] scratch buffers allocated (the partial histograms of histogram commands),
+ * [1] their bytes, [2] progress-map slots allocated, [3] progress-map slots in use. Both
+ * pools grow with what is launched and not yet destroyed, not with what waits in the XQueue. */
+XResult HipQueueGetPoolStats(HwQueueHandle hwq, uint64_t *out);
+
 /* For tests of the guard protocol: stores the queue's current preempt epoch into its
  * "flushed" word, as a work-group does that leaves because a deactivation reached it.
  * Guarded launches of that epoch then do nothing (they wait for a replay, which only a

@@ -119,6 +119,34 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     assert int(got.sum()) % (1 << 32) == (times * n) % (1 << 32)
 
 
+def test_commands_waiting_in_the_xqueue_hold_no_device_memory(xs, gpu):
+    """A burst of guarded histogram commands far deeper than the in-flight window: the
+    queue's pools (partial-histogram buffers, progress maps) grow with what is launched and
+    not yet destroyed, not with what waits in the XQueue."""
+    torch = gpu
+    n, n_bins, burst = 1 << 24, 65536, 96
+    print(f"case pool-growth n={n} burst={burst}", flush=True)
+    keys_h = oracle.fill_zipf(13, 1, 0, n, oracle.zipf_table(n_bins), n_bins)
+    keys = torch.from_numpy(keys_h).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, level=2, threshold=2, batch=1)
+    for _ in range(burst):
+        q.submit(hist_cmd(xs, keys, n, bins, n_bins, 1))
+    q.wait()
+    pools = (c_uint64 * 4)()
+    xs.check(xs.halhip().HipQueueGetPoolStats(q.hwq, pools))
+    got = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    print("pools", list(pools), flush=True)
+    # threshold 2 in flight, plus the commands whose completion the queue has not yet seen,
+    # plus the one kept free ahead of the next launch
+    assert 1 <= pools[0] <= 8, "scratch buffers grew with the submission burst"
+    assert pools[2] <= 16, "progress maps grew with the submission burst"
+    assert pools[3] == 0
+    one = oracle.histogram(keys_h, n_bins).astype(np.uint64)
+    assert np.array_equal(got.astype(np.uint64), (one * burst) & 0xFFFFFFFF)
+
+
 @pytest.mark.parametrize("tile", [128, 256])
 def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile):
     torch = gpu

@@ -77,12 +77,16 @@ public:
     Slot AcquireSlot();
     void ReleaseSlot(const Slot &slot);
     uint64_t SlotsInUse();
-    /// Allocates the first arena now (its device must be current), so that the first
-    /// guarded command does not wait for the allocation. Does nothing later on.
+    uint64_t SlotsAllocated();
+    /// Makes sure that a slot is free, allocating an arena if none is (the queue's device
+    /// must be current). Called where waiting for an allocation harms nobody: when the queue
+    /// goes to level 2 and at every submission of a guarded command, so that AcquireSlot(),
+    /// which runs at launch time with the XQueue's locks held, finds one.
     void ReserveSlots();
 
 private:
-    void AddArenaLocked();
+    uint8_t *AllocateArena();
+    void AddArenaLocked(uint8_t *arena);
     const int device_;
     bool flag_on_host_ = false;
     uint32_t copies_ = 1;            // power of two
@@ -92,7 +96,8 @@ private:
     std::atomic<uint32_t> epoch_ { 0 };
 
     bool write_through_bar_ = false; // CPU stores straight into device memory
-    std::mutex mtx_;
+    std::mutex mtx_;                    // the preempt word (Deactivate)
+    std::mutex slots_mtx_;              // everything below; never held across an allocation
     std::vector<uint8_t *> arenas_;
     std::vector<uint8_t *> slot_ptr_;   // by slot index
     std::vector<uint32_t> slot_gen_;    // last generation handed out, by slot index
@@ -113,15 +118,24 @@ public:
     explicit ScratchPool(int device): device_(device) {}
     ~ScratchPool();
     /// A buffer of at least `bytes`, or nullptr when the device has no memory for one.
+    /// Allocates only when none is free.
     void *Acquire(size_t bytes);
     void Release(void *ptr);
     size_t Buffers();
+    size_t Bytes();
+    /// Makes sure that a buffer of `bytes` is free (the first time: one for each command that
+    /// will be in flight), so that the next Acquire(), at launch time, allocates nothing. The
+    /// pool grows to what the queue holds at once plus one, however many commands wait in
+    /// the XQueue.
+    void Reserve(size_t bytes);
 
 private:
     struct Buffer { void *ptr; size_t bytes; bool busy; };
     static constexpr int kInitialBuffers = 3;
+    bool HasFreeLocked(size_t bytes) const;
+    void *Allocate(size_t bytes);
     const int device_;
-    std::mutex mtx_;
+    std::mutex mtx_;                 // never held across an allocation
     std::vector<Buffer> buffers_;
 };
 
@@ -174,10 +188,12 @@ public:
     virtual bool ReplayOnReactivate() const override { return guard_mode_ != 0; }
     uint32_t WorkGroups() const { return n_wg_; }
 
-    /// What the first launch would otherwise take with the XQueue's locks held: the progress
-    /// map (level 2) and whatever PrepareLaunch() borrows from the queue. Either can mean a
-    /// hipMalloc, which synchronises the device; called from HipQueue::OnHwCommandSubmit(),
-    /// on the submitting thread and before any lock of the XQueue is taken.
+    /// The first launch takes a progress map (level 2) and whatever PrepareLaunch() borrows
+    /// from the queue, with the XQueue's locks held. Either can mean a hipMalloc, which
+    /// synchronises the device, when the queue's pools have nothing free: this call, from
+    /// HipQueue::OnHwCommandSubmit() on the submitting thread and before any lock of the
+    /// XQueue is taken, makes sure they have. It takes nothing itself: a command that waits
+    /// in the XQueue holds no device memory.
     void PrepareOnSubmit(HipQueue &q);
 
 protected:
@@ -185,6 +201,8 @@ protected:
     /// Called before every LaunchKernel() with the queue the command is launched on, for
     /// commands that need something of the queue (its scratch buffer).
     virtual hipError_t PrepareLaunch(HipQueue &) { return hipSuccess; }
+    /// Called at submission: reserve in the queue's pools what PrepareLaunch() will take.
+    virtual void ReserveOnSubmit(HipQueue &) {}
     /// Launch the kernel. `guarded` selects the variant with the guard compiled in.
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) = 0;
 

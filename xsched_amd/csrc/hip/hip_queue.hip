@@ -21,6 +21,31 @@ namespace xsched::hip
 namespace
 {
 
+/// Makes `device` current for the calling thread and restores what was current before.
+/// The launch thread always has it current (OnXQueueCreate); an application thread that
+/// launches directly may not.
+class DeviceScope
+{
+public:
+    explicit DeviceScope(int device)
+    {
+        int cur = device;
+        if (hipGetDevice(&cur) == hipSuccess && cur != device) {
+            previous_ = cur;
+            HIP_ASSERT(hipSetDevice(device));
+        }
+    }
+    ~DeviceScope() { if (previous_ >= 0) (void)hipSetDevice(previous_); }
+
+private:
+    int previous_ = -1;
+};
+
+} // namespace
+
+namespace
+{
+
 /// The runtime takes the completion signals of a device queue's packets from a pool (64 to
 /// begin with), and every 256 packets of a queue (a kernel launch is one packet, an event
 /// record two) one call into it takes 30-45 us longer than the others. For a queue that gets a
@@ -244,8 +269,9 @@ void GuardState::WaitFlagWritten(hipStream_t op_stream)
     if (!flag_on_host_ && !write_through_bar_) HIP_ASSERT(hipStreamSynchronize(op_stream));
 }
 
-void GuardState::AddArenaLocked()
+uint8_t *GuardState::AllocateArena()
 {
+    DeviceScope scope(device_);
     RelaxedCaptureScope relaxed;
     uint8_t *arena = nullptr;
     const size_t bytes = (size_t)kSlotsPerArena * kSlotBytes;
@@ -254,6 +280,11 @@ void GuardState::AddArenaLocked()
     // progress bytes were then wiped, and a replay applied those work-groups again).
     // Every slot is cleared in the order of its owner's stream instead, see Enqueue().
     HIP_ASSERT(hipMalloc((void **)&arena, bytes));
+    return arena;
+}
+
+void GuardState::AddArenaLocked(uint8_t *arena)
+{
     arenas_.push_back(arena);
     for (uint32_t i = 0; i < kSlotsPerArena; ++i) {
         free_slots_.push_back((uint32_t)slot_ptr_.size());
@@ -264,14 +295,26 @@ void GuardState::AddArenaLocked()
 
 void GuardState::ReserveSlots()
 {
-    std::lock_guard<std::mutex> lock(mtx_);
-    if (arenas_.empty()) AddArenaLocked();
+    {
+        std::lock_guard<std::mutex> lock(slots_mtx_);
+        if (!free_slots_.empty()) return;
+    }
+    // Outside the lock: a launch that finds a slot free does not wait for this allocation.
+    // Two threads that both find nothing free add an arena each, which is harmless.
+    uint8_t *arena = AllocateArena();
+    std::lock_guard<std::mutex> lock(slots_mtx_);
+    AddArenaLocked(arena);
 }
 
 GuardState::Slot GuardState::AcquireSlot()
 {
-    std::lock_guard<std::mutex> lock(mtx_);
-    if (free_slots_.empty()) AddArenaLocked();
+    std::unique_lock<std::mutex> lock(slots_mtx_);
+    while (free_slots_.empty()) {
+        lock.unlock();
+        uint8_t *arena = AllocateArena();
+        lock.lock();
+        AddArenaLocked(arena);
+    }
     Slot slot;
     slot.index = free_slots_.back();
     free_slots_.pop_back();
@@ -288,14 +331,20 @@ GuardState::Slot GuardState::AcquireSlot()
 
 void GuardState::ReleaseSlot(const Slot &slot)
 {
-    std::lock_guard<std::mutex> lock(mtx_);
+    std::lock_guard<std::mutex> lock(slots_mtx_);
     free_slots_.push_back(slot.index);
     in_use_--;
 }
 
+uint64_t GuardState::SlotsAllocated()
+{
+    std::lock_guard<std::mutex> lock(slots_mtx_);
+    return slot_ptr_.size();
+}
+
 uint64_t GuardState::SlotsInUse()
 {
-    std::lock_guard<std::mutex> lock(mtx_);
+    std::lock_guard<std::mutex> lock(slots_mtx_);
     return in_use_;
 }
 
@@ -384,7 +433,7 @@ hipError_t HipGuardedCommand::Enqueue(HipQueue &q, bool replay)
     g.flushed = q.Guard()->FlushedDevPtr();
 
     if (guarded && level2) {
-        if (slot_.done == nullptr) TakeSlot(q);   // normally taken at submission already
+        if (slot_.done == nullptr) TakeSlot(q);   // a free one was seen to at submission
         if (slot_.needs_clear) {
             slot_.needs_clear = false;
             // a kernel, not hipMemsetAsync: a stream under capture records no memset node
@@ -410,8 +459,8 @@ void HipGuardedCommand::TakeSlot(HipQueue &q)
 
 void HipGuardedCommand::PrepareOnSubmit(HipQueue &q)
 {
-    if (guard_mode_ != 0 && q.Level() >= kPreemptLevelDeactivate && slot_.done == nullptr) TakeSlot(q);
-    (void)PrepareLaunch(q);   // idempotent; Enqueue() calls it again and reports what it returns
+    if (guard_mode_ != 0 && q.Level() >= kPreemptLevelDeactivate && slot_.done == nullptr) q.Guard()->ReserveSlots();
+    ReserveOnSubmit(q);
 }
 
 // ---- HipQueue ----------------------------------------------------------------
@@ -440,31 +489,6 @@ HipQueue::~HipQueue()
 
 void HipQueue::OnXQueueCreate() { HIP_ASSERT(hipSetDevice(device_)); }
 
-namespace
-{
-
-/// Makes `device` current for the calling thread and restores what was current before.
-/// The launch thread always has it current (OnXQueueCreate); an application thread that
-/// launches directly may not.
-class DeviceScope
-{
-public:
-    explicit DeviceScope(int device)
-    {
-        int cur = device;
-        if (hipGetDevice(&cur) == hipSuccess && cur != device) {
-            previous_ = cur;
-            HIP_ASSERT(hipSetDevice(device));
-        }
-    }
-    ~DeviceScope() { if (previous_ >= 0) (void)hipSetDevice(previous_); }
-
-private:
-    int previous_ = -1;
-};
-
-} // namespace
-
 void HipQueue::OnPreemptLevelChange(XPreemptLevel level)
 {
     XASSERT(level <= kPreemptLevelDeactivate, "unsupported level: %d", level);
@@ -483,28 +507,57 @@ ScratchPool::~ScratchPool()
     for (auto &buf : buffers_) (void)hipFree(buf.ptr);
 }
 
-void *ScratchPool::Acquire(size_t bytes)
+void *ScratchPool::Allocate(size_t bytes)
 {
-    std::lock_guard<std::mutex> lock(mtx_);
-    Buffer *best = nullptr;
-    for (auto &buf : buffers_) {
-        if (!buf.busy && buf.bytes >= bytes && (best == nullptr || buf.bytes < best->bytes)) best = &buf;
-    }
-    if (best != nullptr) { best->busy = true; return best->ptr; }
-    // Nothing free: allocate for this command and, the first time, for the ones that will
-    // be in flight with it, so that a queue in steady state allocates nothing while its
-    // kernels run.
     DeviceScope scope(device_);
     RelaxedCaptureScope relaxed;
-    void *first = nullptr;
-    const int count = buffers_.empty() ? kInitialBuffers : 1;
-    for (int i = 0; i < count; ++i) {
-        void *ptr = nullptr;
-        if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
-        buffers_.push_back(Buffer { ptr, bytes, first == nullptr });
-        if (first == nullptr) first = ptr;
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    return ptr;
+}
+
+bool ScratchPool::HasFreeLocked(size_t bytes) const
+{
+    for (auto &buf : buffers_) {
+        if (!buf.busy && buf.bytes >= bytes) return true;
     }
-    return first;
+    return false;
+}
+
+void *ScratchPool::Acquire(size_t bytes)
+{
+    {
+        std::lock_guard<std::mutex> lock(mtx_);
+        Buffer *best = nullptr;
+        for (auto &buf : buffers_) {
+            if (!buf.busy && buf.bytes >= bytes && (best == nullptr || buf.bytes < best->bytes)) best = &buf;
+        }
+        if (best != nullptr) { best->busy = true; return best->ptr; }
+    }
+    // Nothing free (more commands in flight than Reserve() has seen submissions ahead of
+    // them, or no Reserve() at all): allocate for this command.
+    void *ptr = Allocate(bytes);
+    if (ptr == nullptr) return nullptr;
+    std::lock_guard<std::mutex> lock(mtx_);
+    buffers_.push_back(Buffer { ptr, bytes, true });
+    return ptr;
+}
+
+void ScratchPool::Reserve(size_t bytes)
+{
+    int count = 0;
+    {
+        std::lock_guard<std::mutex> lock(mtx_);
+        if (HasFreeLocked(bytes)) return;
+        // the first time: for this command and the ones that will be in flight with it
+        count = buffers_.empty() ? kInitialBuffers : 1;
+    }
+    for (int i = 0; i < count; ++i) {
+        void *ptr = Allocate(bytes);
+        if (ptr == nullptr) return;
+        std::lock_guard<std::mutex> lock(mtx_);
+        buffers_.push_back(Buffer { ptr, bytes, false });
+    }
 }
 
 void ScratchPool::Release(void *ptr)
@@ -519,6 +572,14 @@ size_t ScratchPool::Buffers()
 {
     std::lock_guard<std::mutex> lock(mtx_);
     return buffers_.size();
+}
+
+size_t ScratchPool::Bytes()
+{
+    std::lock_guard<std::mutex> lock(mtx_);
+    size_t bytes = 0;
+    for (auto &buf : buffers_) bytes += buf.bytes;
+    return bytes;
 }
 
 // On the submitting thread, before the XQueue takes any of its locks: a guarded command takes
@@ -668,5 +729,17 @@ EXPORT_C_FUNC XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out)
     out[5] = q->n_wait_blocked.load();
     out[6] = q->Guard()->SlotsInUse();
     out[7] = q->Guard()->Epoch();
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipQueueGetPoolStats(HwQueueHandle hwq, uint64_t *out)
+{
+    if (out == nullptr) return kXSchedErrorInvalidValue;
+    auto q = std::dynamic_pointer_cast<HipQueue>(HwQueueManager::Get(hwq));
+    if (q == nullptr) return kXSchedErrorNotFound;
+    out[0] = q->Scratch()->Buffers();
+    out[1] = q->Scratch()->Bytes();
+    out[2] = q->Guard()->SlotsAllocated();
+    out[3] = q->Guard()->SlotsInUse();
     return kXSchedSuccess;
 }

@@ -730,13 +730,20 @@ public:
     virtual ~HipHistogramCommand() { if (partials_ != nullptr) pool_->Release(partials_); }
 
 protected:
+    size_t ScratchBytes() const { return (size_t)n_count_wg_ * kPartialWords * sizeof(uint32_t); }
+
+    virtual void ReserveOnSubmit(HipQueue &q) override
+    {
+        if (merge_ && n_ != 0 && partials_ == nullptr) q.Scratch()->Reserve(ScratchBytes());
+    }
+
     virtual hipError_t PrepareLaunch(HipQueue &q) override
     {
         // A replay must find the partials of the flushed launch: the buffer taken at the
         // first launch is kept until the command is destroyed.
         if (!merge_ || n_ == 0 || partials_ != nullptr) return hipSuccess;
         pool_ = q.Scratch();
-        partials_ = (uint32_t *)pool_->Acquire((size_t)n_count_wg_ * kPartialWords * sizeof(uint32_t));
+        partials_ = (uint32_t *)pool_->Acquire(ScratchBytes());
         // No scratch: the one-kernel layout works on the same chunks (decided before the
         // first launch, so every replay takes the same path).
         if (partials_ == nullptr) merge_ = false;
