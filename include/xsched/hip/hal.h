@@ -37,6 +37,17 @@ XResult HipQueueCreate(HwQueueHandle *hwq, void *stream);
  * block in the driver, [6] progress-map slots in use, [7] current preempt epoch. */
 XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
 
+/* How the queue's kernel commands carry their completion markers. on != 0 (the default,
+ * XSCHED_HIP_MARKER_ON_KERNEL=OFF changes it): as the stop event of the kernel's own launch,
+ * which saves the device a packet per marked command (1-3 us) and a waiting caller 2 us.
+ * The HIP runtime then learns of the kernel's completion some 20 us after XQueueWait /
+ * XQueueWaitAll have returned: hipStreamQuery() on the raw stream says "not ready" and
+ * hipStreamSynchronize() blocks for that long. on == 0: every marker is a hipEventRecord()
+ * behind its command, and the stream is idle for the runtime as soon as the XQueue is.
+ * For programs that wait on the raw stream themselves (the interception shim does this for
+ * its queues). Takes effect for commands launched afterwards. */
+XResult HipQueueSetMarkerOnKernel(HwQueueHandle hwq, int on);
+
 /* Device memory the queue's pools hold for guarded commands, for tests. `out` receives 4
  * values: [0] scratch buffers allocated (the partial histograms of histogram commands),
  * [1] their bytes, [2] progress-map slots allocated, [3] progress-map slots in use. Both

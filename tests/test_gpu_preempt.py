@@ -119,6 +119,56 @@ def test_histogram_preempt_resume_bit_exact(xs, gpu, monkeypatch, layout):
     assert int(got.sum()) % (1 << 32) == (times * n) % (1 << 32)
 
 
+@pytest.mark.parametrize("on_kernel", [1, 0])
+def test_marker_on_the_kernel_or_recorded_behind_it(xs, gpu, on_kernel):
+    """A queue's kernel commands carry their markers as the stop event of their own launch
+    (the default) or as events recorded behind them (HipQueueSetMarkerOnKernel(hwq, 0)). Either
+    way every command is waited for and the results are the oracle's, also across suspensions
+    that flush and replay; with recorded markers the runtime sees the stream idle the moment
+    the XQueue is."""
+    torch = gpu
+    n, times = (1 << 22) + 3, 60
+    print(f"case marker-mode on_kernel={on_kernel} n={n} times={times}", flush=True)
+    x_h = oracle.fill_uniform(6, 1, 0, n)
+    y_h = oracle.fill_uniform(6, 2, 0, n)
+    x = torch.from_numpy(x_h).cuda()
+    y = torch.from_numpy(y_h.copy()).cuda()
+    n_bins, nk = 4096, 1 << 20
+    keys_h = oracle.fill_zipf(6, 3, 0, nk, oracle.zipf_table(n_bins), n_bins)
+    keys = torch.from_numpy(keys_h).cuda()
+    bins = torch.zeros(n_bins, dtype=torch.int32, device="cuda")
+    q = Queue(xs, torch, level=2, threshold=2, batch=1)   # every command carries a marker
+    xs.check(xs.halhip().HipQueueSetMarkerOnKernel(q.hwq, on_kernel))
+    idle_at_once = 0
+    for i in range(times):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+        q.submit(hist_cmd(xs, keys, nk, bins, n_bins, 1))
+        if i % 10 == 9:
+            q.wait()
+            idle_at_once += 1 if q.stream.query() else 0
+    stop = threading.Event()
+    t = threading.Thread(target=churn, args=(xs, q, stop, 3))
+    t.start()
+    for i in range(times):
+        q.submit(axpy_cmd(xs, 0.5, x, y, n, 1))
+        q.submit(hist_cmd(xs, keys, nk, bins, n_bins, 1))
+    time.sleep(0.02)
+    stop.set()
+    t.join()
+    q.wait()
+    st = hip_stats(xs, q.hwq)
+    got_y = y.cpu().numpy()
+    got_bins = bins.cpu().numpy().view(np.uint32)
+    q.close()
+    print("stats", st, "stream idle at once", idle_at_once, "of", times // 10, flush=True)
+    want = oracle.axpy(0.5, x_h, y_h, 2 * times)
+    assert np.array_equal(got_y.view(np.uint32), want.view(np.uint32))
+    one = oracle.histogram(keys_h, n_bins).astype(np.uint64)
+    assert np.array_equal(got_bins.astype(np.uint64), (one * 2 * times) & 0xFFFFFFFF)
+    if not on_kernel:
+        assert idle_at_once == times // 10
+
+
 def test_commands_waiting_in_the_xqueue_hold_no_device_memory(xs, gpu):
     """A burst of guarded histogram commands far deeper than the in-flight window: the
     queue's pools (partial-histogram buffers, progress maps) grow with what is launched and

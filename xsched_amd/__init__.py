@@ -118,6 +118,7 @@ HALHIP_API = {
     "HipQueueCreate": (XResult, [POINTER(c_uint64), c_void_p]),
     "HipQueueGetStats": (XResult, [c_uint64, POINTER(c_uint64)]),
     "HipQueueGetPoolStats": (XResult, [c_uint64, POINTER(c_uint64)]),
+    "HipQueueSetMarkerOnKernel": (XResult, [c_uint64, c_int]),
     "HipQueueMarkEpochFlushed": (XResult, [c_uint64]),
     "HipAxpyCommandCreate": (XResult, [POINTER(c_uint64), c_float, c_void_p, c_void_p, c_size_t, c_int]),
     "HipGemmBf16CommandCreate": (XResult, [POINTER(c_uint64), c_void_p, c_void_p, c_void_p,

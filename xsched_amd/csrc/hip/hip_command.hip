@@ -126,9 +126,15 @@ public:
             off += ROUND_UP(sizes[i], 16);
         }
     }
+    virtual bool MarkerGoesWithKernel() const override { return true; }
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool) override
-    { return hipLaunchKernel(func_, grid_, block_, arg_ptrs_.data(), shmem_, q.Stream()); }
+    {
+        if (const hipEvent_t stop = TakeStopEvent()) {
+            return hipExtLaunchKernel(func_, grid_, block_, arg_ptrs_.data(), shmem_, q.Stream(), nullptr, stop, 0);
+        }
+        return hipLaunchKernel(func_, grid_, block_, arg_ptrs_.data(), shmem_, q.Stream());
+    }
 private:
     const void *func_; dim3 grid_, block_; uint32_t shmem_;
     std::vector<char> storage_;
@@ -147,12 +153,21 @@ public:
                            const void *packed, size_t bytes)
         : func_(func), grid_(grid), block_(block), shmem_(shmem)
         , storage_((const char *)packed, (const char *)packed + bytes) {}
+    virtual bool MarkerGoesWithKernel() const override { return true; }
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool) override
     {
         size_t bytes = storage_.size();
         void *extra[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, storage_.data(),
                           HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END };
+        // The launch that takes a stop event counts work-items, in 32 bits per dimension.
+        const uint64_t items[3] = { (uint64_t)grid_.x * block_.x, (uint64_t)grid_.y * block_.y, (uint64_t)grid_.z * block_.z };
+        const bool fits = items[0] <= UINT32_MAX && items[1] <= UINT32_MAX && items[2] <= UINT32_MAX;
+        if (const hipEvent_t stop = fits ? TakeStopEvent() : nullptr) {
+            return hipExtModuleLaunchKernel(func_, (uint32_t)items[0], (uint32_t)items[1], (uint32_t)items[2],
+                                            block_.x, block_.y, block_.z, shmem_, q.Stream(), nullptr, extra,
+                                            nullptr, stop, 0);
+        }
         return hipModuleLaunchKernel(func_, grid_.x, grid_.y, grid_.z, block_.x, block_.y, block_.z,
                                      shmem_, q.Stream(), nullptr, extra);
     }
@@ -192,6 +207,9 @@ protected:
     {
         guard_args_ = g;
         arg_ptrs_.back() = &guard_args_;
+        if (const hipEvent_t stop = TakeStopEvent()) {
+            return hipExtLaunchKernel(func_, dim3(n_wg_), block_, arg_ptrs_.data(), shmem_, stream, nullptr, stop, 0);
+        }
         return hipLaunchKernel(func_, dim3(n_wg_), block_, arg_ptrs_.data(), shmem_, stream);
     }
 private:

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include "shim_hooks.h"
 #include "xsched/hip/guard.h"
@@ -33,15 +34,22 @@ namespace xsched::hip
 /// Process-wide pool of timing-less events used as completion markers. Grows by
 /// small chunks on demand (the reference creates 513 at the first use:
 /// event_pool.h:26-32, utils/pool.h:15-24).
+/// Events for markers, in two lists. An event that has gone through hipEventRecord() keeps
+/// the stream of that record with the runtime: asking it while THAT stream captures a graph
+/// fails (hipErrorCapturedEvent), whatever the event has been used for since. Handing an
+/// event to a kernel launch as its stop event leaves no such trace and clears none, so the
+/// markers that ride on kernels are events that were never recorded, and stay apart.
 class EventPool
 {
 public:
     static EventPool &Instance();
-    hipEvent_t Pop();
-    void Push(hipEvent_t ev);
+    /// never_recorded: an event that no hipEventRecord() has seen (for a stop event).
+    hipEvent_t Pop(bool never_recorded = false);
+    void Push(hipEvent_t ev, bool recorded = true);
 private:
     std::mutex mtx_;
-    std::vector<hipEvent_t> free_;
+    std::vector<hipEvent_t> fresh_;     // never recorded
+    std::vector<hipEvent_t> recorded_;
 };
 
 /// Level-2 state of one queue: the preempt word and the progress-map slots.
@@ -149,8 +157,10 @@ public:
     virtual ~HipCommand();
 
     virtual void Synchronize() override;
-    virtual bool Synchronizable() override { return marker_ != nullptr; }
-    virtual bool EnableSynchronization() override;
+    virtual bool Synchronizable() override { return wants_marker_; }
+    /// The event itself is taken at launch, when the queue (and with it the kind of marker)
+    /// is known.
+    virtual bool EnableSynchronization() override { wants_marker_ = true; return true; }
 
     /// Enqueue on the queue's stream and (re-)record the marker behind it.
     /// `replay` is true when called from Reactivate().
@@ -160,6 +170,10 @@ public:
     virtual bool ReplayOnReactivate() const { return false; }
 
 
+    /// Whether Enqueue() ends with a kernel launch that takes the marker (TakeStopEvent());
+    /// decides which kind of event the command gets as its marker.
+    virtual bool MarkerGoesWithKernel() const { return false; }
+
     /// Every command of this adapter except the host-side event wait only enqueues on
     /// the stream, so it may be launched on the submitting thread.
     virtual bool DirectLaunchable() override { return true; }
@@ -167,13 +181,33 @@ public:
 
 protected:
     virtual hipError_t Enqueue(HipQueue &q, bool replay) = 0;
+    /// For an Enqueue() that ends with a kernel launch: the marker, to be handed to that LAST
+    /// launch as its stop event (hipExtLaunchKernel and its relatives). The runtime then puts
+    /// the event's completion signal on the kernel's own dispatch packet, and LaunchWrapper()
+    /// records no marker behind the command. A recorded marker is a packet of its own that
+    /// the next dispatch has to wait for: 1-3 us of device time per marked command, 2 us of a
+    /// waiting caller's latency. nullptr when the command carries no marker or its queue
+    /// records markers (HipQueue::MarkerOnKernel()): then launch the ordinary way. Whoever
+    /// receives an event here must launch with it.
+    hipEvent_t TakeStopEvent();
     /// Polls the event for the marker polling budget (no system call), then blocks in the driver.
     void WaitForEvent(hipEvent_t event);
     hipEvent_t marker_ = nullptr;
 
 private:
     HipQueue *queue_ = nullptr; // for wait statistics; set at launch
+    bool wants_marker_ = false;     // EnableSynchronization() was called
+    bool marker_on_kernel_ = false; // this launch: the marker went out with a kernel
+    bool marker_recorded_ = false;  // the marker has been through hipEventRecord()
 };
+
+/// hipLaunchKernelGGL, with `stop` (may be null) bound to the dispatch as its stop event.
+template <typename... Args, typename F = void (*)(Args...)>
+inline void LaunchWithStop(hipEvent_t stop, F kernel, const dim3 &grid, const dim3 &block, hipStream_t stream, Args... args)
+{
+    if (stop != nullptr) hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, nullptr, stop, 0, args...);
+    else hipLaunchKernelGGL(kernel, grid, block, 0, stream, args...);
+}
 
 /// Base of the guarded victim kernels.
 class HipGuardedCommand : public HipCommand
@@ -186,6 +220,7 @@ public:
     virtual ~HipGuardedCommand();
 
     virtual bool ReplayOnReactivate() const override { return guard_mode_ != 0; }
+    virtual bool MarkerGoesWithKernel() const override { return true; }
     uint32_t WorkGroups() const { return n_wg_; }
 
     /// The first launch takes a progress map (level 2) and whatever PrepareLaunch() borrows
@@ -240,6 +275,15 @@ public:
 
     hipStream_t Stream() const { return stream_; }
     XPreemptLevel Level() const { return level_.load(std::memory_order_acquire); }
+    /// Whether the markers of kernel commands go out as the stop event of the kernel itself
+    /// (see HipCommand::TakeStopEvent()) instead of being recorded behind it. The price: the
+    /// runtime learns of such a kernel's completion from its own handler thread, some 20 us
+    /// after the event shows it, and until then hipStreamQuery() on the stream says "not
+    /// ready" and hipStreamSynchronize() blocks. Queues whose users wait through the XQueue
+    /// want it on (the default, XSCHED_HIP_MARKER_ON_KERNEL); the interception shim, whose
+    /// applications ask the stream, turns it off for its queues.
+    bool MarkerOnKernel() const { return marker_on_kernel_.load(std::memory_order_relaxed); }
+    void SetMarkerOnKernel(bool on) { marker_on_kernel_.store(on, std::memory_order_relaxed); }
     const std::shared_ptr<GuardState> &Guard() const { return guard_; }
     const std::shared_ptr<ScratchPool> &Scratch() const { return scratch_; }
 
@@ -252,6 +296,7 @@ private:
     int device_ = 0;
     XDevice xdevice_ = 0;
     std::atomic<XPreemptLevel> level_ { kPreemptLevelUnknown };
+    std::atomic<bool> marker_on_kernel_ { true };
     std::shared_ptr<GuardState> guard_;
     hipStream_t op_stream_ = nullptr; // flag writes when the word lives in device memory
     std::shared_ptr<ScratchPool> scratch_;

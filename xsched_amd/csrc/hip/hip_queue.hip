@@ -120,25 +120,26 @@ EventPool &EventPool::Instance()
     return *pool;
 }
 
-hipEvent_t EventPool::Pop()
+hipEvent_t EventPool::Pop(bool never_recorded)
 {
     std::lock_guard<std::mutex> lock(mtx_);
-    if (free_.empty()) {
+    std::vector<hipEvent_t> &from = (never_recorded || recorded_.empty()) ? fresh_ : recorded_;
+    if (from.empty()) {
         for (int i = 0; i < 16; ++i) {
             hipEvent_t ev = nullptr;
             HIP_ASSERT(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-            free_.push_back(ev);
+            fresh_.push_back(ev);
         }
     }
-    hipEvent_t ev = free_.back();
-    free_.pop_back();
+    hipEvent_t ev = from.back();
+    from.pop_back();
     return ev;
 }
 
-void EventPool::Push(hipEvent_t ev)
+void EventPool::Push(hipEvent_t ev, bool recorded)
 {
     std::lock_guard<std::mutex> lock(mtx_);
-    free_.push_back(ev);
+    (recorded ? recorded_ : fresh_).push_back(ev);
 }
 
 // ---- GuardState --------------------------------------------------------------
@@ -352,24 +353,45 @@ uint64_t GuardState::SlotsInUse()
 
 HipCommand::~HipCommand()
 {
-    if (marker_ != nullptr) EventPool::Instance().Push(marker_);
-}
-
-bool HipCommand::EnableSynchronization()
-{
-    if (marker_ == nullptr) marker_ = EventPool::Instance().Pop();
-    return marker_ != nullptr;
+    if (marker_ != nullptr) EventPool::Instance().Push(marker_, marker_recorded_);
 }
 
 hipError_t HipCommand::LaunchWrapper(HipQueue &q, bool replay)
 {
     queue_ = &q;
-    hipError_t err = Enqueue(q, replay);
+    if (wants_marker_ && marker_ == nullptr) {
+        const bool for_a_kernel = MarkerGoesWithKernel() && q.MarkerOnKernel();
+        marker_ = EventPool::Instance().Pop(for_a_kernel);
+        marker_recorded_ = !for_a_kernel;
+    }
+    marker_on_kernel_ = false;
+    hipError_t err;
+    if (marker_ != nullptr && !marker_recorded_) {
+        // A launch that takes an event is one of the calls that the runtime refuses, and
+        // answers by invalidating the capture, while ANOTHER stream of the process captures a
+        // graph in the default (global) mode; like the adapter's waits it concerns this
+        // queue's stream only.
+        RelaxedCaptureScope relaxed;
+        err = Enqueue(q, replay);
+    } else {
+        err = Enqueue(q, replay);
+    }
     if (UNLIKELY(err != hipSuccess)) return err;
     // Recording again after a replay moves the marker behind the replayed work,
-    // which is what a later Synchronize() has to wait for.
-    if (marker_ != nullptr) err = hipEventRecord(marker_, q.Stream());
+    // which is what a later Synchronize() has to wait for (a replayed kernel that carries
+    // the marker itself does the same).
+    if (marker_ != nullptr && !marker_on_kernel_) {
+        marker_recorded_ = true;
+        err = hipEventRecord(marker_, q.Stream());
+    }
     return err;
+}
+
+hipEvent_t HipCommand::TakeStopEvent()
+{
+    if (marker_ == nullptr || marker_recorded_) return nullptr;
+    marker_on_kernel_ = true;
+    return marker_;
 }
 
 bool HipCommand::CompletedWithoutWaiting()
@@ -473,6 +495,7 @@ HipQueue::HipQueue(hipStream_t stream): stream_(stream)
     xdevice_ = MakeDevice(kDeviceTypeGPU, MakePciId(prop.pciDomainID, prop.pciBusID, prop.pciDeviceID, 0));
     guard_ = std::make_shared<GuardState>(device_);
     scratch_ = std::make_shared<ScratchPool>(device_);
+    marker_on_kernel_.store(GetEnvOption("XSCHED_HIP_MARKER_ON_KERNEL", true));
     HIP_ASSERT(hipStreamCreateWithFlags(&op_stream_, hipStreamNonBlocking)); // default priority
     // The entry point that allocates nothing needs the address of its static array on this
     // device; looked up here, at set-up, it never has to be looked up under a graph capture.
@@ -639,7 +662,7 @@ void HipQueue::Synchronize()
         return;
     }
     RelaxedCaptureScope relaxed;
-    hipEvent_t marker = EventPool::Instance().Pop();
+    hipEvent_t marker = EventPool::Instance().Pop(false);
     hipError_t err = hipEventRecord(marker, stream_);
     XASSERT(err == hipSuccess, "hipEventRecord failed: %d (%s)", (int)err, hipGetErrorString(err));
     if (!PollEvent(marker, SyncSpinMicros())) HIP_ASSERT(hipEventSynchronize(marker));
@@ -729,6 +752,14 @@ EXPORT_C_FUNC XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out)
     out[5] = q->n_wait_blocked.load();
     out[6] = q->Guard()->SlotsInUse();
     out[7] = q->Guard()->Epoch();
+    return kXSchedSuccess;
+}
+
+EXPORT_C_FUNC XResult HipQueueSetMarkerOnKernel(HwQueueHandle hwq, int on)
+{
+    auto q = std::dynamic_pointer_cast<HipQueue>(HwQueueManager::Get(hwq));
+    if (q == nullptr) return kXSchedErrorNotFound;
+    q->SetMarkerOnKernel(on != 0);
     return kXSchedSuccess;
 }
 

@@ -241,17 +241,18 @@ protected:
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
     {
         if (n_ == 0) return hipSuccess;
+        const hipEvent_t stop = TakeStopEvent();
         const bool aligned = (((uintptr_t)x_ | (uintptr_t)y_) & 15) == 0;
         const dim3 grid(n_wg_), block(kLanes);
         const uint32_t waves = PersistentWaves();
         if (aligned && guarded && !chunk_grid_) {
             const dim3 pgrid(n_wg_ < waves ? n_wg_ : waves);
-            hipLaunchKernelGGL((AxpyPersistentKernel<3, true>), pgrid, block, 0, stream, alpha_, (const float4 *)x_,
+            LaunchWithStop(stop, (AxpyPersistentKernel<3, true>), pgrid, block, stream, alpha_, (const float4 *)x_,
                                (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
         } else if (aligned && !guarded && !chunk_grid_ && n_wg_ >= 16 * waves) {
             // A long array: the same few long-lived waves stream it as fast as one wave per
             // chunk does and leave nearly all wave slots to whatever else runs on the device.
-            hipLaunchKernelGGL((AxpyPersistentKernel<3, false>), dim3(waves), block, 0, stream, alpha_, (const float4 *)x_,
+            LaunchWithStop(stop, (AxpyPersistentKernel<3, false>), dim3(waves), block, stream, alpha_, (const float4 *)x_,
                                (float4 *)y_, (uint64_t)(n_ / 4), (uint32_t)(n_ % 4), steps_, n_wg_, g);
         } else if (aligned) {
             const uint64_t n4 = n_ / 4;
@@ -262,16 +263,16 @@ protected:
             const uint32_t steps = wide ? steps_ / 2 : steps_;
             const float4 *xv = (const float4 *)x_;
             float4 *yv = (float4 *)y_;
-            if (guarded && wide)       hipLaunchKernelGGL((AxpyVec4Kernel<true, 8>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else if (guarded)          hipLaunchKernelGGL((AxpyVec4Kernel<true, 4>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else if (wide)             hipLaunchKernelGGL((AxpyVec4Kernel<false, 8>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
-            else                       hipLaunchKernelGGL((AxpyVec4Kernel<false, 4>), grid, block, 0, stream, alpha_, xv, yv, n4, tail, steps, g);
+            if (guarded && wide)       LaunchWithStop(stop, (AxpyVec4Kernel<true, 8>), grid, block, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (guarded)          LaunchWithStop(stop, (AxpyVec4Kernel<true, 4>), grid, block, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else if (wide)             LaunchWithStop(stop, (AxpyVec4Kernel<false, 8>), grid, block, stream, alpha_, xv, yv, n4, tail, steps, g);
+            else                       LaunchWithStop(stop, (AxpyVec4Kernel<false, 4>), grid, block, stream, alpha_, xv, yv, n4, tail, steps, g);
         } else {
             if (guarded) {
-                hipLaunchKernelGGL(AxpyScalarKernel<true>, grid, block, 0, stream, alpha_, x_, y_,
+                LaunchWithStop(stop, AxpyScalarKernel<true>, grid, block, stream, alpha_, x_, y_,
                                    (uint64_t)n_, steps_, g);
             } else {
-                hipLaunchKernelGGL(AxpyScalarKernel<false>, grid, block, 0, stream, alpha_, x_, y_,
+                LaunchWithStop(stop, AxpyScalarKernel<false>, grid, block, stream, alpha_, x_, y_,
                                    (uint64_t)n_, steps_, g);
             }
         }

@@ -416,14 +416,15 @@ protected:
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
     {
         const dim3 grid(n_wg_);
+        const hipEvent_t stop = TakeStopEvent();
         if (tile_ == kLargeTile) {
             const dim3 block(512);
-            if (guarded) hipLaunchKernelGGL((GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
-            else         hipLaunchKernelGGL((GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+            if (guarded) LaunchWithStop(stop, (GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
+            else         LaunchWithStop(stop, (GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
         } else {
             const dim3 block(256);
-            if (guarded) hipLaunchKernelGGL((GemmBf16Kernel<true, kSmallTile, 2, 2>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
-            else         hipLaunchKernelGGL((GemmBf16Kernel<false, kSmallTile, 2, 2>), grid, block, 0, stream, A_, B_, C_, M_, N_, K_, g);
+            if (guarded) LaunchWithStop(stop, (GemmBf16Kernel<true, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
+            else         LaunchWithStop(stop, (GemmBf16Kernel<false, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
         }
         return hipGetLastError();
     }

@@ -640,7 +640,7 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
         first[i] = load_words(row + i * kRows);
         first_outside[i] = load_outside(row + i * kRows);
     }
-    if (tid == 0) outside_total = 0;
+    if (tid == 0) { outside_total = 0; guard_word = 1; }
 
     if (kGuard) {
         // A flushed counting launch leaves partials missing: every counting group must have
@@ -651,20 +651,24 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
             const uint32_t p = tid + i * kThreads;
             tag[i] = g.done != nullptr && p < n_part ? __builtin_nontemporal_load(&g.done[p]) : (uint8_t)g.gen;
         }
+        // guard_word = 1 is in place before any wave takes it back: the loads above take a
+        // memory round trip, this barrier none. (A vote of the whole group instead of the
+        // plain stores below costs two barriers and a reduction through the LDS.)
+        __syncthreads();
         // This kernel does not look at the preempt word itself: it runs for a few
         // microseconds, and what it must not do is run after a counting launch that was
         // flushed. Every flushed group has left its epoch in the `flushed` word, and the tags
         // say whether every partial is there; its own tag says whether it ran before the flush.
+        bool stop = false;
         if (tid == 0) {
-            bool go = !xguard_epoch_flushed(g);
-            if (go && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) go = false;
-            guard_word = go ? 1u : 0u;
+            stop = xguard_epoch_flushed(g);
+            if (!stop && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) stop = true;
         }
-        int all = 1;
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) all &= tag[i] == (uint8_t)g.gen;
-        const int complete = __syncthreads_and(all);   // also publishes guard_word (and outside_total = 0)
-        if (!complete || guard_word == 0) return;
+        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) stop |= tag[i] != (uint8_t)g.gen;
+        if (stop) guard_word = 0;   // any number of threads, the same value
+        __syncthreads();
+        if (guard_word == 0) return;
     } else {
         __syncthreads();
     }
@@ -755,17 +759,20 @@ protected:
         if (n_ == 0) return hipSuccess;
         const dim3 grid(n_count_wg_), block(kThreads);
         if (!merge_) {
-            if (guarded) hipLaunchKernelGGL((HistogramKernel<true, false>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
-            else         hipLaunchKernelGGL((HistogramKernel<false, false>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
+            const hipEvent_t stop = TakeStopEvent();
+            if (guarded) LaunchWithStop(stop, (HistogramKernel<true, false>), grid, block, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
+            else         LaunchWithStop(stop, (HistogramKernel<false, false>), grid, block, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, (uint32_t *)nullptr, g);
             return hipGetLastError();
         }
-        if (guarded) hipLaunchKernelGGL((HistogramKernel<true, true>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
-        else         hipLaunchKernelGGL((HistogramKernel<false, true>), grid, block, 0, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
+        hipEvent_t stop = nullptr;    // the merge kernel is the command's last
+        if (guarded) LaunchWithStop(stop, (HistogramKernel<true, true>), grid, block, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
+        else         LaunchWithStop(stop, (HistogramKernel<false, true>), grid, block, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) return err;
         const dim3 merge_grid(kMergeGroups);
-        if (guarded) hipLaunchKernelGGL(HistogramMergeKernel<true>, merge_grid, block, 0, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
-        else         hipLaunchKernelGGL(HistogramMergeKernel<false>, merge_grid, block, 0, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
+        stop = TakeStopEvent();
+        if (guarded) LaunchWithStop(stop, HistogramMergeKernel<true>, merge_grid, block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
+        else         LaunchWithStop(stop, HistogramMergeKernel<false>, merge_grid, block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
         return hipGetLastError();
     }
 

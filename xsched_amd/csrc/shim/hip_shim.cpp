@@ -446,7 +446,14 @@ void OnStreamCreated(hipStream_t stream, unsigned flags)
         std::unique_lock<std::shared_mutex> lock(S().stream_mtx);
         S().stream_flags[stream] = flags;
     }
-    (void)XQueueManager::AutoCreate([&](HwQueueHandle *hwq) { return HipQueueCreate(hwq, stream); });
+    (void)XQueueManager::AutoCreate([&](HwQueueHandle *hwq) {
+        const XResult res = HipQueueCreate(hwq, stream);
+        // The application waits on the stream itself (hipStreamSynchronize, hipStreamQuery):
+        // the runtime has to see the stream idle as soon as the XQueue does, which it does
+        // not for markers that ride on kernels.
+        if (res == kXSchedSuccess) (void)HipQueueSetMarkerOnKernel(*hwq, 0);
+        return res;
+    });
 }
 
 hipError_t RecordEvent(hipEvent_t event, hipStream_t stream, bool with_flags, unsigned flags)
