@@ -81,11 +81,14 @@ XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, v
                              size_t n, int guard);
 
 /* C[M,N] = A[M,K] * B[K,N]; A, B, C row-major bf16, fp32 accumulation in ascending
- * k, round-to-nearest-even on store. M, N multiples of 128 and K a multiple of 64; other
- * shapes are refused (InvalidValue). The MFMA kernel works on 256x256 tiles of C, or on
- * 128x128 tiles when M or N is no multiple of 256 or the large tiles would cover at most half
- * of the compute units (XSCHED_HIP_GEMM_TILE=128|256 overrides that); every element is
- * summed in the same order either way. */
+ * k, round-to-nearest-even on store. Any M, N, K >= 1 (at most 2^18 tiles). The fast MFMA
+ * kernel takes M, N in multiples of 128, K in multiples of 64 (K, N <= 2^22) and matrices
+ * aligned to 16 bytes: it works on 256x256 tiles of C, or on 128x128 tiles when M or N is no
+ * multiple of 256 or the large tiles would cover at most half of the compute units
+ * (XSCHED_HIP_GEMM_TILE=128|256 overrides that). Every other shape or alignment runs on a
+ * bounds-checked kernel with 64x64 tiles (XSCHED_HIP_GEMM_TILE=64 forces it): correct and
+ * guarded like the others, several times slower. Every element is summed in the same order
+ * in all three. */
 XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void *A, const void *B, void *C,
                                  int M, int N, int K, int guard);
 

@@ -373,6 +373,62 @@ def test_gemm_shapes_that_only_small_tiles_fit(xs, gpu, M, N, K, level, guard):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (127, 129, 65), (130, 70, 33),
+                                   (256, 128, 100), (200, 256, 64), (128, 128, 8), (1, 300, 129), (300, 1, 250)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_gemm_any_shape(xs, gpu, M, N, K, level, guard):
+    """Shapes the fast kernels do not take (M or N no multiple of 128, K no multiple of 64) go
+    to the any-shape kernel: integers as above, so the result is determined; the matrices lie
+    in larger buffers whose other elements must come back untouched."""
+    torch = gpu
+    print(f"case gemm-any M={M} N={N} K={K} level={level} guard={guard}", flush=True)
+    rng = np.random.default_rng(9)
+    a_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b_i = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    a_bits, b_bits = oracle.f32_to_bf16_bits(a_i), oracle.f32_to_bf16_bits(b_i)
+    want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K)
+    pad = 3   # elements in front: the matrices start at odd multiples of two bytes
+    a = torch.from_numpy(np.concatenate([np.full(pad, 0x7FC0, np.uint16), a_bits.ravel(), np.full(64, 0x7FC0, np.uint16)]).view(np.int16)).cuda()
+    b = torch.from_numpy(np.concatenate([np.full(pad, 0x7FC0, np.uint16), b_bits.ravel(), np.full(64, 0x7FC0, np.uint16)]).view(np.int16)).cuda()
+    c = torch.full((pad + M * N + 64,), 0x1234, dtype=torch.int16, device="cuda")
+    cmd = c_uint64()
+    xs.check(xs.halhip().HipGemmBf16CommandCreate(byref(cmd), a.data_ptr() + 2 * pad, b.data_ptr() + 2 * pad,
+                                                  c.data_ptr() + 2 * pad, M, N, K, guard))
+    q = Queue(xs, torch, level)
+    q.submit(cmd.value)
+    q.wait()
+    got = c.cpu().numpy().view(np.uint16)
+    q.close()
+    assert np.array_equal(got[pad:pad + M * N].reshape(M, N), want.reshape(M, N))
+    assert np.all(got[:pad] == 0x1234) and np.all(got[pad + M * N:] == 0x1234)
+
+
+def test_gemm_any_shape_kernel_sums_as_the_fast_kernels_do(xs, gpu, monkeypatch):
+    """Seeded normal inputs on a shape every kernel takes: the any-shape kernel (forced)
+    feeds the matrix cores the same slices of 16 along K in the same order, so the bits agree."""
+    M, N, K = 256, 384, 512
+    print(f"case gemm-any-vs-fast M={M} N={N} K={K}", flush=True)
+    a_bits = oracle.fill_normal_bf16(19, 1, 0, M * K)
+    b_bits = oracle.fill_normal_bf16(19, 2, 0, K * N)
+    out = {}
+    for tile in (64, 128):
+        monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
+        out[tile] = _gemm_case(xs, gpu, a_bits, b_bits, M, N, K, 2, 1)
+    assert np.array_equal(out[64], out[128])
+
+
+def test_gemm_refuses_what_no_kernel_takes(xs, gpu):
+    torch = gpu
+    t = torch.zeros(64, dtype=torch.int16, device="cuda")
+    cmd = c_uint64()
+    h = xs.halhip()
+    for M, N, K in ((0, 8, 8), (8, 0, 8), (8, 8, 0), (-1, 8, 8)):
+        assert h.HipGemmBf16CommandCreate(byref(cmd), t.data_ptr(), t.data_ptr(), t.data_ptr(), M, N, K, 1) == xs.kXSchedErrorInvalidValue
+    assert h.HipGemmBf16CommandCreate(byref(cmd), t.data_ptr() + 1, t.data_ptr(), t.data_ptr(), 4, 4, 4, 1) == xs.kXSchedErrorInvalidValue
+    # more tiles than a progress map has bytes
+    assert h.HipGemmBf16CommandCreate(byref(cmd), t.data_ptr(), t.data_ptr(), t.data_ptr(), 64 * 1024, 64 * 1024 + 1, 1, 1) == xs.kXSchedErrorInvalidValue
+
+
 def test_gemm_seeded_random_shapes(xs, gpu, monkeypatch):
     """Ten seeded shapes (M, N multiples of 128 up to 1152, K multiples of 64 up to 448), each
     with the tile sizes its shape allows; integer inputs, so every result is determined."""

@@ -197,13 +197,14 @@ def test_commands_waiting_in_the_xqueue_hold_no_device_memory(xs, gpu):
     assert np.array_equal(got.astype(np.uint64), (one * burst) & 0xFFFFFFFF)
 
 
-@pytest.mark.parametrize("tile", [128, 256])
-def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile):
+@pytest.mark.parametrize("tile,shape", [(128, (2048, 2048, 2048)), (256, (2048, 2048, 2048)), (64, (1000, 1999, 1030))])
+def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile, shape):
+    """Both tile sizes of the fast kernel, and the any-shape kernel on a shape only it takes."""
     torch = gpu
     monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
-    M = N = K = 2048
+    M, N, K = shape
     times = 12
-    print(f"case gemm-preempt {M}^3 times={times} x 10", flush=True)
+    print(f"case gemm-preempt {M}x{N}x{K} tile={tile} times={times} x 10", flush=True)
     a_bits = oracle.fill_normal_bf16(13, 1, 0, M * K)
     b_bits = oracle.fill_normal_bf16(13, 2, 0, K * N)
     a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
@@ -290,7 +291,8 @@ def test_null_stream_and_bad_arguments(xs, gpu):
     assert h.HipQueueCreate(byref(hwq), None) == xs.kXSchedErrorNotSupported
     assert h.HipQueueCreate(None, 1) == xs.kXSchedErrorInvalidValue
     cmd = c_uint64()
-    assert h.HipGemmBf16CommandCreate(byref(cmd), 16, 16, 16, 100, 256, 64, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipGemmBf16CommandCreate(byref(cmd), 16, 16, 16, 100, 0, 64, 0) == xs.kXSchedErrorInvalidValue
+    assert h.HipGemmBf16CommandCreate(byref(cmd), 17, 16, 16, 100, 256, 64, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipHistogramCommandCreate(byref(cmd), 16, 4, 16, 70000, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, None, None, 4, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, 16, 16, 4, 4) == xs.kXSchedErrorInvalidValue

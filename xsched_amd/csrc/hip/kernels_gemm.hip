@@ -405,11 +405,79 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
 }
 
 
+// Any shape: M, N, K >= 1, any alignment of the three matrices to two bytes. 64 x 64 tiles of
+// C, four waves of one 32x32 block each, K in slices of 16 through the same MFMA as above and
+// in the same order (so an element is summed as the kernels above sum it; what lies beyond
+// K is zero). Every load and store is checked against the matrix: this kernel is the fall-back
+// for the shapes the fast kernels do not take, not a fast kernel. The guard is at entry only:
+// a tile is short.
+constexpr int kAnyTile = 64;
+constexpr int kAnyK = 16;
+
+template <bool kGuard>
+__global__ __launch_bounds__(256)
+void GemmBf16AnyShapeKernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                            uint16_t *__restrict__ C, int M, int N, int K, uint32_t tiles_n, XGuardArgs g)
+{
+    // a row of 16 k values padded to 24: 48-byte rows, every 16-byte fragment aligned
+    __shared__ __attribute__((aligned(16))) uint16_t a_rows[kAnyTile][kAnyK + 8];
+    __shared__ __attribute__((aligned(16))) uint16_t b_cols[kAnyTile][kAnyK + 8];   // B transposed: [column][k]
+    __shared__ uint32_t guard_word;
+
+    XGuardBlock guard(g, blockIdx.x, &guard_word);
+    if (kGuard && !guard.Enter()) return;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1;
+    const size_t m0 = (size_t)(blockIdx.x / tiles_n) * kAnyTile, n0 = (size_t)(blockIdx.x % tiles_n) * kAnyTile;
+
+    // loads of a slice: thread t takes A[m0 + t / 4][k0 + 4 (t % 4) + 0..3] and
+    // B[k0 + t / 16][n0 + 4 (t % 16) + 0..3]
+    const uint32_t a_row = tid >> 2, a_k = (tid & 3) * 4;
+    const uint32_t b_k = tid >> 4, b_col = (tid & 15) * 4;
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+    for (size_t k0 = 0; k0 < (size_t)K; k0 += kAnyK) {
+        uint16_t a[4], b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const size_t row = m0 + a_row, k = (size_t)k0 + a_k + i;
+            a[i] = row < (size_t)M && k < (size_t)K ? A[row * (size_t)K + k] : (uint16_t)0;
+            const size_t kk = (size_t)k0 + b_k, col = n0 + b_col + i;
+            b[i] = kk < (size_t)K && col < (size_t)N ? B[kk * (size_t)N + col] : (uint16_t)0;
+        }
+        __syncthreads();   // the fragments of the previous slice have been read
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a_rows[a_row][a_k + i] = a[i];
+            b_cols[b_col + i][b_k] = b[i];
+        }
+        __syncthreads();
+        // lane l: A[row l % 32][k 8 (l / 32) + 0..7], B[k 8 (l / 32) + 0..7][column l % 32]
+        const bf16x8 fa = *(const bf16x8 *)&a_rows[32 * wm + (lane & 31)][8 * (lane >> 5)];
+        const bf16x8 fb = *(const bf16x8 *)&b_cols[32 * wn + (lane & 31)][8 * (lane >> 5)];
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+    }
+
+    // accumulator 4 run + r of lane l: row 8 run + 4 (l / 32) + r, column l % 32 of the block
+    const size_t col = n0 + 32 * wn + (lane & 31);
+    if (col < (size_t)N) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const size_t row = m0 + 32 * wm + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+            if (row < (size_t)M) C[row * (size_t)N + col] = (uint16_t)f32x2_to_bf16x2_rne(acc[i], 0.0f);
+        }
+    }
+    if (kGuard) guard.Commit();
+}
+
 class HipGemmCommand final : public HipGuardedCommand
 {
 public:
     HipGemmCommand(const void *A, const void *B, void *C, int M, int N, int K, int tile, int guard_mode)
-        : HipGuardedCommand((uint32_t)(M / tile) * (uint32_t)(N / tile), guard_mode)
+        : HipGuardedCommand((uint32_t)((M + tile - 1) / tile) * (uint32_t)((N + tile - 1) / tile), guard_mode)
         , A_((const uint16_t *)A), B_((const uint16_t *)B), C_((uint16_t *)C), M_(M), N_(N), K_(K), tile_(tile) {}
 
 protected:
@@ -417,7 +485,12 @@ protected:
     {
         const dim3 grid(n_wg_);
         const hipEvent_t stop = TakeStopEvent();
-        if (tile_ == kLargeTile) {
+        if (tile_ == kAnyTile) {
+            const dim3 block(256);
+            const uint32_t tiles_n = (uint32_t)((N_ + kAnyTile - 1) / kAnyTile);
+            if (guarded) LaunchWithStop(stop, GemmBf16AnyShapeKernel<true>, grid, block, stream, A_, B_, C_, M_, N_, K_, tiles_n, g);
+            else         LaunchWithStop(stop, GemmBf16AnyShapeKernel<false>, grid, block, stream, A_, B_, C_, M_, N_, K_, tiles_n, g);
+        } else if (tile_ == kLargeTile) {
             const dim3 block(512);
             if (guarded) LaunchWithStop(stop, (GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
             else         LaunchWithStop(stop, (GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
@@ -441,6 +514,13 @@ private:
 /// of the device idle. Small tiles when the large ones would cover at most half of the compute
 /// units, or when M or N is no multiple of the large edge. XSCHED_HIP_GEMM_TILE=128|256
 /// overrides the choice where the shape allows.
+/// Whether the fast kernels take the shape and the pointers.
+inline bool FastKernelsTake(const void *A, const void *B, const void *C, int M, int N, int K)
+{
+    return M % kSmallTile == 0 && N % kSmallTile == 0 && K % kStepK == 0 && K <= kMaxK && N <= kMaxK &&
+           (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) == 0;
+}
+
 inline int TileFor(int M, int N)
 {
     const bool large_fits = M % kLargeTile == 0 && N % kLargeTile == 0;
@@ -468,15 +548,19 @@ EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void 
     if (cmd == nullptr || A == nullptr || B == nullptr || C == nullptr || guard < 0 || guard > 3) {
         return kXSchedErrorInvalidValue;
     }
-    if (M <= 0 || N <= 0 || K <= 0 || M % gemm::kSmallTile || N % gemm::kSmallTile || K % gemm::kStepK ||
-        K > gemm::kMaxK || N > gemm::kMaxK) {
-        XWARN("HipGemmBf16CommandCreate: M and N must be multiples of 128 and K of 64, K and N at most 2^22 (got %d %d %d)", M, N, K);
+    if (M <= 0 || N <= 0 || K <= 0 || (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 1) != 0) {
+        XWARN("HipGemmBf16CommandCreate: M, N and K must be positive and the matrices aligned to their elements (got %d %d %d)", M, N, K);
         return kXSchedErrorInvalidValue;
     }
-    const int tile = gemm::TileFor(M, N);
-    if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) return kXSchedErrorInvalidValue;
+    // The fast kernels take M and N in multiples of 128, K in multiples of 64 (K and N at most
+    // 2^22) and matrices aligned to 16 bytes; every other shape goes to the any-shape kernel.
+    int64_t forced = 0;
+    const bool any_shape = !gemm::FastKernelsTake(A, B, C, M, N, K) ||
+                           (GetEnvInt64("XSCHED_HIP_GEMM_TILE", forced) && forced == gemm::kAnyTile);
+    const int tile = any_shape ? gemm::kAnyTile : gemm::TileFor(M, N);
     // one progress-map byte per tile
-    if ((uint64_t)(M / tile) * (uint64_t)(N / tile) > GuardState::kMaxWorkGroups) {
+    if ((uint64_t)((M + tile - 1) / tile) * (uint64_t)((N + tile - 1) / tile) > GuardState::kMaxWorkGroups) {
+        XWARN("HipGemmBf16CommandCreate: %d x %d has more than 2^18 tiles of %d x %d", M, N, tile, tile);
         return kXSchedErrorInvalidValue;
     }
     *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, tile, guard));
