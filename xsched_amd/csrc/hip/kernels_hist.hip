@@ -114,6 +114,7 @@ static_assert(kCountWords <= kLdsBins, "the merge layout's counters fit the grou
 // words: the counts of bins 0..255, which are kept outside the bytes, partial by partial
 // (1 KiB each).
 constexpr uint32_t kMergeGroups = 256;
+constexpr uint32_t kMergeThreads = 256;             // threads of a merge group
 constexpr uint32_t kMergeWords = kColdWords / kMergeGroups;          // byte words per column (64)
 constexpr uint32_t kPartialWords = kColdWords + kWarmBins;           // 65 KiB of scratch per counting group
 
@@ -525,6 +526,8 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
         for (uint32_t k = tid * 4; k < kColdWords; k += kThreads * 4) {
             const uint32_t i = (k + turn) & (kColdWords - 1);
             const u32x4 w = *(const u32x4 *)&sh.bins[i];
+            // (a plain store: non-temporal ones make the command 1.5 us slower, the counting
+            // kernel and the merge kernel's reads both)
             *(u32x4 *)&partials[ColumnAt(i / kMergeWords, me, n_part) + i % kMergeWords] = w;
             counted += ByteSum(w);
         }
@@ -597,17 +600,18 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 /// Sums the partial histograms of the counting groups and adds the totals to bins. Group j
 /// owns column j of every partial: 64 words of byte counters (word w, byte b = bin
 /// w + b * 16384) and the count of bin j, which is kept outside the bytes. Thread (row, col)
-/// reads four byte words of its column from partials row, row + 64, ... (the sixteen threads
+/// reads four byte words of its column from partials row, row + 16, ... (the sixteen threads
 /// of a row one partial's 256 bytes, the four rows of a wave four neighbouring partials: one
 /// KiB in a piece); the threads of col 0 also read the outside count. The group's progress
-/// byte is first_wg + j.
+/// byte is first_wg + j. Four waves per group: the kernel is one round trip to its partials,
+/// a reduction and 256 atomics, and most of its time is getting its waves started.
 template <bool kGuard>
-__global__ __launch_bounds__(kThreads)
+__global__ __launch_bounds__(kMergeThreads)
 void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part, uint32_t *__restrict__ bins,
                           uint32_t n_bins, uint32_t first_wg, XGuardArgs g)
 {
-    constexpr uint32_t kCols = kMergeWords / 4, kRows = kThreads / kCols; // 16 x 64
-    constexpr uint32_t kAhead = 4;                                       // rows requested before the guard's reads
+    constexpr uint32_t kCols = kMergeWords / 4, kRows = kMergeThreads / kCols; // 16 x 16
+    constexpr uint32_t kAhead = 16;                                      // rows requested before the guard's reads
     __shared__ uint32_t red[kRows][16][kCols];   // per row: the 16 byte counters of each of the 16 word quads
     __shared__ uint32_t total[16][kCols];
     __shared__ uint32_t outside_total;
@@ -623,7 +627,7 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
         return col == 0 && p < n_part ? partials[OutsideAt(p, n_part) + column] : 0u;
     };
     // even[i] holds bytes 0 and 2 of word i in its halves, odd[i] bytes 1 and 3; a thread adds
-    // at most kMaxPartials / kRows = 16 values of 255 into a half.
+    // at most kMaxPartials / kRows = 64 values of 255 into a half.
     uint32_t even[4] = { 0, 0, 0, 0 }, odd[4] = { 0, 0, 0, 0 }, outside = 0;
     auto add_words = [&](const u32x4 &w) {
         const uint32_t v[4] = { w.x, w.y, w.z, w.w };
@@ -645,10 +649,10 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
     if (kGuard) {
         // A flushed counting launch leaves partials missing: every counting group must have
         // committed. Their progress bytes are requested ahead of the other reads.
-        uint8_t tag[kMaxPartials / kThreads];
+        uint8_t tag[kMaxPartials / kMergeThreads];
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) {
-            const uint32_t p = tid + i * kThreads;
+        for (uint32_t i = 0; i < kMaxPartials / kMergeThreads; ++i) {
+            const uint32_t p = tid + i * kMergeThreads;
             tag[i] = g.done != nullptr && p < n_part ? __builtin_nontemporal_load(&g.done[p]) : (uint8_t)g.gen;
         }
         // guard_word = 1 is in place before any wave takes it back: the loads above take a
@@ -665,7 +669,7 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
             if (!stop && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) stop = true;
         }
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxPartials / kThreads; ++i) stop |= tag[i] != (uint8_t)g.gen;
+        for (uint32_t i = 0; i < kMaxPartials / kMergeThreads; ++i) stop |= tag[i] != (uint8_t)g.gen;
         if (stop) guard_word = 0;   // any number of threads, the same value
         __syncthreads();
         if (guard_word == 0) return;
@@ -687,7 +691,8 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
     }
     if (outside != 0) LdsAdd(&outside_total, outside);
     __syncthreads();
-    if (tid < 16 * kCols) {
+    static_assert(kMergeThreads == 16 * kCols, "one thread per counter of the column");
+    {
         const uint32_t v = tid / kCols, c = tid % kCols;
         uint32_t t = 0;
 #pragma unroll 16
@@ -696,22 +701,16 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
     }
     __syncthreads();
 
-    // 256 counters, 128 pairs of neighbouring bins: counter (b, i) of quad c is bin
-    // column * 64 + c * 4 + i + b * 16384.
-    const bool pair_ok = (((uintptr_t)bins) & 7) == 0;
-    if (tid < 128) {
-        const uint32_t b = tid / 32, c = (tid % 32) / 2, i = (tid % 2) * 2;
-        const uint32_t lo = total[b * 4 + i][c], hi = total[b * 4 + i + 1][c];
+    // 256 counters: counter (b, i) of quad c is bin column * 64 + c * 4 + i + b * 16384. One
+    // 32-bit add each, nothing returned, so no wave waits for the round trip; the 64 lanes of a
+    // wave add to 64 neighbouring bins.
+    {
+        const uint32_t b = tid / 64, c = (tid % 64) / 4, i = tid % 4;
+        const uint32_t count = total[b * 4 + i][c];
         const uint32_t bin = column * kMergeWords + c * 4 + i + b * kColdWords;
-        if ((lo | hi) != 0) {
-            if (pair_ok && bin + 1 < n_bins) {
-                PairFix(bins + bin, PairAdd(bins + bin, lo, hi), lo);
-            } else {
-                if (lo != 0 && bin < n_bins) GlobalAdd(bins + bin, lo);
-                if (hi != 0 && bin + 1 < n_bins) GlobalAdd(bins + bin + 1, hi);
-            }
-        }
-    } else if (tid == 128) {
+        if (count != 0 && bin < n_bins) GlobalAdd(bins + bin, count);
+    }
+    if (tid == 0) {
         // bin <column>, counted outside the bytes (which hold nothing for bins below 256)
         if (outside_total != 0 && column < n_bins) GlobalAdd(bins + column, outside_total);
     }
@@ -769,10 +768,10 @@ protected:
         else         LaunchWithStop(stop, (HistogramKernel<false, true>), grid, block, stream, keys_, (uint64_t)n_, bins_, n_bins_, chunk_, partials_, g);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) return err;
-        const dim3 merge_grid(kMergeGroups);
+        const dim3 merge_grid(kMergeGroups), merge_block(kMergeThreads);
         stop = TakeStopEvent();
-        if (guarded) LaunchWithStop(stop, HistogramMergeKernel<true>, merge_grid, block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
-        else         LaunchWithStop(stop, HistogramMergeKernel<false>, merge_grid, block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
+        if (guarded) LaunchWithStop(stop, HistogramMergeKernel<true>, merge_grid, merge_block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
+        else         LaunchWithStop(stop, HistogramMergeKernel<false>, merge_grid, merge_block, stream, (const uint32_t *)partials_, n_count_wg_, bins_, n_bins_, n_count_wg_, g);
         return hipGetLastError();
     }
 
@@ -888,7 +887,7 @@ EXPORT_C_FUNC XResult HipHistogramLaunchNoAlloc(void *stream_ptr, const void *ke
                            (const int32_t *)keys, (uint64_t)n, (uint32_t *)bins, n_bins, chunk, partials, inert);
         hipError_t err = hipGetLastError();
         if (err == hipSuccess) {
-            hipLaunchKernelGGL(hist::HistogramMergeKernel<false>, dim3(hist::kMergeGroups), block, 0, stream,
+            hipLaunchKernelGGL(hist::HistogramMergeKernel<false>, dim3(hist::kMergeGroups), dim3(hist::kMergeThreads), 0, stream,
                                (const uint32_t *)partials, (uint32_t)n_wg, (uint32_t *)bins, n_bins, (uint32_t)n_wg, inert);
             err = hipGetLastError();
         }
