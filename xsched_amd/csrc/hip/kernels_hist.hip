@@ -644,38 +644,25 @@ void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part
         first[i] = load_words(row + i * kRows);
         first_outside[i] = load_outside(row + i * kRows);
     }
-    if (tid == 0) { outside_total = 0; guard_word = 1; }
-
-    if (kGuard) {
-        // A flushed counting launch leaves partials missing: every counting group must have
-        // committed. Their progress bytes are requested ahead of the other reads.
-        uint8_t tag[kMaxPartials / kMergeThreads];
-#pragma unroll
-        for (uint32_t i = 0; i < kMaxPartials / kMergeThreads; ++i) {
-            const uint32_t p = tid + i * kMergeThreads;
-            tag[i] = g.done != nullptr && p < n_part ? __builtin_nontemporal_load(&g.done[p]) : (uint8_t)g.gen;
-        }
-        // guard_word = 1 is in place before any wave takes it back: the loads above take a
-        // memory round trip, this barrier none. (A vote of the whole group instead of the
-        // plain stores below costs two barriers and a reduction through the LDS.)
-        __syncthreads();
+    if (tid == 0) {
+        outside_total = 0;
         // This kernel does not look at the preempt word itself: it runs for a few
         // microseconds, and what it must not do is run after a counting launch that was
-        // flushed. Every flushed group has left its epoch in the `flushed` word, and the tags
-        // say whether every partial is there; its own tag says whether it ran before the flush.
-        bool stop = false;
-        if (tid == 0) {
-            stop = xguard_epoch_flushed(g);
-            if (!stop && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) stop = true;
+        // flushed, whose partials are incomplete. Every counting group that leaves because of
+        // a deactivation puts the epoch of its launch into the `flushed` word before it does
+        // (and every group that starts later finds the word and leaves the same way): the
+        // word differs from this launch's epoch exactly when every counting group has run to
+        // its end, now or in an earlier launch. The group's own tag says whether it has added
+        // its column already, before a flush that made this launch a replay.
+        bool go = true;
+        if (kGuard) {
+            go = !xguard_epoch_flushed(g);
+            if (go && g.resume && g.done && xguard_committed(g, first_wg + blockIdx.x)) go = false;
         }
-#pragma unroll
-        for (uint32_t i = 0; i < kMaxPartials / kMergeThreads; ++i) stop |= tag[i] != (uint8_t)g.gen;
-        if (stop) guard_word = 0;   // any number of threads, the same value
-        __syncthreads();
-        if (guard_word == 0) return;
-    } else {
-        __syncthreads();
+        guard_word = go ? 1u : 0u;
     }
+    __syncthreads();
+    if (kGuard && guard_word == 0) return;
 
 #pragma unroll
     for (uint32_t i = 0; i < kAhead; ++i) { add_words(first[i]); outside += first_outside[i]; }
