@@ -850,7 +850,8 @@ def main():
 
     line = {2: config2, 3: config3, 4: config4, 5: config5}[a.config](H, a)
     if isinstance(line.get("config"), dict):
-        line["config"]["runtime_env"] = {"ROC_SIGNAL_POOL_SIZE": os.environ.get("ROC_SIGNAL_POOL_SIZE")}
+        line["config"]["runtime_env"] = {"ROC_SIGNAL_POOL_SIZE": os.environ.get("ROC_SIGNAL_POOL_SIZE"),
+                                         "XSCHED_HIP_MARKER_ON_KERNEL": os.environ.get("XSCHED_HIP_MARKER_ON_KERNEL", "ON (default)")}
     if a.config == 2 and not a.quick:
         line["others"] = other_configurations(H, a)
         line["shim_launch_cost"] = shim_launch_cost()

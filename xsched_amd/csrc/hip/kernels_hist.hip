@@ -604,7 +604,7 @@ void HistogramKernel(const int32_t *__restrict__ keys, uint64_t n, uint32_t *__r
 /// of a row one partial's 256 bytes, the four rows of a wave four neighbouring partials: one
 /// KiB in a piece); the threads of col 0 also read the outside count. The group's progress
 /// byte is first_wg + j. Four waves per group: the kernel is one round trip to its partials,
-/// a reduction and 256 atomics, and most of its time is getting its waves started.
+/// a reduction through 16 KiB of LDS and 256 atomics.
 template <bool kGuard>
 __global__ __launch_bounds__(kMergeThreads)
 void HistogramMergeKernel(const uint32_t *__restrict__ partials, uint32_t n_part, uint32_t *__restrict__ bins,
