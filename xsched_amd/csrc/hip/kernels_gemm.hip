@@ -63,7 +63,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int kLargeTile = 256;     // edge of the large tile of C (M and N)
 constexpr int kSmallTile = 128;     // edge of the small one
 constexpr int kStepK = 64;          // K per step
-constexpr int kPollSteps = 8;       // K steps between two looks at the preempt word
+constexpr int kPollSteps = 4;       // K steps between two looks at the preempt word
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 4;       // tile rows walked together
 constexpr int kMaxK = 1 << 22;      // 32-bit byte offsets inside a 256-row panel of A
