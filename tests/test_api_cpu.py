@@ -59,20 +59,26 @@ def test_hip_library_loads_without_a_gpu(xs):
     assert lib.HipQueueCreate is not None
 
 
-def test_gemm_command_refuses_shapes_its_kernel_cannot_address(xs):
-    """Creating a command launches nothing, so the argument checks run without a GPU: M and N in
-    multiples of 128, K of 64, K and N at most 2^22 (the kernel addresses a tile's panels with
-    32-bit byte offsets), operands 16-byte aligned, guard mode 0..3."""
+def test_gemm_command_takes_any_shape_and_refuses_what_no_kernel_can_address(xs):
+    """Creating a command launches nothing, so the argument checks run without a GPU. The fast
+    kernels take M and N in multiples of 128, K of 64 (K and N at most 2^22) and operands
+    aligned to 16 bytes; everything else with positive sizes and element-aligned operands goes
+    to the any-shape kernel. Refused: sizes below 1, odd addresses, null pointers, guard modes
+    outside 0..3, more tiles than a progress map has bytes."""
     from ctypes import byref, c_uint64
     lib, cmd = xs.halhip(), c_uint64()
     a, b, c = 1 << 20, 2 << 20, 3 << 20           # never dereferenced here
     ok = lambda *args: lib.HipGemmBf16CommandCreate(byref(cmd), *args)  # noqa: E731
-    assert ok(a, b, c, 256, 384, 64, 0) == xs.kXSchedSuccess
-    assert ok(a, b, c, 128, 128, 1 << 22, 1) == xs.kXSchedSuccess
-    for bad in [(a, b, c, 200, 256, 64, 0), (a, b, c, 256, 200, 64, 0), (a, b, c, 256, 256, 96, 0),
-                (a, b, c, 256, 256, (1 << 22) + 64, 0), (a, b, c, 256, (1 << 22) + 128, 64, 0),
-                (a + 2, b, c, 256, 256, 64, 0), (a, b, c + 8, 256, 256, 64, 0),
-                (a, b, c, 256, 256, 64, 4), (a, b, c, 0, 256, 64, 0), (0, b, c, 256, 256, 64, 0)]:
+    for good in [(a, b, c, 256, 384, 64, 0), (a, b, c, 128, 128, 1 << 22, 1),
+                 (a, b, c, 200, 256, 64, 0), (a, b, c, 256, 200, 64, 0), (a, b, c, 256, 256, 96, 0),
+                 (a, b, c, 256, 256, (1 << 22) + 64, 0), (a + 2, b, c, 256, 256, 64, 0),
+                 (a, b, c + 8, 256, 256, 64, 0), (a, b, c, 1, 1, 1, 3)]:
+        assert ok(*good) == xs.kXSchedSuccess, good
+    for bad in [(a, b, c, 256, 256, 64, 4), (a, b, c, 256, 256, 64, -1), (a, b, c, 0, 256, 64, 0),
+                (a, b, c, 256, 0, 64, 0), (a, b, c, 256, 256, 0, 0), (a, b, c, -128, 256, 64, 0),
+                (0, b, c, 256, 256, 64, 0), (a, 0, c, 256, 256, 64, 0), (a, b, 0, 256, 256, 64, 0),
+                (a + 1, b, c, 256, 256, 64, 0), (a, b, c + 1, 8, 8, 8, 0),
+                (a, b, c, 64 * 1024, 64 * 1024 + 1, 1, 1)]:
         assert ok(*bad) == xs.kXSchedErrorInvalidValue, bad
 
 
