@@ -45,13 +45,16 @@ XResult HipQueueGetStats(HwQueueHandle hwq, uint64_t *out);
  * hipStreamSynchronize() blocks for that long. on == 0: every marker is a hipEventRecord()
  * behind its command, and the stream is idle for the runtime as soon as the XQueue is.
  * For programs that wait on the raw stream themselves (the interception shim does this for
- * its queues). Takes effect for commands launched afterwards. */
+ * its queues). Takes effect for commands launched afterwards. No counterpart in the
+ * reference, whose HIP adapter records an event behind every marked command
+ * (platforms/hip/hal/src/hip_command.cpp:38-44). */
 XResult HipQueueSetMarkerOnKernel(HwQueueHandle hwq, int on);
 
 /* Device memory the queue's pools hold for guarded commands, for tests. `out` receives 4
  * values: [0] scratch buffers allocated (the partial histograms of histogram commands),
  * [1] their bytes, [2] progress-map slots allocated, [3] progress-map slots in use. Both
- * pools grow with what is launched and not yet destroyed, not with what waits in the XQueue. */
+ * pools grow with what is launched and not yet destroyed, not with what waits in the XQueue.
+ * No counterpart in the reference (its HIP adapter has no level 2). */
 XResult HipQueueGetPoolStats(HwQueueHandle hwq, uint64_t *out);
 
 /* For tests of the guard protocol: stores the queue's current preempt epoch into its
