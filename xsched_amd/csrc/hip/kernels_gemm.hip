@@ -406,20 +406,22 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
 
 
 // Any shape: M, N, K >= 1, any alignment of the three matrices to two bytes. 64 x 64 tiles of
-// C, four waves of one 32x32 block each, K in slices of 16 through the same MFMA as above and
-// in the same order (so an element is summed as the kernels above sum it; what lies beyond
-// K is zero). Every load and store is checked against the matrix: this kernel is the fall-back
-// for the shapes the fast kernels do not take, not a fast kernel. The guard is at entry only:
-// a tile is short.
+// C, four waves of one 32x32 block each, K in steps of 32 (two slices of 16 through the same
+// MFMA as above and in the same order, so an element is summed as the kernels above sum it;
+// what lies beyond K is zero). Every load and store is checked against the matrix; a thread's
+// eight neighbouring elements come as one 16-byte load where they lie inside the matrix and
+// are aligned, one by one otherwise. The loads of the next step are on their way while the
+// current one is multiplied. This kernel is the fall-back for the shapes the fast kernels do
+// not take, 10-20 times slower than they are. The guard is at entry only: a tile is short.
 constexpr int kAnyTile = 64;
-constexpr int kAnyK = 16;
+constexpr int kAnyK = 32;
 
 template <bool kGuard>
 __global__ __launch_bounds__(256)
 void GemmBf16AnyShapeKernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                             uint16_t *__restrict__ C, int M, int N, int K, uint32_t tiles_n, XGuardArgs g)
 {
-    // a row of 16 k values padded to 24: 48-byte rows, every 16-byte fragment aligned
+    // a row of 32 k values padded to 40: 80-byte rows, every 16-byte fragment aligned
     __shared__ __attribute__((aligned(16))) uint16_t a_rows[kAnyTile][kAnyK + 8];
     __shared__ __attribute__((aligned(16))) uint16_t b_cols[kAnyTile][kAnyK + 8];   // B transposed: [column][k]
     __shared__ uint32_t guard_word;
@@ -430,44 +432,57 @@ void GemmBf16AnyShapeKernel(const uint16_t *__restrict__ A, const uint16_t *__re
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave >> 1, wn = wave & 1;
     const size_t m0 = (size_t)(blockIdx.x / tiles_n) * kAnyTile, n0 = (size_t)(blockIdx.x % tiles_n) * kAnyTile;
+    const size_t Ms = (size_t)M, Ns = (size_t)N, Ks = (size_t)K;
 
-    // loads of a slice: thread t takes A[m0 + t / 4][k0 + 4 (t % 4) + 0..3] and
-    // B[k0 + t / 16][n0 + 4 (t % 16) + 0..3]
-    const uint32_t a_row = tid >> 2, a_k = (tid & 3) * 4;
-    const uint32_t b_k = tid >> 4, b_col = (tid & 15) * 4;
+    // loads of a step: thread t takes A[m0 + t / 4][k0 + 8 (t % 4) + 0..7] and
+    // B[k0 + t / 8][n0 + 8 (t % 8) + 0..7]
+    const uint32_t a_row = tid >> 2, a_k = (tid & 3) * 8;
+    const uint32_t b_k = tid >> 3, b_col = (tid & 7) * 8;
+    union Eight { u32x4 v; uint16_t e[8]; };
+    auto load_eight = [](const uint16_t *base, size_t first, size_t end, bool row_inside) {
+        Eight r;
+        r.v = u32x4 { 0, 0, 0, 0 };
+        if (!row_inside || first >= end) return r;
+        const uint16_t *p = base + first;
+        if (first + 8 <= end && (((uintptr_t)p) & 15) == 0) {
+            r.v = *(const u32x4 *)p;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r.e[i] = first + i < end ? p[i] : (uint16_t)0;
+        }
+        return r;
+    };
+    auto load_a = [&](size_t k0) { return load_eight(A + (m0 + a_row) * Ks, k0 + a_k, Ks, m0 + a_row < Ms); };
+    auto load_b = [&](size_t k0) { return load_eight(B + (k0 + b_k) * Ns, n0 + b_col, Ns, k0 + b_k < Ks); };
+
     f32x16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-    for (size_t k0 = 0; k0 < (size_t)K; k0 += kAnyK) {
-        uint16_t a[4], b[4];
+    Eight a = load_a(0), b = load_b(0);
+    for (size_t k0 = 0; k0 < Ks; k0 += kAnyK) {
+        __syncthreads();   // the fragments of the previous step have been read
+        *(u32x4 *)&a_rows[a_row][a_k] = a.v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const size_t row = m0 + a_row, k = (size_t)k0 + a_k + i;
-            a[i] = row < (size_t)M && k < (size_t)K ? A[row * (size_t)K + k] : (uint16_t)0;
-            const size_t kk = (size_t)k0 + b_k, col = n0 + b_col + i;
-            b[i] = kk < (size_t)K && col < (size_t)N ? B[kk * (size_t)N + col] : (uint16_t)0;
-        }
-        __syncthreads();   // the fragments of the previous slice have been read
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            a_rows[a_row][a_k + i] = a[i];
-            b_cols[b_col + i][b_k] = b[i];
-        }
+        for (int i = 0; i < 8; ++i) b_cols[b_col + i][b_k] = b.e[i];
         __syncthreads();
-        // lane l: A[row l % 32][k 8 (l / 32) + 0..7], B[k 8 (l / 32) + 0..7][column l % 32]
-        const bf16x8 fa = *(const bf16x8 *)&a_rows[32 * wm + (lane & 31)][8 * (lane >> 5)];
-        const bf16x8 fb = *(const bf16x8 *)&b_cols[32 * wn + (lane & 31)][8 * (lane >> 5)];
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+        if (k0 + kAnyK < Ks) { a = load_a(k0 + kAnyK); b = load_b(k0 + kAnyK); }
+        // lane l: A[row l % 32][k 8 (l / 32) + 0..7], B[k 8 (l / 32) + 0..7][column l % 32], per slice of 16
+#pragma unroll
+        for (int kk = 0; kk < kAnyK; kk += 16) {
+            const bf16x8 fa = *(const bf16x8 *)&a_rows[32 * wm + (lane & 31)][kk + 8 * (lane >> 5)];
+            const bf16x8 fb = *(const bf16x8 *)&b_cols[32 * wn + (lane & 31)][kk + 8 * (lane >> 5)];
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+        }
     }
 
     // accumulator 4 run + r of lane l: row 8 run + 4 (l / 32) + r, column l % 32 of the block
     const size_t col = n0 + 32 * wn + (lane & 31);
-    if (col < (size_t)N) {
+    if (col < Ns) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const size_t row = m0 + 32 * wm + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-            if (row < (size_t)M) C[row * (size_t)N + col] = (uint16_t)f32x2_to_bf16x2_rne(acc[i], 0.0f);
+            if (row < Ms) C[row * Ns + col] = (uint16_t)f32x2_to_bf16x2_rne(acc[i], 0.0f);
         }
     }
     if (kGuard) guard.Commit();
