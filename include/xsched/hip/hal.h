@@ -88,7 +88,9 @@ XResult HipAxpyCommandCreate(HwCommandHandle *cmd, float alpha, const void *x, v
  * kernel takes M, N in multiples of 128, K in multiples of 64 (K, N <= 2^22) and matrices
  * aligned to 16 bytes: it works on 256x256 tiles of C, or on 128x128 tiles when M or N is no
  * multiple of 256 or the large tiles would cover at most half of the compute units
- * (XSCHED_HIP_GEMM_TILE=128|256 overrides that). Every other shape or alignment runs on a
+ * (XSCHED_HIP_GEMM_TILE=128|256 overrides that). Where only M is not as the fast kernel wants
+ * it, the fast kernel takes the rows up to the last multiple of 128 and the kernel below the
+ * rest, in one command. Every other shape or alignment runs on a
  * bounds-checked kernel with 64x64 tiles (XSCHED_HIP_GEMM_TILE=64 forces it): correct and
  * guarded like the others, 5-20 times slower (180-230 TFLOP/s where rows are 16-byte aligned,
  * 60 where they are not). Every element is summed in the same order

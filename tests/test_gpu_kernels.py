@@ -403,6 +403,32 @@ def test_gemm_any_shape(xs, gpu, M, N, K, level, guard):
     assert np.all(got[:pad] == 0x1234) and np.all(got[pad + M * N:] == 0x1234)
 
 
+@pytest.mark.parametrize("M,N,K", [(129, 128, 64), (200, 256, 64), (1000, 384, 128), (2049, 256, 192), (127, 256, 64)])
+@pytest.mark.parametrize("level,guard", [(1, 0), (2, 1)])
+def test_gemm_ragged_rows_are_split_between_the_kernels(xs, gpu, M, N, K, level, guard):
+    """N and K as the fast kernel wants them, M not (the usual ragged dimension): the rows up to
+    the last multiple of 128 go to the fast kernel, the rest to the any-shape kernel, in one
+    command (M below 128: all of it to the any-shape kernel). Integers, so the result is
+    determined; the rows behind the matrix in C's buffer stay untouched."""
+    torch = gpu
+    print(f"case gemm-split M={M} N={N} K={K} level={level} guard={guard}", flush=True)
+    rng = np.random.default_rng(10)
+    a_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b_i = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    a_bits, b_bits = oracle.f32_to_bf16_bits(a_i), oracle.f32_to_bf16_bits(b_i)
+    want = oracle.gemm_bf16(a_bits.ravel(), b_bits.ravel(), M, N, K).reshape(M, N)
+    a = torch.from_numpy(a_bits.view(np.int16).reshape(M, K)).cuda()
+    b = torch.from_numpy(b_bits.view(np.int16).reshape(K, N)).cuda()
+    c = torch.full((M + 2, N), 0x1234, dtype=torch.int16, device="cuda")
+    q = Queue(xs, torch, level)
+    q.submit(gemm_cmd(xs, a, b, c, M, N, K, guard))
+    q.wait()
+    got = c.cpu().numpy().view(np.uint16)
+    q.close()
+    assert np.array_equal(got[:M], want)
+    assert np.all(got[M:] == 0x1234)
+
+
 def test_gemm_any_shape_kernel_sums_as_the_fast_kernels_do(xs, gpu, monkeypatch):
     """Seeded normal inputs on a shape every kernel takes: the any-shape kernel (forced)
     feeds the matrix cores the same slices of 16 along K in the same order, so the bits agree."""

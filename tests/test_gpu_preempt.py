@@ -198,9 +198,11 @@ def test_commands_waiting_in_the_xqueue_hold_no_device_memory(xs, gpu):
     assert np.array_equal(got.astype(np.uint64), (one * burst) & 0xFFFFFFFF)
 
 
-@pytest.mark.parametrize("tile,shape", [(128, (2048, 2048, 2048)), (256, (2048, 2048, 2048)), (64, (1000, 1999, 1030))])
+@pytest.mark.parametrize("tile,shape", [(128, (2048, 2048, 2048)), (256, (2048, 2048, 2048)), (64, (1000, 1999, 1030)),
+                                        (128, (1960, 2048, 1024))])
 def test_gemm_preempt_resume_matches_uninterrupted(xs, gpu, monkeypatch, tile, shape):
-    """Both tile sizes of the fast kernel, and the any-shape kernel on a shape only it takes."""
+    """Both tile sizes of the fast kernel, the any-shape kernel on a shape only it takes, and a
+    command whose rows are split between the two."""
     torch = gpu
     monkeypatch.setenv("XSCHED_HIP_GEMM_TILE", str(tile))
     M, N, K = shape

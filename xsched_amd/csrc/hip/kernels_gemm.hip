@@ -412,21 +412,22 @@ void GemmBf16Kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__
 // eight neighbouring elements come as one 16-byte load where they lie inside the matrix and
 // are aligned, one by one otherwise. The loads of the next step are on their way while the
 // current one is multiplied. This kernel is the fall-back for the shapes the fast kernels do
-// not take, 10-20 times slower than they are. The guard is at entry only: a tile is short.
+// not take, 5-20 times slower than they are. The guard is at entry only: a tile is short.
 constexpr int kAnyTile = 64;
 constexpr int kAnyK = 32;
 
 template <bool kGuard>
 __global__ __launch_bounds__(256)
 void GemmBf16AnyShapeKernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                            uint16_t *__restrict__ C, int M, int N, int K, uint32_t tiles_n, XGuardArgs g)
+                            uint16_t *__restrict__ C, int M, int N, int K, uint32_t tiles_n, uint32_t first_wg,
+                            XGuardArgs g)
 {
     // a row of 32 k values padded to 40: 80-byte rows, every 16-byte fragment aligned
     __shared__ __attribute__((aligned(16))) uint16_t a_rows[kAnyTile][kAnyK + 8];
     __shared__ __attribute__((aligned(16))) uint16_t b_cols[kAnyTile][kAnyK + 8];   // B transposed: [column][k]
     __shared__ uint32_t guard_word;
 
-    XGuardBlock guard(g, blockIdx.x, &guard_word);
+    XGuardBlock guard(g, first_wg + blockIdx.x, &guard_word);   // its progress bytes follow the fast kernel's
     if (kGuard && !guard.Enter()) return;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -488,32 +489,50 @@ void GemmBf16AnyShapeKernel(const uint16_t *__restrict__ A, const uint16_t *__re
     if (kGuard) guard.Commit();
 }
 
+/// Rows [0, rows_fast) of C go to the fast kernel with tiles of fast_tile (rows_fast is then a
+/// multiple of it and the shape one the fast kernel takes), rows [rows_fast, M) to the any-shape
+/// kernel; either part may be empty. The progress map holds the fast kernel's tiles first.
 class HipGemmCommand final : public HipGuardedCommand
 {
 public:
-    HipGemmCommand(const void *A, const void *B, void *C, int M, int N, int K, int tile, int guard_mode)
-        : HipGuardedCommand((uint32_t)((M + tile - 1) / tile) * (uint32_t)((N + tile - 1) / tile), guard_mode)
-        , A_((const uint16_t *)A), B_((const uint16_t *)B), C_((uint16_t *)C), M_(M), N_(N), K_(K), tile_(tile) {}
+    HipGemmCommand(const void *A, const void *B, void *C, int M, int N, int K, int rows_fast, int fast_tile, int guard_mode)
+        : HipGuardedCommand(FastTiles(rows_fast, N, fast_tile) + AnyTiles(M - rows_fast, N), guard_mode)
+        , A_((const uint16_t *)A), B_((const uint16_t *)B), C_((uint16_t *)C), M_(M), N_(N), K_(K)
+        , rows_fast_(rows_fast), fast_tile_(fast_tile) {}
+
+    static uint32_t FastTiles(int rows, int N, int tile) { return rows > 0 ? (uint32_t)(rows / tile) * (uint32_t)(N / tile) : 0u; }
+    static uint32_t AnyTiles(int rows, int N)
+    {
+        return rows > 0 ? (uint32_t)((rows + kAnyTile - 1) / kAnyTile) * (uint32_t)((N + kAnyTile - 1) / kAnyTile) : 0u;
+    }
 
 protected:
     virtual hipError_t LaunchKernel(hipStream_t stream, bool guarded, const XGuardArgs &g) override
     {
-        const dim3 grid(n_wg_);
-        const hipEvent_t stop = TakeStopEvent();
-        if (tile_ == kAnyTile) {
-            const dim3 block(256);
-            const uint32_t tiles_n = (uint32_t)((N_ + kAnyTile - 1) / kAnyTile);
-            if (guarded) LaunchWithStop(stop, GemmBf16AnyShapeKernel<true>, grid, block, stream, A_, B_, C_, M_, N_, K_, tiles_n, g);
-            else         LaunchWithStop(stop, GemmBf16AnyShapeKernel<false>, grid, block, stream, A_, B_, C_, M_, N_, K_, tiles_n, g);
-        } else if (tile_ == kLargeTile) {
-            const dim3 block(512);
-            if (guarded) LaunchWithStop(stop, (GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
-            else         LaunchWithStop(stop, (GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
-        } else {
-            const dim3 block(256);
-            if (guarded) LaunchWithStop(stop, (GemmBf16Kernel<true, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
-            else         LaunchWithStop(stop, (GemmBf16Kernel<false, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, M_, N_, K_, g);
+        const uint32_t fast_tiles = FastTiles(rows_fast_, N_, fast_tile_), any_tiles = AnyTiles(M_ - rows_fast_, N_);
+        const hipEvent_t stop = TakeStopEvent();   // for the command's last kernel
+        if (fast_tiles != 0) {
+            const hipEvent_t mine = any_tiles == 0 ? stop : nullptr;
+            const dim3 grid(fast_tiles);
+            if (fast_tile_ == kLargeTile) {
+                const dim3 block(512);
+                if (guarded) LaunchWithStop(mine, (GemmBf16Kernel<true, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, rows_fast_, N_, K_, g);
+                else         LaunchWithStop(mine, (GemmBf16Kernel<false, kLargeTile, 2, 4>), grid, block, stream, A_, B_, C_, rows_fast_, N_, K_, g);
+            } else {
+                const dim3 block(256);
+                if (guarded) LaunchWithStop(mine, (GemmBf16Kernel<true, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, rows_fast_, N_, K_, g);
+                else         LaunchWithStop(mine, (GemmBf16Kernel<false, kSmallTile, 2, 2>), grid, block, stream, A_, B_, C_, rows_fast_, N_, K_, g);
+            }
+            const hipError_t err = hipGetLastError();
+            if (err != hipSuccess || any_tiles == 0) return err;
         }
+        const dim3 grid(any_tiles), block(256);
+        const uint32_t tiles_n = (uint32_t)((N_ + kAnyTile - 1) / kAnyTile);
+        const uint16_t *a = A_ + (size_t)rows_fast_ * (size_t)K_;
+        uint16_t *c = C_ + (size_t)rows_fast_ * (size_t)N_;
+        const int rows = M_ - rows_fast_;
+        if (guarded) LaunchWithStop(stop, GemmBf16AnyShapeKernel<true>, grid, block, stream, a, B_, c, rows, N_, K_, tiles_n, fast_tiles, g);
+        else         LaunchWithStop(stop, GemmBf16AnyShapeKernel<false>, grid, block, stream, a, B_, c, rows, N_, K_, tiles_n, fast_tiles, g);
         return hipGetLastError();
     }
 
@@ -521,7 +540,7 @@ private:
     const uint16_t *A_, *B_;
     uint16_t *C_;
     const int M_, N_, K_;
-    const int tile_;
+    const int rows_fast_, fast_tile_;
 };
 
 /// The tile edge for an M x N output: large tiles do more arithmetic per byte read from LDS,
@@ -529,6 +548,8 @@ private:
 /// of the device idle. Small tiles when the large ones would cover at most half of the compute
 /// units, or when M or N is no multiple of the large edge. XSCHED_HIP_GEMM_TILE=128|256
 /// overrides the choice where the shape allows.
+inline int TileFor(int M, int N);
+
 /// Whether the fast kernels take the shape and the pointers.
 inline bool FastKernelsTake(const void *A, const void *B, const void *C, int M, int N, int K)
 {
@@ -568,16 +589,22 @@ EXPORT_C_FUNC XResult HipGemmBf16CommandCreate(HwCommandHandle *cmd, const void 
         return kXSchedErrorInvalidValue;
     }
     // The fast kernels take M and N in multiples of 128, K in multiples of 64 (K and N at most
-    // 2^22) and matrices aligned to 16 bytes; every other shape goes to the any-shape kernel.
+    // 2^22) and matrices aligned to 16 bytes. Where only M stands in the way, they take the
+    // rows up to the last multiple of 128 and the any-shape kernel the rest (the rows of a
+    // row-major matrix can be cut anywhere); every other shape goes to the any-shape kernel whole.
     int64_t forced = 0;
-    const bool any_shape = !gemm::FastKernelsTake(A, B, C, M, N, K) ||
-                           (GetEnvInt64("XSCHED_HIP_GEMM_TILE", forced) && forced == gemm::kAnyTile);
-    const int tile = any_shape ? gemm::kAnyTile : gemm::TileFor(M, N);
+    const bool force_any = GetEnvInt64("XSCHED_HIP_GEMM_TILE", forced) && forced == gemm::kAnyTile;
+    const int whole_rows = M / gemm::kSmallTile * gemm::kSmallTile;
+    int rows_fast = 0;
+    if (!force_any && whole_rows > 0 && gemm::FastKernelsTake(A, B, C, whole_rows, N, K)) rows_fast = whole_rows;
+    const int fast_tile = rows_fast > 0 ? gemm::TileFor(rows_fast, N) : gemm::kSmallTile;
     // one progress-map byte per tile
-    if ((uint64_t)((M + tile - 1) / tile) * (uint64_t)((N + tile - 1) / tile) > GuardState::kMaxWorkGroups) {
-        XWARN("HipGemmBf16CommandCreate: %d x %d has more than 2^18 tiles of %d x %d", M, N, tile, tile);
+    const uint64_t tiles = (uint64_t)gemm::HipGemmCommand::FastTiles(rows_fast, N, fast_tile) +
+                           (uint64_t)((M - rows_fast + gemm::kAnyTile - 1) / gemm::kAnyTile) * (uint64_t)((N + gemm::kAnyTile - 1) / gemm::kAnyTile);
+    if (tiles > GuardState::kMaxWorkGroups) {
+        XWARN("HipGemmBf16CommandCreate: %d x %d needs more than 2^18 tiles", M, N);
         return kXSchedErrorInvalidValue;
     }
-    *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, tile, guard));
+    *cmd = HwCommandManager::Add(std::make_shared<gemm::HipGemmCommand>(A, B, C, M, N, K, rows_fast, fast_tile, guard));
     return kXSchedSuccess;
 }
