@@ -299,6 +299,10 @@ def test_null_stream_and_bad_arguments(xs, gpu):
     assert h.HipHistogramCommandCreate(byref(cmd), 16, 4, 16, 70000, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, None, None, 4, 0) == xs.kXSchedErrorInvalidValue
     assert h.HipAxpyCommandCreate(byref(cmd), 1.0, 16, 16, 4, 4) == xs.kXSchedErrorInvalidValue
+    out = (c_uint64 * 8)()
+    assert h.HipQueueGetStats(0x1234, out) == xs.kXSchedErrorNotFound
+    assert h.HipQueueGetPoolStats(0x1234, out) == xs.kXSchedErrorNotFound
+    assert h.HipQueueSetMarkerOnKernel(0x1234, 1) == xs.kXSchedErrorNotFound
 
 
 def test_cross_queue_wait_on_recorded_event_follows_replays(xs, gpu):
