@@ -497,7 +497,7 @@ def config4(H, a):
             out = {"bg%d" % q: check_hist_bins(b, 0, q, q + 1, bg_n) for q in range(4)}
             out["fg"] = check_hist_bins(b, 1, 0, 0, fg_n)
             return out
-        runs[lax] = contended_run(H, cfg, a.steps, a.warmup, bg_warm=2, bg_cmds=6, keep=after if lax == 300 else None)
+        runs[lax] = contended_run(H, cfg, a.steps, a.warmup, bg_warm=16, bg_cmds=60, keep=after if lax == 300 else None)
     head = runs[300]
     fg = fg_summary(H, head["fg_alone"], head["fg_contended"])
     # Roofline of the kernel itself: one queue streaming it back to back, Level 2, guarded.
