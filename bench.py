@@ -527,6 +527,8 @@ def config4(H, a):
     line["bg"] = {"alone_GBs_4_queues_side_by_side":
                       hist_bytes(bg_n) * head["bg_alone_cmds"] / head["bg_alone_elapsed"] / 1e9,
                   "contended_GBs": hist_bytes(bg_n) * head["bg_cont_cmds"] / head["bg_cont_elapsed"] / 1e9}
+    line["bg"]["alone_frac_of_hbm_peak"] = line["bg"]["alone_GBs_4_queues_side_by_side"] / HBM_PEAK_GBS
+    line["bg"]["contended_frac_of_hbm_peak"] = line["bg"]["contended_GBs"] / HBM_PEAK_GBS
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("histogram_2p26_hbm_traffic.md"), "kernel": "HistogramKernel + HistogramMergeKernel",
                         "algorithmic_bytes_per_launch": hist_bytes(bg_n), "avg_launch_ms": per_launch_ms,
