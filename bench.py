@@ -782,6 +782,9 @@ def compact_of(line):
     for k in ("deadline_miss_rate", "bit_exact", "vendor_library"):
         if k in line:
             keep[k] = line[k]
+    if isinstance(line.get("bg"), dict) and "contended_frac_of_hbm_peak" in line["bg"]:
+        keep["bg_all_queues_frac_of_hbm_peak"] = {"alone": line["bg"]["alone_frac_of_hbm_peak"],
+                                                  "contended": line["bg"]["contended_frac_of_hbm_peak"]}
     if isinstance(keep.get("bit_exact"), dict) and "all_ok" in keep["bit_exact"]:
         keep["bit_exact"] = keep["bit_exact"]["all_ok"]
     if "per_priority_latency_us" in line:
